@@ -1,0 +1,132 @@
+/*
+ * C-ABI of libskywalker_hip.so: the alias-method hot path of Skywalker on one MI355X.
+ *
+ * The reference has no FFI; its host boundary is the set of `float f(Obj&)` entry
+ * functions declared in include/sampler.cuh:510-529 plus the gpu_graph / Sampler /
+ * Walker objects they take.  Each entry point below names the reference interface
+ * it replaces.  The C++ facade in skywalker_amd/host keeps the reference's class
+ * and function names on top of this ABI.
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative sky_status; the message of
+ *     the last failure on the calling thread is available from sky_last_error().
+ *   - a sky_graph owns the device-resident CSR and, after sky_alias_build_all, the
+ *     alias tables.  One host thread per sky_graph; calls are synchronous.
+ *   - "device pointer" arguments are HIP device addresses on the current device
+ *     (from sky_device_malloc, or any other allocator of the same process).
+ *   - `seconds` outputs report the kernel region only (launch to completion,
+ *     measured with HIP events on the stream the kernels run on), like the
+ *     gettimeofday bracket of the reference (src/util.cu:35-44).
+ *   - unreached output slots are never written; callers that want a sentinel
+ *     pre-fill with sky_device_fill_u32.
+ */
+#ifndef SKYWALKER_HIP_H_
+#define SKYWALKER_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct sky_graph sky_graph;
+
+enum sky_status {
+  SKY_OK = 0,
+  SKY_ERR_ARG = -1,     /* null pointer, zero size, inconsistent CSR */
+  SKY_ERR_HIP = -2,     /* a HIP runtime call failed */
+  SKY_ERR_STATE = -3,   /* e.g. walk on tables that were never built */
+  SKY_ERR_NO_GPU = -4,  /* no usable device */
+  SKY_ERR_LIMIT = -5    /* size beyond what the entry point supports */
+};
+
+enum sky_bias { SKY_BIAS_STATIC = 0, SKY_BIAS_NODE2VEC = 1 };
+enum sky_weight_kind { SKY_W_UNIFORM = 0, SKY_W_UNIT = 1, SKY_W_LOGNORMAL = 2 };
+
+#define SKY_INVALID 0xFFFFFFFFu /* alias value of rows whose total weight is zero */
+
+const char* sky_last_error(void);
+const char* sky_version(void);
+
+/* ---- device memory helpers (replace the cudaMalloc/cudaMemcpy calls scattered through
+ *      include/sampler_result.cuh:490-566 and include/gpu_graph.cuh:68-117) ---- */
+int sky_device_malloc(size_t bytes, void** out);
+int sky_device_free(void* p);
+int sky_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
+int sky_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
+int sky_device_fill_u32(void* dst_device, uint32_t value, size_t count);
+int sky_device_synchronize(void);
+int sky_device_name(char* buf, size_t buflen, int* compute_units);
+
+/* ---- graph residency: replaces gpu_graph::gpu_graph(Graph*, uint) (include/gpu_graph.cuh:68-117).
+ *      xadj[V+1], adjncy[E], adjwgt[E] are host arrays; rows must be sorted by neighbour id for
+ *      node2vec (gpu_graph.cuh:204-238 assumes the same). adjwgt may be NULL (all weights 1). ---- */
+int sky_graph_upload(const uint32_t* xadj, const uint32_t* adjncy, const float* adjwgt, uint32_t V, uint32_t E,
+                     sky_graph** out);
+/* Synthetic R-MAT graph (a,b,c,d = .57,.19,.19,.05) generated and sorted on the device; no counterpart in the
+ * reference, which reads Galois .gr files (include/graph.cuh:164-327).  weight_kind: sky_weight_kind with
+ * parameters (wa, wb) = (lo, hi) for UNIFORM, ignored for UNIT, (mu, sigma) for LOGNORMAL. */
+int sky_graph_generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int weight_kind, float wa,
+                            float wb, uint64_t weight_seed, sky_graph** out);
+int sky_graph_info(const sky_graph* g, uint32_t* V, uint32_t* E, uint32_t* max_degree);
+/* Copies to host; any destination may be NULL. */
+int sky_graph_download(const sky_graph* g, uint32_t* xadj, uint32_t* adjncy, float* adjwgt);
+/* Device addresses of the resident arrays (xadj, adjncy, adjwgt, prob, alias, valid); any output may be NULL. */
+int sky_graph_device_ptrs(const sky_graph* g, const uint32_t** xadj, const uint32_t** adjncy, const float** adjwgt,
+                          const float** prob, const uint32_t** alias, const int8_t** valid);
+/* Replaces gpu_graph::Free + Sampler::Free (gpu_graph.cuh:164-177, sampler.cuh:65-81). */
+int sky_graph_free(sky_graph* g);
+
+/* ---- offline alias tables for every vertex: replaces ConstructTable(Sampler&, ngpu=1, index=0)
+ *      (src/createTable.cu:119-179, kernel :48-108).  Allocates prob[E] f32, alias[E] u32 (row-local
+ *      index, same slot as the CSR edge) and valid[V] i8 inside the graph.  Unlike the reference the
+ *      edge weights are kept (createTable.cu:175-177 frees them). ---- */
+int sky_alias_build_all(sky_graph* g, double* seconds);
+int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid);
+/* Installs caller-built tables (host arrays) instead of building: for tests and table persistence. */
+int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, const int8_t* valid);
+
+/* ---- start vertices uniform over [0,V): Philox(seed; i). seeds_device[N]. The reference uses 0..N-1
+ *      (include/sampler.cuh:494-503); sequential seeds are simply uploaded by the caller. ---- */
+int sky_gen_seeds(uint64_t seed, uint32_t V, uint32_t N, uint32_t* seeds_device);
+
+/* ---- biased walk on prebuilt tables: replaces OfflineWalk(Walker&) (src/offline_walk.cu:181-230, kernels
+ *      :10-175); stop_prob > 0 adds the PPR stop test the reference only has online (online_walk.cu:109-110).
+ *      paths_device[N*(len+1)] walker-major, lengths_device[N]; *sampled = sum of lengths. ---- */
+int sky_walk_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uint32_t len, float stop_prob,
+                     uint64_t philox_seed, uint32_t* paths_device, uint32_t* lengths_device, uint64_t* sampled,
+                     double* seconds);
+
+/* ---- walk that rebuilds the table of the current vertex at every step: replaces OnlineWalkShMem(Walker&) /
+ *      OnlineWalkGMem(Walker&) (src/online_walk.cu:245-327, online_walk_gmem.cu); bias SKY_BIAS_NODE2VEC applies
+ *      the second-order factors of src/api/bias_node2vec.cu:15-27 with (p, q). ---- */
+int sky_walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds_device, uint32_t N,
+                    uint32_t len, float stop_prob, uint64_t philox_seed, uint32_t* paths_device,
+                    uint32_t* lengths_device, uint64_t* sampled, double* seconds);
+
+/* ---- k-hop neighbour sampling: replaces OfflineSample(Sampler_new&) (src/offline_sample.cu:443-513) and
+ *      OnlineGBSampleNew(Sampler_new&) (src/online_sample_new.cu:459-547).  fanout[hops] with fanout[0] == 1
+ *      (host array, e.g. {1,25,10}); data_device[N*length_per_sample], sample_lengths_device[N*size_of_lengths]
+ *      in the layout of include/sampler_result.cuh:226-260 (see sky_sample_layout). ---- */
+int sky_sample_layout(const uint32_t* fanout, uint32_t hops, uint64_t* length_per_sample,
+                      uint64_t* size_of_sample_lengths);
+int sky_sample_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                       uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device,
+                       uint64_t* sampled, double* seconds);
+int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                      uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device, uint64_t* sampled,
+                      double* seconds);
+
+/* ---- self-test hook: runs Philox4x32-10 on the device for n (counter, key) pairs.
+ *      ctr_host[4n], key_host[2n] -> out_host[4n]. ---- */
+int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint32_t n, uint32_t* out_host);
+
+/* ---- per-kernel timing of the last sky_alias_build_all on this graph, for roofline reporting:
+ *      names[i] is a static string, ms[i] its HIP-event duration.  Returns the number of entries. ---- */
+int sky_last_build_profile(const sky_graph* g, const char** names, float* ms, uint64_t* edges, int max_entries);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SKYWALKER_HIP_H_ */

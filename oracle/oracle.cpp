@@ -34,12 +34,13 @@
 //   S    = sum_i floor(w'_i * 2^64)          exact, 128-bit unsigned integer
 //   Sd   = ((double)l3*2^32 + (double)l2) + ((double)l1*2^-32 + (double)l0*2^-64)   (l0..l3 = 32-bit limbs of S)
 //   scale= (double)deg / Sd ;  p_i = (double)w'_i * scale
-//   t_i  = (p_i - 1.0) * 2^32
+//   F    = 40 if deg < 2^22, else 62 - floor(log2(deg))    (fraction bits of the integer ledger)
+//   t_i  = (p_i - 1.0) * 2^F
 //   heavy iff t_i >= 0.5, with surplus U_i = floor(t_i + 0.5) >= 1                 (64-bit unsigned)
-//   light otherwise, with deficit D_i = min(floor(-t_i + 0.5), 2^32-1)
+//   light otherwise, with deficit D_i = floor(-t_i + 0.5)
 //   lights and heavies are taken in CSR slot order.  A sweep lets heavy j fill
-//   lights while its residual r (units of 2^-32) exceeds 2^32; when r <= 2^32 the
-//   heavy becomes a bucket {prob = r*2^-32, alias = next heavy} and the next
+//   lights while its residual r (units of 2^-F) exceeds 2^F; when r <= 2^F the
+//   heavy becomes a bucket {prob = r*2^-F, alias = next heavy} and the next
 //   heavy inherits r + U.  The last heavy always ends {prob 1, alias self};
 //   lights left without a donor take the last heavy; a row without heavies is
 //   {prob (float)p, alias self}.  A light stores prob = (float)p_i.
@@ -206,6 +207,13 @@ static inline double fixed_to_double(u128 S) {
   return hi + lo;
 }
 
+static inline int frac_bits(uint32_t deg) {
+  if (deg < (1u << 22)) return 40;
+  int lg = 0;
+  while ((deg >> (lg + 1)) != 0) ++lg;
+  return 62 - lg;
+}
+
 // One row by the two-pointer sweep.  getw(i) yields the raw weight of slot i.
 // Returns 1 if the row is valid.
 template <class GetW>
@@ -221,14 +229,16 @@ static int alias_row_sweep(uint32_t deg, GetW getw, float* prob, uint32_t* alias
   const double scale = (double)deg / fixed_to_double(S);
   p.resize(deg);
   heavy.clear();
-  auto excess = [&](uint32_t i) -> double { return (p[i] - 1.0) * 4294967296.0; };
+  const int F = frac_bits(deg);
+  const double FS = std::ldexp(1.0, F), INV_FS = std::ldexp(1.0, -F);
+  auto excess = [&](uint32_t i) -> double { return (p[i] - 1.0) * FS; };
   for (uint32_t i = 0; i < deg; ++i) {
     p[i] = (double)clamp_weight(getw(i)) * scale;
     if (excess(i) >= 0.5) heavy.push_back(i);
   }
   const size_t nH = heavy.size();
   auto surplus = [&](uint32_t j) -> uint64_t { return (uint64_t)std::floor(excess(heavy[j]) + 0.5); };
-  const uint64_t ONE = 1ull << 32;
+  const uint64_t ONE = 1ull << F;
   if (nH == 0) {
     for (uint32_t i = 0; i < deg; ++i) { prob[i] = (float)p[i]; alias[i] = i; }
     return 1;
@@ -239,13 +249,12 @@ static int alias_row_sweep(uint32_t deg, GetW getw, float* prob, uint32_t* alias
     if (excess(i) >= 0.5) continue;
     // retire heavies that can no longer donate
     while (r <= ONE && j + 1 < nH) {
-      prob[heavy[j]] = (float)((double)r * (1.0 / 4294967296.0));
+      prob[heavy[j]] = (float)((double)r * INV_FS);
       alias[heavy[j]] = heavy[j + 1];
       r += surplus(j + 1);
       ++j;
     }
-    double x = -excess(i) + 0.5;
-    uint64_t D = x >= 4294967295.0 ? 4294967295ull : (uint64_t)std::floor(x);
+    const uint64_t D = (uint64_t)std::floor(-excess(i) + 0.5);
     prob[i] = (float)p[i];
     alias[i] = heavy[j];  // the last heavy also absorbs lights left without a donor
     // a heavy that is not the last has r > 2^32 > D here; the last heavy's r is never read again
@@ -253,7 +262,7 @@ static int alias_row_sweep(uint32_t deg, GetW getw, float* prob, uint32_t* alias
   }
   // lights are done: retire the chain of heavies whose residual is spent
   while (r <= ONE && j + 1 < nH) {
-    prob[heavy[j]] = (float)((double)r * (1.0 / 4294967296.0));
+    prob[heavy[j]] = (float)((double)r * INV_FS);
     alias[heavy[j]] = heavy[j + 1];
     r += surplus(j + 1);
     ++j;

@@ -1,0 +1,53 @@
+"""Compiles libskywalker_hip.so (hand-written HIP for gfx950) in-tree with hipcc."""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libskywalker_hip.so")
+SOURCES = ["sky_capi.hip", "sky_build.hip", "sky_walk.hip", "sky_online.hip", "sky_sample.hip", "sky_gen.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
+    # packed fp32 instructions are kept out of every kernel of this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _compile(src):
+    obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    warn = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip())
+    return obj, warn
+
+
+def build_library(verbose=False, jobs=6):
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(_compile, SOURCES))
+    objs = [o for o, _ in results]
+    if verbose:
+        for _, w in results:
+            if w:
+                print(w, file=sys.stderr)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))
+
+
+def build_host():
+    """Builds the C++ facade and the `skywalker` CLI on top of the C-ABI (skywalker_amd/host)."""
+    host = os.path.join(HERE, "host")
+    if os.path.exists(os.path.join(host, "Makefile")):
+        subprocess.check_call(["make", "-C", host, "-B", "-j4"], stdout=subprocess.DEVNULL)

@@ -1,0 +1,686 @@
+// Offline alias-table construction for every vertex (replaces ConstructAliasTableKernel /
+// ConstructTable of the reference, src/createTable.cu:48-179, and the constructors of
+// include/alias_table_new.cuh it calls).
+//
+// The table of a row is a pure function of its weights, defined with exact integer
+// prefix sums so that no kernel below can change a bit of it by changing how it
+// parallelises:
+//   S     = sum floor(w_i 2^64)  (128 bit)        scale = deg / double(S)      p_i = w_i * scale
+//   F     = 40 fraction bits (62 - floor(log2 deg) for rows of 2^22 entries and more)
+//   t_i   = (p_i - 1) 2^F  ;  heavy iff t_i >= 0.5 : surplus U_i = floor(t_i + .5)
+//                             light otherwise      : deficit D_i = floor(-t_i + .5)
+//   SL(i) = inclusive prefix sum of deficits over slots <= i,  SH(i) likewise of surpluses
+//   light i : prob = float(p_i), alias = first slot m with SH(m) > SL(i) - D_i
+//             (the last heavy if there is none; itself if the row has no heavy)
+//   heavy j : last heavy of the row -> prob 1, alias itself; otherwise with y = SH(j):
+//             l = first slot with SL(l) >= y;  found -> prob = (2^F + y - SL(l)) 2^-F, alias = next heavy
+//                                              none  -> prob 1, alias itself
+// This is the pairing a sequential two-pointer Vose sweep over (lights in slot order,
+// heavies in slot order) produces, written so that every entry is resolved by two
+// prefix sums and a binary search: no queues, no float atomics, no rollback.
+//
+// Dispatch is by degree class (sky_graph.h): one lane per vertex while binning (deg <= 2),
+// 4/8/16/32/64 lanes per vertex with the prefix arrays in a per-wave LDS strip,
+// one wavefront / 256 / 1024 threads per vertex with the row's prefix arrays in LDS,
+// and 1024 threads streaming through a global scratch for rows beyond 128 KB of LDS.
+#include <algorithm>
+
+#include "sky_graph.h"
+
+namespace sky {
+
+__host__ __device__ __forceinline__ int degree_class(uint32_t d) {
+  if (d == 0) return CLS_EMPTY;
+  if (d <= 2) return CLS_TINY;
+  if (d <= 4) return CLS_SUB4;
+  if (d <= 8) return CLS_SUB8;
+  if (d <= 16) return CLS_SUB16;
+  if (d <= 32) return CLS_SUB32;
+  if (d <= 64) return CLS_WAVE;
+  if (d <= 253) return CLS_LDS_W1;
+  if (d <= 1021) return CLS_LDS_W4;
+  if (d <= 4093) return CLS_LDS_B4;
+  if (d <= 8189) return CLS_LDS_X2;
+  return CLS_HUGE;
+}
+
+// first m in [lo, n) with a[m] > key, else n
+__device__ __forceinline__ uint32_t first_greater(const uint64_t* a, uint32_t lo, uint32_t n, uint64_t key) {
+  uint32_t len = n - lo;
+  while (len > 0) {
+    const uint32_t half = len >> 1;
+    if (a[lo + half] <= key) {
+      lo += half + 1;
+      len -= half + 1;
+    } else {
+      len = half;
+    }
+  }
+  return lo;
+}
+
+// ---------------------------------------------------------------- binning
+// `src` lists the vertices to bin (n of them); a null src means vertices 0..n-1.
+__global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restrict__ xadj,
+                                                        const uint32_t* __restrict__ src, uint32_t n,
+                                                        uint32_t* __restrict__ counts) {
+  __shared__ uint32_t s_cnt[CLS_COUNT];
+  if (threadIdx.x < CLS_COUNT) s_cnt[threadIdx.x] = 0;
+  __syncthreads();
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += gridDim.x * 256u) {
+    const uint32_t v = src ? src[i] : i;
+    const int c = degree_class(xadj[v + 1] - xadj[v]);
+    if (c >= CLS_SUB4) atomicAdd(&s_cnt[c], 1u);
+  }
+  __syncthreads();
+  if (threadIdx.x < CLS_COUNT && s_cnt[threadIdx.x]) atomicAdd(&counts[threadIdx.x], s_cnt[threadIdx.x]);
+}
+
+constexpr int BIN_ITEMS = 4;  // vertices per thread in the scatter pass
+
+// Writes each vertex of class >= CLS_SUB4 into its class segment of vlist, and finishes
+// the classes that need no cooperation: deg 0 (valid = 0) and deg 1..2 (closed form).
+__global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __restrict__ xadj,
+                                                          const float* __restrict__ wgt,
+                                                          const uint32_t* __restrict__ src, uint32_t n,
+                                                          uint32_t* __restrict__ cursors,
+                                                          uint32_t* __restrict__ vlist, float* __restrict__ prob,
+                                                          uint32_t* __restrict__ alias, int8_t* __restrict__ valid) {
+  __shared__ uint32_t s_cnt[CLS_COUNT], s_base[CLS_COUNT];
+  if (threadIdx.x < CLS_COUNT) s_cnt[threadIdx.x] = 0;
+  __syncthreads();
+  const uint32_t chunk = blockIdx.x * (256u * BIN_ITEMS);
+  int cls[BIN_ITEMS];
+  uint32_t rank[BIN_ITEMS], vtx[BIN_ITEMS];
+#pragma unroll
+  for (int i = 0; i < BIN_ITEMS; ++i) {
+    const uint32_t item = chunk + i * 256u + threadIdx.x;
+    cls[i] = -1;
+    if (item >= n) continue;
+    const uint32_t v = src ? src[item] : item;
+    vtx[i] = v;
+    const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+    const int c = degree_class(d);
+    cls[i] = c;
+    if (c == CLS_EMPTY) {
+      valid[v] = 0;
+    } else if (c == CLS_TINY) {
+      const float w0 = clamp_weight(wgt[off]);
+      if (d == 1) {
+        const u128 q = weight_fixed(w0);
+        const bool ok = (q.lo | q.hi) != 0;
+        prob[off] = ok ? 1.0f : 0.0f;
+        alias[off] = ok ? 0u : SKY_INVALID;
+        valid[v] = ok;
+      } else {
+        const float w1 = clamp_weight(wgt[off + 1]);
+        const u128 s = add128(weight_fixed(w0), weight_fixed(w1));
+        if ((s.lo | s.hi) == 0) {
+          prob[off] = prob[off + 1] = 0.0f;
+          alias[off] = alias[off + 1] = SKY_INVALID;
+          valid[v] = 0;
+        } else {
+          const Ledger L = make_ledger(2, s);
+          const Entry e0 = classify(w0, L), e1 = classify(w1, L);
+          // a lone heavy is the last heavy: it keeps its bucket and tops up the light
+          prob[off] = e0.heavy ? 1.0f : (float)e0.p;
+          prob[off + 1] = e1.heavy ? 1.0f : (float)e1.p;
+          alias[off] = (!e0.heavy && e1.heavy) ? 1u : 0u;
+          alias[off + 1] = (!e1.heavy && e0.heavy) ? 0u : 1u;
+          valid[v] = 1;
+        }
+      }
+    } else {
+      rank[i] = atomicAdd(&s_cnt[c], 1u);
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < CLS_COUNT && s_cnt[threadIdx.x])
+    s_base[threadIdx.x] = atomicAdd(&cursors[threadIdx.x], s_cnt[threadIdx.x]);
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < BIN_ITEMS; ++i) {
+    if (cls[i] >= CLS_SUB4) vlist[s_base[cls[i]] + rank[i]] = vtx[i];
+  }
+}
+
+// ---------------------------------------------------------------- 4..64 lanes per vertex
+// One table entry per lane.  Prefix sums run over the group with shuffles; the two
+// searches read the group's strip of a per-wave LDS array.
+template <int G>
+__global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+                                                            const uint32_t* __restrict__ xadj,
+                                                            const float* __restrict__ wgt, float* __restrict__ prob,
+                                                            uint32_t* __restrict__ alias,
+                                                            int8_t* __restrict__ valid) {
+  __shared__ uint64_t s_sl[256], s_sh[256];
+  const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t grp = tid / G;
+  const int gl = threadIdx.x & (G - 1);
+  const int lane = lane_id();
+  const int gb_lane = lane - gl;           // first lane of the group inside the wave
+  const int gb = threadIdx.x - gl;         // first LDS slot of the group
+  uint32_t v = 0, off = 0, d = 0;
+  if (grp < count) {
+    v = vlist[grp];
+    off = xadj[v];
+    d = xadj[v + 1] - off;
+  }
+  const bool act = (uint32_t)gl < d;
+  const float w = act ? clamp_weight(wgt[off + gl]) : 0.0f;
+  const u128 S = group_sum_u128<G>(weight_fixed(w));
+  const bool row_ok = (S.lo | S.hi) != 0;
+  Ledger L = make_ledger(d, S);
+  if (!row_ok) L.scale = 0.0;
+  Entry e = classify(w, L);
+  if (!act) { e.heavy = false; e.amount = 0; }
+  const uint64_t SL = group_scan_u64<G>(e.heavy ? 0 : e.amount);
+  const uint64_t SH = group_scan_u64<G>(e.heavy ? e.amount : 0);
+  s_sl[threadIdx.x] = SL;
+  s_sh[threadIdx.x] = SH;
+  const uint64_t hm = __ballot(e.heavy);
+  const uint64_t gm = G == 64 ? ~0ull : (((1ull << (G & 63)) - 1) << gb_lane);
+  const uint64_t hmg = hm & gm;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  // light: first slot with SH > SL - D.  heavy: first slot with SL >= SH, i.e. SL > SH - 1.
+  const uint64_t* arr = (e.heavy ? s_sl : s_sh) + gb;
+  const uint64_t key = e.heavy ? SH - 1 : SL - e.amount;
+  int pos = 0;
+#pragma unroll
+  for (int step = G / 2; step >= 1; step >>= 1)
+    if (arr[pos + step - 1] <= key) pos += step;
+  const uint64_t at = arr[pos];
+  const bool found = at > key;
+  float out_p;
+  uint32_t out_a;
+  if (!e.heavy) {
+    out_p = (float)e.p;
+    out_a = found ? (uint32_t)pos : (hmg ? (uint32_t)(63 - __clzll(hmg) - gb_lane) : (uint32_t)gl);
+  } else {
+    const uint64_t above = hmg & ~((2ull << lane) - 1);
+    if (above == 0 || !found) {
+      out_p = 1.0f;
+      out_a = gl;
+    } else {
+      out_p = residual_prob(L.one + SH - at, L);
+      out_a = (uint32_t)(__ffsll((unsigned long long)above) - 1 - gb_lane);
+    }
+  }
+  if (!row_ok) { out_p = 0.0f; out_a = SKY_INVALID; }
+  if (act) {
+    prob[off + gl] = out_p;
+    alias[off + gl] = out_a;
+  }
+  if (gl == 0 && grp < count) valid[v] = row_ok;
+}
+
+// ---------------------------------------------------------------- one row per workgroup, prefix arrays in LDS
+// ROWT threads cooperate on one row of at most ROWT*4*T slots (counted from the row's
+// 16-byte aligned start).  Weights are read once as aligned float4 quads and stay in
+// registers; SL and SH of every slot live in LDS for the searches.
+template <int ROWT, int T>
+__global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restrict__ vlist,
+                                                         const uint32_t* __restrict__ xadj,
+                                                         const float* __restrict__ wgt, float* __restrict__ prob,
+                                                         uint32_t* __restrict__ alias, int8_t* __restrict__ valid) {
+  constexpr int CAP = ROWT * 4 * T;
+  constexpr int NW = ROWT / 64;
+  extern __shared__ uint64_t smem[];
+  uint64_t* s_sl = smem;
+  uint64_t* s_sh = smem + CAP;
+  __shared__ u128 s_wsum[NW];
+  __shared__ uint64_t s_wl[NW], s_wh[NW];
+
+  const uint32_t v = vlist[blockIdx.x];
+  const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+  const uint32_t base = off & ~3u, lead = off - base, span = lead + d;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+
+  float w[T][4];
+  u128 sum{0, 0};
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const uint32_t pos = 4u * (t * ROWT + tid);
+    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pos < span) x = *reinterpret_cast<const float4*>(wgt + base + pos);
+    const float xs[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = pos + k;
+      w[t][k] = (idx >= lead && idx < span) ? clamp_weight(xs[k]) : 0.0f;
+      sum = add128(sum, weight_fixed(w[t][k]));
+    }
+  }
+  sum = group_sum_u128<64>(sum);
+  if (NW > 1) {
+    if (lane == 0) s_wsum[wave] = sum;
+    __syncthreads();
+    sum = s_wsum[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) sum = add128(sum, s_wsum[i]);
+  }
+  if ((sum.lo | sum.hi) == 0) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const uint32_t pos = 4u * (t * ROWT + tid);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t idx = pos + k;
+        if (idx >= lead && idx < span) {
+          prob[base + idx] = 0.0f;
+          alias[base + idx] = SKY_INVALID;
+        }
+      }
+    }
+    if (tid == 0) valid[v] = 0;
+    return;
+  }
+  const Ledger L = make_ledger(d, sum);
+
+  uint64_t carry_l = 0, carry_h = 0;
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const uint32_t pos = 4u * (t * ROWT + tid);
+    uint64_t l[4], h[4], rl = 0, rh = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = pos + k;
+      const Entry e = classify(w[t][k], L);
+      const bool in = idx >= lead && idx < span;
+      rl += (in && !e.heavy) ? e.amount : 0;
+      rh += (in && e.heavy) ? e.amount : 0;
+      l[k] = rl;
+      h[k] = rh;
+    }
+    const uint64_t il = group_scan_u64<64>(rl), ih = group_scan_u64<64>(rh);
+    uint64_t base_l = carry_l + il - rl, base_h = carry_h + ih - rh;
+    if (NW > 1) {
+      if (t > 0) __syncthreads();  // previous tile's wave totals have been consumed
+      if (lane == 63) { s_wl[wave] = il; s_wh[wave] = ih; }
+      __syncthreads();
+      uint64_t tl = 0, th = 0;
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        if (i == wave) { base_l += tl; base_h += th; }
+        tl += s_wl[i];
+        th += s_wh[i];
+      }
+      carry_l += tl;
+      carry_h += th;
+    } else {
+      carry_l += shfl_u64(il, 63);
+      carry_h += shfl_u64(ih, 63);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      s_sl[pos + k] = base_l + l[k];
+      s_sh[pos + k] = base_h + h[k];
+    }
+  }
+  __syncthreads();
+  const uint64_t total_h = carry_h;
+
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const uint32_t pos = 4u * (t * ROWT + tid);
+    if (pos >= span) continue;
+    float op[4];
+    uint32_t oa[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = pos + k;
+      op[k] = 0.0f;
+      oa[k] = 0;
+      if (idx < lead || idx >= span) continue;
+      const Entry e = classify(w[t][k], L);
+      const uint32_t self = idx - lead;
+      if (!e.heavy) {
+        const uint64_t x = s_sl[idx] - e.amount;
+        const uint32_t m = first_greater(s_sh, lead, span, x);
+        op[k] = (float)e.p;
+        if (m < span) {
+          oa[k] = m - lead;
+        } else if (total_h) {
+          oa[k] = first_greater(s_sh, lead, span, total_h - 1) - lead;  // the last heavy
+        } else {
+          oa[k] = self;
+        }
+      } else {
+        const uint64_t y = s_sh[idx];
+        const uint32_t nxt = first_greater(s_sh, idx + 1, span, y);
+        const uint32_t li = nxt < span ? first_greater(s_sl, lead, span, y - 1) : span;
+        if (li < span) {
+          op[k] = residual_prob(L.one + y - s_sl[li], L);
+          oa[k] = nxt - lead;
+        } else {
+          op[k] = 1.0f;
+          oa[k] = self;
+        }
+      }
+    }
+    if (pos >= lead && pos + 4 <= span) {
+      *reinterpret_cast<float4*>(prob + base + pos) = make_float4(op[0], op[1], op[2], op[3]);
+      *reinterpret_cast<uint4*>(alias + base + pos) = make_uint4(oa[0], oa[1], oa[2], oa[3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t idx = pos + k;
+        if (idx >= lead && idx < span) {
+          prob[base + idx] = op[k];
+          alias[base + idx] = oa[k];
+        }
+      }
+    }
+  }
+  if (tid == 0) valid[v] = 1;
+}
+
+// ---------------------------------------------------------------- rows beyond LDS: global scratch
+// 1024 threads stream one row three times: exact sum; prefix sums written to a scratch
+// region private to the row (16 bytes per slot); searches over that scratch.
+constexpr int HUGE_T = 1024;
+
+__device__ __forceinline__ u128 block_sum_u128(u128 v, u128* s_tmp) {
+  v = group_sum_u128<64>(v);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __syncthreads();
+  if (lane == 0) s_tmp[wave] = v;
+  __syncthreads();
+  u128 r = s_tmp[0];
+  for (int i = 1; i < HUGE_T / 64; ++i) r = add128(r, s_tmp[i]);
+  return r;
+}
+
+__global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+                                                            const uint64_t* __restrict__ scratch_off,
+                                                            const uint32_t* __restrict__ xadj,
+                                                            const float* __restrict__ wgt,
+                                                            uint64_t* __restrict__ scratch, float* __restrict__ prob,
+                                                            uint32_t* __restrict__ alias,
+                                                            int8_t* __restrict__ valid) {
+  constexpr int NW = HUGE_T / 64;
+  __shared__ u128 s_tmp[NW];
+  __shared__ uint64_t s_wl[NW], s_wh[NW];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  for (uint32_t r = blockIdx.x; r < count; r += gridDim.x) {
+    const uint32_t v = vlist[r];
+    const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+    const float* wr = wgt + off;
+    uint64_t* g_sl = scratch + 2 * scratch_off[r];
+    uint64_t* g_sh = g_sl + d;
+
+    u128 sum{0, 0};
+    for (uint32_t i = tid; i < d; i += HUGE_T) sum = add128(sum, weight_fixed(clamp_weight(wr[i])));
+    sum = block_sum_u128(sum, s_tmp);
+    if ((sum.lo | sum.hi) == 0) {
+      for (uint32_t i = tid; i < d; i += HUGE_T) {
+        prob[off + i] = 0.0f;
+        alias[off + i] = SKY_INVALID;
+      }
+      if (tid == 0) valid[v] = 0;
+      continue;
+    }
+    const Ledger L = make_ledger(d, sum);
+
+    uint64_t carry_l = 0, carry_h = 0;
+    for (uint32_t tile = 0; tile < d; tile += HUGE_T) {
+      const uint32_t i = tile + tid;
+      uint64_t dl = 0, dh = 0;
+      if (i < d) {
+        const Entry e = classify(clamp_weight(wr[i]), L);
+        if (e.heavy) dh = e.amount; else dl = e.amount;
+      }
+      const uint64_t il = group_scan_u64<64>(dl), ih = group_scan_u64<64>(dh);
+      __syncthreads();
+      if (lane == 63) { s_wl[wave] = il; s_wh[wave] = ih; }
+      __syncthreads();
+      uint64_t bl = carry_l, bh = carry_h, tl = 0, th = 0;
+      for (int k = 0; k < NW; ++k) {
+        if (k == wave) { bl += tl; bh += th; }
+        tl += s_wl[k];
+        th += s_wh[k];
+      }
+      if (i < d) {
+        g_sl[i] = bl + il;
+        g_sh[i] = bh + ih;
+      }
+      carry_l += tl;
+      carry_h += th;
+    }
+    const uint64_t total_h = carry_h;
+    __threadfence();
+    __syncthreads();
+
+    for (uint32_t i = tid; i < d; i += HUGE_T) {
+      const Entry e = classify(clamp_weight(wr[i]), L);
+      float op;
+      uint32_t oa;
+      if (!e.heavy) {
+        const uint64_t x = g_sl[i] - e.amount;
+        const uint32_t m = first_greater(g_sh, 0, d, x);
+        op = (float)e.p;
+        if (m < d) oa = m;
+        else if (total_h) oa = first_greater(g_sh, 0, d, total_h - 1);
+        else oa = i;
+      } else {
+        const uint64_t y = g_sh[i];
+        const uint32_t nxt = first_greater(g_sh, i + 1, d, y);
+        const uint32_t li = nxt < d ? first_greater(g_sl, 0, d, y - 1) : d;
+        if (li < d) {
+          op = residual_prob(L.one + y - g_sl[li], L);
+          oa = nxt;
+        } else {
+          op = 1.0f;
+          oa = i;
+        }
+      }
+      prob[off + i] = op;
+      alias[off + i] = oa;
+    }
+    if (tid == 0) valid[v] = 1;
+    __syncthreads();
+  }
+}
+
+// Exclusive prefix sum of the degrees of the huge rows (a few thousand at most per launch of
+// 1024 threads; longer lists are walked in chunks by the same block).
+__global__ __launch_bounds__(1024) void huge_prefix_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+                                                           const uint32_t* __restrict__ xadj,
+                                                           uint64_t* __restrict__ scratch_off,
+                                                           uint64_t* __restrict__ total) {
+  __shared__ uint64_t s_w[16];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  uint64_t carry = 0;
+  for (uint32_t chunk = 0; chunk < count; chunk += 1024) {
+    const uint32_t r = chunk + tid;
+    uint64_t d = 0;
+    if (r < count) {
+      const uint32_t v = vlist[r];
+      d = xadj[v + 1] - xadj[v];
+    }
+    const uint64_t inc = group_scan_u64<64>(d);
+    __syncthreads();
+    if (lane == 63) s_w[wave] = inc;
+    __syncthreads();
+    uint64_t b = carry, t = 0;
+    for (int k = 0; k < 16; ++k) {
+      if (k == wave) b += t;
+      t += s_w[k];
+    }
+    if (r < count) scratch_off[r] = b + inc - d;
+    carry += t;
+  }
+  if (tid == 0) *total = carry;
+}
+
+// ---------------------------------------------------------------- host driver
+namespace {
+
+struct BuildScratch {
+  uint32_t* vlist = nullptr;     // [vcap]
+  uint32_t* counters = nullptr;  // [2*CLS_COUNT] counts then cursors
+  uint64_t* huge_off = nullptr;  // [huge_cap + 1], last = total
+  uint64_t* huge_scratch = nullptr;
+  uint32_t vcap = 0, huge_cap = 0;
+  uint64_t huge_scratch_cap = 0;
+  bool lds_enabled = false;
+};
+BuildScratch g_scratch;  // reused across builds; one build at a time per process
+
+template <class K>
+int enable_big_lds(K kernel, size_t bytes) {
+  SKY_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)bytes));
+  return SKY_OK;
+}
+
+}  // namespace
+
+int EventTimer::mark(const char* name, uint64_t e) {
+  hipEvent_t x;
+  SKY_HIP(hipEventCreate(&x));
+  SKY_HIP(hipEventRecord(x, stream));
+  ev.push_back(x);
+  names.push_back(name);
+  edges.push_back(e);
+  return SKY_OK;
+}
+int EventTimer::finish(std::vector<sky_graph::ProfileEntry>* profile, double* seconds) {
+  SKY_HIP(hipStreamSynchronize(stream));
+  SKY_HIP(hipGetLastError());
+  if (profile) profile->clear();
+  for (size_t i = 1; i < ev.size(); ++i) {
+    float ms = 0;
+    SKY_HIP(hipEventElapsedTime(&ms, ev[i - 1], ev[i]));
+    if (profile) profile->push_back({names[i], ms, edges[i]});
+  }
+  float total_ms = 0;
+  if (ev.size() >= 2) SKY_HIP(hipEventElapsedTime(&total_ms, ev.front(), ev.back()));
+  if (seconds) *seconds = total_ms * 1e-3;
+  return SKY_OK;
+}
+EventTimer::~EventTimer() {
+  for (hipEvent_t e : ev) (void)hipEventDestroy(e);
+}
+
+int ensure_table_storage(sky_graph* g) {
+  if (!g->prob) SKY_TRY(alloc_padded(&g->prob, (size_t)g->E));
+  if (!g->alias) SKY_TRY(alloc_padded(&g->alias, (size_t)g->E));
+  if (!g->valid) SKY_TRY(alloc_padded(&g->valid, (size_t)g->V));
+  return SKY_OK;
+}
+
+int prepare_build_scratch(uint32_t max_rows) {
+  BuildScratch& sc = g_scratch;
+  if (sc.vcap < max_rows) {
+    if (sc.vlist) SKY_HIP(hipFree(sc.vlist));
+    sc.vlist = nullptr;
+    sc.vcap = 0;
+    SKY_HIP(hipMalloc((void**)&sc.vlist, (size_t)max_rows * 4 + 16));
+    sc.vcap = max_rows;
+  }
+  if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, 2 * CLS_COUNT * 4));
+  if (!sc.lds_enabled) {
+    SKY_TRY(enable_big_lds(build_lds_kernel<64, 4>, 64 * 4 * 4 * 16));
+    SKY_TRY(enable_big_lds(build_lds_kernel<256, 4>, 256 * 4 * 4 * 16));
+    SKY_TRY(enable_big_lds(build_lds_kernel<1024, 2>, 1024 * 4 * 2 * 16));
+    sc.lds_enabled = true;
+  }
+  return SKY_OK;
+}
+
+// Builds the rows listed in `src` (device array of n vertex ids; null = vertices 0..n-1).
+// prepare_build_scratch(n) and ensure_table_storage must have been called.
+int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
+  hipStream_t st = g->stream;
+  BuildScratch& sc = g_scratch;
+  uint32_t counts[CLS_COUNT] = {0}, starts[CLS_COUNT] = {0};
+  if (n > 0) {
+    SKY_HIP(hipMemsetAsync(sc.counters, 0, 2 * CLS_COUNT * 4, st));
+    const uint32_t grid = std::min<uint32_t>((n + 255) / 256, 256 * 8);
+    hipLaunchKernelGGL(bin_count_kernel, dim3(grid), dim3(256), 0, st, g->xadj, src, n, sc.counters);
+    SKY_HIP(hipMemcpyAsync(counts, sc.counters, sizeof(counts), hipMemcpyDeviceToHost, st));
+    SKY_HIP(hipStreamSynchronize(st));
+    uint32_t acc = 0;
+    for (int c = 0; c < CLS_COUNT; ++c) {
+      starts[c] = acc;
+      acc += counts[c];
+    }
+    SKY_HIP(hipMemcpyAsync(sc.counters + CLS_COUNT, starts, sizeof(starts), hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(bin_scatter_kernel, dim3((n + 256 * BIN_ITEMS - 1) / (256 * BIN_ITEMS)), dim3(256), 0, st,
+                       g->xadj, g->adjwgt, src, n, sc.counters + CLS_COUNT, sc.vlist, g->prob, g->alias, g->valid);
+  }
+  if (tm) SKY_TRY(tm->mark("bin", 0));
+  uint32_t* const vlist = sc.vlist;
+
+  auto sub = [&](int cls, auto kernel, int G, const char* name) -> int {
+    const uint32_t cnt = counts[cls];
+    if (cnt) {
+      const uint32_t per_block = 256 / G;
+      hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, st, vlist + starts[cls],
+                         cnt, g->xadj, g->adjwgt, g->prob, g->alias, g->valid);
+    }
+    return tm ? tm->mark(name, cnt) : SKY_OK;
+  };
+  SKY_TRY(sub(CLS_SUB4, build_subwave_kernel<4>, 4, "sub4"));
+  SKY_TRY(sub(CLS_SUB8, build_subwave_kernel<8>, 8, "sub8"));
+  SKY_TRY(sub(CLS_SUB16, build_subwave_kernel<16>, 16, "sub16"));
+  SKY_TRY(sub(CLS_SUB32, build_subwave_kernel<32>, 32, "sub32"));
+  SKY_TRY(sub(CLS_WAVE, build_subwave_kernel<64>, 64, "wave64"));
+
+  auto lds = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
+    const uint32_t cnt = counts[cls];
+    if (cnt) {
+      const size_t bytes = (size_t)rowt * 4 * t * 16;
+      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
+                         g->prob, g->alias, g->valid);
+    }
+    return tm ? tm->mark(name, cnt) : SKY_OK;
+  };
+  SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
+  SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<64, 4>, 64, 4, "lds_w4"));
+  SKY_TRY(lds(CLS_LDS_B4, build_lds_kernel<256, 4>, 256, 4, "lds_b4"));
+  SKY_TRY(lds(CLS_LDS_X2, build_lds_kernel<1024, 2>, 1024, 2, "lds_x2"));
+
+  if (counts[CLS_HUGE]) {
+    const uint32_t cnt = counts[CLS_HUGE];
+    if (sc.huge_cap < cnt) {
+      if (sc.huge_off) SKY_HIP(hipFree(sc.huge_off));
+      sc.huge_off = nullptr;
+      sc.huge_cap = 0;
+      SKY_HIP(hipMalloc((void**)&sc.huge_off, ((size_t)cnt + 1) * 8));
+      sc.huge_cap = cnt;
+    }
+    hipLaunchKernelGGL(huge_prefix_kernel, dim3(1), dim3(1024), 0, st, sc.vlist + starts[CLS_HUGE], cnt, g->xadj,
+                       sc.huge_off, sc.huge_off + cnt);
+    uint64_t total = 0;
+    SKY_HIP(hipMemcpyAsync(&total, sc.huge_off + cnt, 8, hipMemcpyDeviceToHost, st));
+    SKY_HIP(hipStreamSynchronize(st));
+    if (sc.huge_scratch_cap < total) {
+      if (sc.huge_scratch) SKY_HIP(hipFree(sc.huge_scratch));
+      sc.huge_scratch = nullptr;
+      sc.huge_scratch_cap = 0;
+      SKY_HIP(hipMalloc((void**)&sc.huge_scratch, total * 16));
+      sc.huge_scratch_cap = total;
+    }
+    hipLaunchKernelGGL(build_huge_kernel, dim3(std::min<uint32_t>(cnt, 512)), dim3(HUGE_T), 0, st,
+                       sc.vlist + starts[CLS_HUGE], cnt, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch, g->prob,
+                       g->alias, g->valid);
+  }
+  if (tm) SKY_TRY(tm->mark("huge", counts[CLS_HUGE]));
+  return SKY_OK;
+}
+
+int build_all_tables(sky_graph* g, double* seconds) {
+  SKY_TRY(ensure_table_storage(g));
+  SKY_TRY(prepare_build_scratch(g->V));
+  EventTimer tm(g->stream);
+  SKY_TRY(tm.mark("start", 0));
+  SKY_TRY(build_rows(g, nullptr, g->V, &tm));
+  SKY_TRY(tm.finish(&g->build_profile, seconds));
+  g->has_tables = true;
+  return SKY_OK;
+}
+
+}  // namespace sky

@@ -1,0 +1,302 @@
+// extern "C" surface of libskywalker_hip.so (declared in include/skywalker_hip.h).
+#include <cstring>
+
+#include "sky_graph.h"
+
+namespace sky {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string& msg) { g_last_error = msg; }
+int fail(int code, const std::string& msg) {
+  g_last_error = msg;
+  return code;
+}
+
+static int ensure_device() {
+  static thread_local bool checked = false;
+  if (checked) return SKY_OK;
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return fail(SKY_ERR_NO_GPU, "no HIP device is visible to this process");
+  }
+  checked = true;
+  return SKY_OK;
+}
+
+}  // namespace sky
+
+using namespace sky;
+
+extern "C" {
+
+const char* sky_last_error(void) { return g_last_error.c_str(); }
+const char* sky_version(void) { return "skywalker_hip 0.1 (gfx950)"; }
+
+int sky_device_malloc(size_t bytes, void** out) {
+  if (!out) return fail(SKY_ERR_ARG, "sky_device_malloc: null output");
+  SKY_TRY(ensure_device());
+  SKY_HIP(hipMalloc(out, bytes ? bytes : 16));
+  return SKY_OK;
+}
+int sky_device_free(void* p) {
+  if (p) SKY_HIP(hipFree(p));
+  return SKY_OK;
+}
+int sky_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  if (bytes && (!dst || !src)) return fail(SKY_ERR_ARG, "sky_memcpy_h2d: null pointer");
+  if (bytes) SKY_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  return SKY_OK;
+}
+int sky_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  if (bytes && (!dst || !src)) return fail(SKY_ERR_ARG, "sky_memcpy_d2h: null pointer");
+  if (bytes) SKY_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return SKY_OK;
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+int sky_device_fill_u32(void* dst, uint32_t value, size_t count) {
+  if (count && !dst) return fail(SKY_ERR_ARG, "sky_device_fill_u32: null pointer");
+  if (count) {
+    const unsigned grid = (unsigned)std::min<size_t>((count + 255) / 256, 65536);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(grid), dim3(256), 0, nullptr, (uint32_t*)dst, value, count);
+    SKY_HIP(hipStreamSynchronize(nullptr));
+    SKY_HIP(hipGetLastError());
+  }
+  return SKY_OK;
+}
+int sky_device_synchronize(void) {
+  SKY_HIP(hipDeviceSynchronize());
+  return SKY_OK;
+}
+int sky_device_name(char* buf, size_t buflen, int* compute_units) {
+  SKY_TRY(ensure_device());
+  hipDeviceProp_t prop;
+  int dev = 0;
+  SKY_HIP(hipGetDevice(&dev));
+  SKY_HIP(hipGetDeviceProperties(&prop, dev));
+  if (buf && buflen) {
+    std::string s = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+    strncpy(buf, s.c_str(), buflen - 1);
+    buf[buflen - 1] = 0;
+  }
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  return SKY_OK;
+}
+
+static int check_csr(const uint32_t* xadj, uint32_t V, uint32_t E) {
+  if (xadj[0] != 0 || xadj[V] != E) return fail(SKY_ERR_ARG, "sky_graph_upload: xadj[0] != 0 or xadj[V] != E");
+  for (uint32_t v = 0; v < V; ++v)
+    if (xadj[v] > xadj[v + 1]) return fail(SKY_ERR_ARG, "sky_graph_upload: xadj is not monotone");
+  return SKY_OK;
+}
+
+int sky_graph_upload(const uint32_t* xadj, const uint32_t* adjncy, const float* adjwgt, uint32_t V, uint32_t E,
+                     sky_graph** out) {
+  if (!out || !xadj || (E && !adjncy)) return fail(SKY_ERR_ARG, "sky_graph_upload: null pointer");
+  SKY_TRY(ensure_device());
+  SKY_TRY(check_csr(xadj, V, E));
+  for (uint32_t i = 0; i < E; ++i)
+    if (adjncy[i] >= V) return fail(SKY_ERR_ARG, "sky_graph_upload: neighbour id out of range");
+  sky_graph* g = new sky_graph();
+  g->V = V;
+  g->E = E;
+  int rc = SKY_OK;
+  auto body = [&]() -> int {
+    SKY_TRY(alloc_padded(&g->xadj, (size_t)V + 1));
+    SKY_TRY(alloc_padded(&g->adjncy, (size_t)E));
+    SKY_TRY(alloc_padded(&g->adjwgt, (size_t)E));
+    SKY_HIP(hipMemcpy(g->xadj, xadj, ((size_t)V + 1) * 4, hipMemcpyHostToDevice));
+    if (E) SKY_HIP(hipMemcpy(g->adjncy, adjncy, (size_t)E * 4, hipMemcpyHostToDevice));
+    if (E) {
+      if (adjwgt) {
+        SKY_HIP(hipMemcpy(g->adjwgt, adjwgt, (size_t)E * 4, hipMemcpyHostToDevice));
+      } else {
+        SKY_TRY(sky_device_fill_u32(g->adjwgt, 0x3F800000u, E));  // 1.0f
+      }
+    }
+    return compute_max_degree(g);
+  };
+  rc = body();
+  if (rc != SKY_OK) {
+    std::string keep = g_last_error;
+    sky_graph_free(g);
+    g_last_error = keep;
+    return rc;
+  }
+  *out = g;
+  return SKY_OK;
+}
+
+int sky_graph_generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int weight_kind, float wa,
+                            float wb, uint64_t weight_seed, sky_graph** out) {
+  SKY_TRY(ensure_device());
+  return generate_rmat(scale, edge_factor, graph_seed, weight_kind, wa, wb, weight_seed, out);
+}
+
+int sky_graph_info(const sky_graph* g, uint32_t* V, uint32_t* E, uint32_t* max_degree) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_graph_info: null graph");
+  if (V) *V = g->V;
+  if (E) *E = g->E;
+  if (max_degree) *max_degree = g->max_degree;
+  return SKY_OK;
+}
+
+int sky_graph_download(const sky_graph* g, uint32_t* xadj, uint32_t* adjncy, float* adjwgt) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_graph_download: null graph");
+  if (xadj) SKY_HIP(hipMemcpy(xadj, g->xadj, ((size_t)g->V + 1) * 4, hipMemcpyDeviceToHost));
+  if (adjncy && g->E) SKY_HIP(hipMemcpy(adjncy, g->adjncy, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  if (adjwgt && g->E) SKY_HIP(hipMemcpy(adjwgt, g->adjwgt, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  return SKY_OK;
+}
+
+int sky_graph_device_ptrs(const sky_graph* g, const uint32_t** xadj, const uint32_t** adjncy, const float** adjwgt,
+                          const float** prob, const uint32_t** alias, const int8_t** valid) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_graph_device_ptrs: null graph");
+  if (xadj) *xadj = g->xadj;
+  if (adjncy) *adjncy = g->adjncy;
+  if (adjwgt) *adjwgt = g->adjwgt;
+  if (prob) *prob = g->prob;
+  if (alias) *alias = g->alias;
+  if (valid) *valid = g->valid;
+  return SKY_OK;
+}
+
+int sky_graph_free(sky_graph* g) {
+  if (!g) return SKY_OK;
+  void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->prob, g->alias, g->valid};
+  for (void* p : ptrs)
+    if (p) (void)hipFree(p);
+  delete g;
+  return SKY_OK;
+}
+
+int sky_alias_build_all(sky_graph* g, double* seconds) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_alias_build_all: null graph");
+  if (g->E && !g->adjwgt) return fail(SKY_ERR_STATE, "sky_alias_build_all: graph has no weights");
+  return build_all_tables(g, seconds);
+}
+
+int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_alias_download: null graph");
+  if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_alias_download: tables have not been built");
+  if (prob && g->E) SKY_HIP(hipMemcpy(prob, g->prob, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  if (alias && g->E) SKY_HIP(hipMemcpy(alias, g->alias, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  if (valid && g->V) SKY_HIP(hipMemcpy(valid, g->valid, (size_t)g->V, hipMemcpyDeviceToHost));
+  return SKY_OK;
+}
+
+int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, const int8_t* valid) {
+  if (!g || !prob || !alias || !valid) return fail(SKY_ERR_ARG, "sky_alias_upload: null pointer");
+  if (!g->prob) SKY_TRY(alloc_padded(&g->prob, (size_t)g->E));
+  if (!g->alias) SKY_TRY(alloc_padded(&g->alias, (size_t)g->E));
+  if (!g->valid) SKY_TRY(alloc_padded(&g->valid, (size_t)g->V));
+  if (g->E) SKY_HIP(hipMemcpy(g->prob, prob, (size_t)g->E * 4, hipMemcpyHostToDevice));
+  if (g->E) SKY_HIP(hipMemcpy(g->alias, alias, (size_t)g->E * 4, hipMemcpyHostToDevice));
+  if (g->V) SKY_HIP(hipMemcpy(g->valid, valid, (size_t)g->V, hipMemcpyHostToDevice));
+  g->has_tables = true;
+  return SKY_OK;
+}
+
+int sky_gen_seeds(uint64_t seed, uint32_t V, uint32_t N, uint32_t* seeds_device) {
+  if (N && !seeds_device) return fail(SKY_ERR_ARG, "sky_gen_seeds: null pointer");
+  if (V == 0) return fail(SKY_ERR_ARG, "sky_gen_seeds: empty graph");
+  SKY_TRY(ensure_device());
+  return gen_seeds(seed, V, N, seeds_device);
+}
+
+static int check_walk_args(const char* who, sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len,
+                           float stop_prob, const uint32_t* paths, const uint32_t* lengths) {
+  if (!g) return fail(SKY_ERR_ARG, std::string(who) + ": null graph");
+  if (N && (!seeds || !paths || !lengths)) return fail(SKY_ERR_ARG, std::string(who) + ": null pointer");
+  if (!(stop_prob >= 0.0f && stop_prob <= 1.0f)) return fail(SKY_ERR_ARG, std::string(who) + ": stop_prob not in [0,1]");
+  if ((uint64_t)N * ((uint64_t)len + 1) > (1ull << 40)) return fail(SKY_ERR_LIMIT, std::string(who) + ": output too large");
+  return SKY_OK;
+}
+
+int sky_walk_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uint32_t len, float stop_prob,
+                     uint64_t philox_seed, uint32_t* paths_device, uint32_t* lengths_device, uint64_t* sampled,
+                     double* seconds) {
+  SKY_TRY(check_walk_args("sky_walk_offline", g, seeds_device, N, len, stop_prob, paths_device, lengths_device));
+  if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_walk_offline: alias tables have not been built");
+  return walk_offline(g, seeds_device, N, len, stop_prob, philox_seed, paths_device, lengths_device, sampled, seconds);
+}
+
+int sky_walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds_device, uint32_t N,
+                    uint32_t len, float stop_prob, uint64_t philox_seed, uint32_t* paths_device,
+                    uint32_t* lengths_device, uint64_t* sampled, double* seconds) {
+  SKY_TRY(check_walk_args("sky_walk_online", g, seeds_device, N, len, stop_prob, paths_device, lengths_device));
+  if (bias_kind != SKY_BIAS_STATIC && bias_kind != SKY_BIAS_NODE2VEC)
+    return fail(SKY_ERR_ARG, "sky_walk_online: unknown bias kind");
+  if (bias_kind == SKY_BIAS_NODE2VEC && !(p > 0.0f && q > 0.0f))
+    return fail(SKY_ERR_ARG, "sky_walk_online: node2vec needs p > 0 and q > 0");
+  return walk_online(g, bias_kind, p, q, seeds_device, N, len, stop_prob, philox_seed, paths_device, lengths_device,
+                     sampled, seconds);
+}
+
+int sky_sample_layout(const uint32_t* fanout, uint32_t hops, uint64_t* length_per_sample,
+                      uint64_t* size_of_sample_lengths) {
+  if (!fanout || hops < 2 || hops > 8 || fanout[0] != 1)
+    return fail(SKY_ERR_ARG, "sky_sample_layout: need 2..8 hops with fanout[0] == 1");
+  uint64_t width = 1, lps = 0, slen = 0;
+  for (uint32_t h = 0; h < hops; ++h) {
+    if (fanout[h] == 0) return fail(SKY_ERR_ARG, "sky_sample_layout: zero fanout");
+    width *= fanout[h];
+    if (width > (1ull << 32)) return fail(SKY_ERR_LIMIT, "sky_sample_layout: fanout product too large");
+    lps += width;
+    if (h + 1 < hops) slen += width;
+  }
+  if (length_per_sample) *length_per_sample = lps;
+  if (size_of_sample_lengths) *size_of_sample_lengths = slen;
+  return SKY_OK;
+}
+
+static int sample_common(const char* who, bool online, sky_graph* g, const uint32_t* seeds, uint32_t N,
+                         const uint32_t* fanout, uint32_t hops, uint64_t seed, uint32_t* data, uint32_t* sl,
+                         uint64_t* sampled, double* seconds) {
+  if (!g) return fail(SKY_ERR_ARG, std::string(who) + ": null graph");
+  if (N && (!seeds || !data || !sl)) return fail(SKY_ERR_ARG, std::string(who) + ": null pointer");
+  uint64_t lps = 0, slen = 0;
+  SKY_TRY(sky_sample_layout(fanout, hops, &lps, &slen));
+  if (!online && !g->has_tables) return fail(SKY_ERR_STATE, std::string(who) + ": alias tables have not been built");
+  return sample_khop(g, online, seeds, N, fanout, hops, seed, data, sl, sampled, seconds);
+}
+
+int sky_sample_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                       uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device,
+                       uint64_t* sampled, double* seconds) {
+  return sample_common("sky_sample_offline", false, g, seeds_device, N, fanout, hops, philox_seed, data_device,
+                       sample_lengths_device, sampled, seconds);
+}
+int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                      uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device, uint64_t* sampled,
+                      double* seconds) {
+  return sample_common("sky_sample_online", true, g, seeds_device, N, fanout, hops, philox_seed, data_device,
+                       sample_lengths_device, sampled, seconds);
+}
+
+int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint32_t n, uint32_t* out_host) {
+  if (n && (!ctr_host || !key_host || !out_host)) return fail(SKY_ERR_ARG, "sky_philox_selftest: null pointer");
+  SKY_TRY(ensure_device());
+  if (n == 0) return SKY_OK;
+  return philox_selftest(ctr_host, key_host, n, out_host);
+}
+
+int sky_last_build_profile(const sky_graph* g, const char** names, float* ms, uint64_t* edges, int max_entries) {
+  if (!g) return 0;
+  int n = 0;
+  for (const auto& e : g->build_profile) {
+    if (n >= max_entries) break;
+    if (names) names[n] = e.name;
+    if (ms) ms[n] = e.ms;
+    if (edges) edges[n] = e.edges;
+    ++n;
+  }
+  return n;
+}
+
+}  // extern "C"

@@ -1,0 +1,188 @@
+// Shared device/host helpers of libskywalker_hip (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/skywalker_hip.h"
+
+namespace sky {
+
+// ---------------------------------------------------------------- error plumbing
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+
+#define SKY_HIP(expr)                                                                                 \
+  do {                                                                                                \
+    hipError_t _e = (expr);                                                                           \
+    if (_e != hipSuccess)                                                                             \
+      return ::sky::fail(SKY_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(_e) + " (" +      \
+                                          __FILE__ + ":" + std::to_string(__LINE__) + ")");           \
+  } while (0)
+
+#define SKY_TRY(expr)         \
+  do {                        \
+    int _rc = (expr);         \
+    if (_rc != SKY_OK) return _rc; \
+  } while (0)
+
+// ---------------------------------------------------------------- Philox4x32-10
+// Counter = (a, b, c, domain), key = 64-bit seed.  Domains separate the streams of
+// the generators and of the samplers so that no two consumers share a counter.
+enum : uint32_t { DOM_RMAT = 1, DOM_WEIGHT = 2, DOM_SEEDS = 3, DOM_WALK = 4, DOM_SAMPLE = 5 };
+
+struct u32x4 {
+  uint32_t x, y, z, w;
+};
+
+__device__ __forceinline__ u32x4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                               uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    c0 = hi1 ^ c1 ^ k0;
+    c1 = lo1;
+    c2 = hi0 ^ c3 ^ k1;
+    c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return u32x4{c0, c1, c2, c3};
+}
+__device__ __forceinline__ u32x4 philox(uint64_t seed, uint32_t a, uint32_t b, uint32_t c, uint32_t dom) {
+  return philox4x32_10(a, b, c, dom, (uint32_t)seed, (uint32_t)(seed >> 32));
+}
+// 24-bit uniform in [0,1): every value and the comparison against an fp32 prob are exact.
+__device__ __forceinline__ float u24(uint32_t r) { return (float)(r >> 8) * (1.0f / 16777216.0f); }
+
+// ---------------------------------------------------------------- exact weight arithmetic
+// The build sums weights as 128-bit fixed point (grid 2^-64) so that the total, and with it
+// every table entry, does not depend on the order of the parallel reduction.
+struct u128 {
+  uint64_t lo, hi;
+};
+__device__ __forceinline__ u128 add128(u128 a, u128 b) {
+  u128 r;
+  r.lo = a.lo + b.lo;
+  r.hi = a.hi + b.hi + (r.lo < a.lo ? 1ull : 0ull);
+  return r;
+}
+__device__ __forceinline__ float clamp_weight(float w) {
+  if (!(w > 0.0f)) return 0.0f;  // zero, negatives, NaN
+  return w > 4294967296.0f ? 4294967296.0f : w;
+}
+// floor(w * 2^64) of a clamped weight.
+__device__ __forceinline__ u128 weight_fixed(float w) {
+  const uint32_t bits = __float_as_uint(w);
+  const uint32_t e = (bits >> 23) & 0xFFu;
+  const uint64_t m = (bits & 0x7FFFFFu) | 0x800000u;
+  const int sh = (int)e - 86;
+  u128 r{0, 0};
+  if (e == 0 || sh <= -24) return r;
+  if (sh < 0) {
+    r.lo = m >> (-sh);
+  } else if (sh < 64) {
+    r.lo = m << sh;
+    r.hi = sh ? (m >> (64 - sh)) : 0;
+  } else {
+    r.hi = m << (sh - 64);
+  }
+  return r;
+}
+__device__ __forceinline__ double fixed_to_double(u128 s) {
+  const uint32_t l0 = (uint32_t)s.lo, l1 = (uint32_t)(s.lo >> 32), l2 = (uint32_t)s.hi, l3 = (uint32_t)(s.hi >> 32);
+  const double hi = (double)l3 * 4294967296.0 + (double)l2;
+  const double lo = (double)l1 * (1.0 / 4294967296.0) + (double)l0 * (1.0 / 18446744073709551616.0);
+  return hi + lo;
+}
+
+// The integer ledger of a row keeps F fraction bits: 40, fewer only for rows of 2^22 entries
+// and more so that the row's prefix sums stay below 2^63.
+struct Ledger {
+  double scale;   // deg / sum(w): p = w * scale
+  double fs;      // 2^F
+  double inv_fs;  // 2^-F
+  uint64_t one;   // 2^F
+};
+__device__ __forceinline__ Ledger make_ledger(uint32_t deg, u128 sum) {
+  const int F = deg < (1u << 22) ? 40 : 62 - (31 - __clz((int)deg));
+  Ledger L;
+  L.scale = (double)deg / fixed_to_double(sum);
+  L.one = 1ull << F;
+  L.fs = (double)L.one;
+  L.inv_fs = 1.0 / L.fs;
+  return L;
+}
+// Per-entry classification: t = (p - 1) * 2^F; heavy iff t >= 0.5.
+struct Entry {
+  double p;
+  uint64_t amount;  // surplus (heavy) or deficit (light), units of 2^-F
+  bool heavy;
+};
+__device__ __forceinline__ Entry classify(float w, const Ledger& L) {
+  Entry e;
+  e.p = (double)w * L.scale;
+  const double t = (e.p - 1.0) * L.fs;
+  e.heavy = t >= 0.5;
+  e.amount = (uint64_t)floor((e.heavy ? t : -t) + 0.5);
+  return e;
+}
+__device__ __forceinline__ float residual_prob(uint64_t r_units, const Ledger& L) {
+  return (float)((double)r_units * L.inv_fs);
+}
+
+// ---------------------------------------------------------------- wave64 primitives
+__device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
+
+__device__ __forceinline__ uint64_t shfl_u64(uint64_t v, int src) {
+  const uint32_t lo = __shfl((int)(uint32_t)v, src, 64);
+  const uint32_t hi = __shfl((int)(uint32_t)(v >> 32), src, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask) {
+  const uint32_t lo = __shfl_xor((int)(uint32_t)v, mask, 64);
+  const uint32_t hi = __shfl_xor((int)(uint32_t)(v >> 32), mask, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ uint64_t shfl_up_u64(uint64_t v, int delta) {
+  const uint32_t lo = __shfl_up((int)(uint32_t)v, delta, 64);
+  const uint32_t hi = __shfl_up((int)(uint32_t)(v >> 32), delta, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+// Sum over aligned groups of G lanes; every lane of the group receives the total.
+template <int G>
+__device__ __forceinline__ u128 group_sum_u128(u128 v) {
+#pragma unroll
+  for (int m = 1; m < G; m <<= 1) {
+    u128 o;
+    o.lo = shfl_xor_u64(v.lo, m);
+    o.hi = shfl_xor_u64(v.hi, m);
+    v = add128(v, o);
+  }
+  return v;
+}
+// Inclusive prefix sum over aligned groups of G lanes.
+template <int G>
+__device__ __forceinline__ uint64_t group_scan_u64(uint64_t v) {
+  const int gl = lane_id() & (G - 1);
+#pragma unroll
+  for (int d = 1; d < G; d <<= 1) {
+    const uint64_t o = shfl_up_u64(v, d);
+    if (gl >= d) v += o;
+  }
+  return v;
+}
+template <int G>
+__device__ __forceinline__ uint32_t group_scan_u32(uint32_t v) {
+  const int gl = lane_id() & (G - 1);
+#pragma unroll
+  for (int d = 1; d < G; d <<= 1) {
+    const uint32_t o = __shfl_up((int)v, d, 64);
+    if (gl >= d) v += o;
+  }
+  return v;
+}
+
+}  // namespace sky

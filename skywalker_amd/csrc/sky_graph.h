@@ -1,0 +1,85 @@
+// Internal definition of the opaque sky_graph handle.
+#pragma once
+#include <vector>
+
+#include "sky_common.h"
+
+struct sky_graph {
+  uint32_t V = 0, E = 0, max_degree = 0;
+  // CSR, device resident.  Arrays are allocated with 16 spare bytes so that kernels may
+  // read whole aligned float4/uint4 quads that straddle the end.
+  uint32_t* xadj = nullptr;    // [V+1]
+  uint32_t* adjncy = nullptr;  // [E]
+  float* adjwgt = nullptr;     // [E]
+  // alias tables: slot i of the table is CSR slot i; alias holds a row-local index
+  float* prob = nullptr;      // [E]
+  uint32_t* alias = nullptr;  // [E]
+  int8_t* valid = nullptr;    // [V]
+  bool has_tables = false;
+  hipStream_t stream = nullptr;  // null stream, like the reference ("0 stream everywhere")
+
+  struct ProfileEntry {
+    const char* name;
+    float ms;
+    uint64_t edges;
+  };
+  std::vector<ProfileEntry> build_profile;
+};
+
+namespace sky {
+
+// Degree classes of the offline build.  Upper bounds are inclusive.
+enum BuildClass : int {
+  CLS_EMPTY = 0,   // deg 0            handled while binning
+  CLS_TINY = 1,    // deg 1..2         one lane per vertex, handled while binning
+  CLS_SUB4 = 2,    // deg 3..4         4 lanes per vertex
+  CLS_SUB8 = 3,    // deg 5..8
+  CLS_SUB16 = 4,   // deg 9..16
+  CLS_SUB32 = 5,   // deg 17..32
+  CLS_WAVE = 6,    // deg 33..64       one wavefront, one entry per lane
+  CLS_LDS_W1 = 7,  // deg <= 253       one wavefront, LDS prefix arrays, 4 entries per lane
+  CLS_LDS_W4 = 8,  // deg <= 1021      one wavefront, 16 entries per lane
+  CLS_LDS_B4 = 9,  // deg <= 4093      256 threads
+  CLS_LDS_X2 = 10, // deg <= 8189      1024 threads, 128 KB of LDS
+  CLS_HUGE = 11,   // above            1024 threads streaming through a global scratch
+  CLS_COUNT = 12
+};
+
+// Sequence of HIP events on one stream; consecutive marks bracket one kernel (or group).
+struct EventTimer {
+  hipStream_t stream;
+  std::vector<hipEvent_t> ev;
+  std::vector<const char*> names;
+  std::vector<uint64_t> edges;
+  explicit EventTimer(hipStream_t s) : stream(s) {}
+  ~EventTimer();
+  int mark(const char* name, uint64_t edges);
+  // synchronises, then fills `profile` (may be null) and the time from first to last mark
+  int finish(std::vector<sky_graph::ProfileEntry>* profile, double* seconds);
+};
+
+int ensure_table_storage(sky_graph* g);
+int prepare_build_scratch(uint32_t max_rows);
+int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm);
+int build_all_tables(sky_graph* g, double* seconds);
+int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
+                 uint32_t* paths, uint32_t* lengths, uint64_t* sampled, double* seconds);
+int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
+                float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
+                double* seconds);
+int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds);
+int generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int weight_kind, float wa, float wb,
+                  uint64_t weight_seed, sky_graph** out);
+int gen_seeds(uint64_t seed, uint32_t V, uint32_t N, uint32_t* seeds_device);
+int philox_selftest(const uint32_t* ctr, const uint32_t* key, uint32_t n, uint32_t* out);
+int compute_max_degree(sky_graph* g);
+
+// Device allocation with the spare bytes described above.
+template <class T>
+int alloc_padded(T** p, size_t count) {
+  SKY_HIP(hipMalloc((void**)p, count * sizeof(T) + 16));
+  return SKY_OK;
+}
+
+}  // namespace sky

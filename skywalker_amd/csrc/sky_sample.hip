@@ -1,0 +1,176 @@
+// k-hop neighbour sampling (replaces the fused sample_kernel and OfflineSample of
+// src/offline_sample.cu:72-141,443-513, and sample_kernel / OnlineGBSampleNew of
+// src/online_sample_new.cu:191-270,459-547).
+//
+// Output layout (include/sampler_result.cuh:226-260,421-426): per seed, hop h occupies
+// width[h] = prod fanout[0..h] slots starting at offsets[h]; the children of slot s of hop h are
+// slots s*fanout[h+1].. of hop h+1; sample_lengths holds one count per parent slot of every hop
+// but the last.  A parent of degree deg with fanout k contributes all its neighbours when
+// k >= deg, else k alias draws with replacement; draw i of slot s uses
+// Philox(seed; seed index, s*k + i, h, DOM_SAMPLE).  One lane per (seed, slot, draw), one launch
+// per hop: no device-side queues, and the result does not depend on scheduling.
+//
+// Online mode builds the table of every distinct frontier vertex, once, through the same
+// kernels as the offline build (into the graph's table storage), then samples the hop.
+#include "sky_graph.h"
+
+namespace sky {
+
+struct HopGeom {
+  uint32_t h, k, fan_h;          // hop index, fanout of the next hop, fanout of this hop
+  uint64_t width, off, off_next; // slots of hop h, where they start, where hop h+1 starts
+  uint64_t loff, loff_prev;      // sample_lengths offsets of hop h and h-1
+  uint64_t lps, slen;            // per-seed strides of data and sample_lengths
+};
+
+__device__ __forceinline__ bool slot_filled(const HopGeom& g, const uint32_t* sl, uint64_t si, uint64_t s) {
+  if (g.h == 0) return true;
+  return sl[si * g.slen + g.loff_prev + s / g.fan_h] > (uint32_t)(s % g.fan_h);
+}
+
+__global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restrict__ xadj,
+                                                         const uint32_t* __restrict__ adjncy,
+                                                         const float* __restrict__ prob,
+                                                         const uint32_t* __restrict__ alias, uint64_t total,
+                                                         HopGeom g, uint64_t seed, uint32_t* __restrict__ data,
+                                                         uint32_t* __restrict__ sl,
+                                                         unsigned long long* __restrict__ sampled) {
+  const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+  unsigned long long mine = 0;
+  if (tid < total) {
+    const uint64_t per_seed = g.width * g.k;
+    const uint64_t si = tid / per_seed, rem = tid % per_seed;
+    const uint64_t s = rem / g.k;
+    const uint32_t i = (uint32_t)(rem % g.k);
+    if (slot_filled(g, sl, si, s)) {
+      const uint32_t v = data[si * g.lps + g.off + s];
+      const uint32_t o = xadj[v], deg = xadj[v + 1] - o;
+      if (deg != 0 && alias[o] != SKY_INVALID) {
+        uint32_t* out = data + si * g.lps + g.off_next + s * g.k;
+        uint32_t cnt;
+        if (g.k >= deg) {
+          cnt = deg;
+          if (i < deg) out[i] = adjncy[o + i];
+        } else {
+          cnt = g.k;
+          const u32x4 r = philox(seed, (uint32_t)si, (uint32_t)(s * g.k + i), g.h, DOM_SAMPLE);
+          const uint32_t col = __umulhi(r.x, deg);
+          const uint32_t cand = u24(r.y) < prob[o + col] ? col : alias[o + col];
+          out[i] = adjncy[o + cand];
+        }
+        if (i == 0) {
+          sl[si * g.slen + g.loff + s] = cnt;
+          mine = cnt;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) mine += shfl_xor_u64(mine, m);
+  if ((threadIdx.x & 63) == 0 && mine) atomicAdd(sampled, mine);
+}
+
+// Collects the distinct vertices of the filled slots of hop h whose table has not been built
+// during this call: first setter of the vertex's bit appends it.
+__global__ __launch_bounds__(256) void frontier_collect_kernel(const uint32_t* __restrict__ data,
+                                                               const uint32_t* __restrict__ sl, uint64_t total,
+                                                               HopGeom g, uint32_t* __restrict__ bitmap,
+                                                               uint32_t* __restrict__ list,
+                                                               uint32_t* __restrict__ count) {
+  const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+  if (tid >= total) return;
+  const uint64_t si = tid / g.width, s = tid % g.width;
+  if (!slot_filled(g, sl, si, s)) return;
+  const uint32_t v = data[si * g.lps + g.off + s];
+  const uint32_t bit = 1u << (v & 31);
+  if (atomicOr(&bitmap[v >> 5], bit) & bit) return;
+  list[atomicAdd(count, 1u)] = v;
+}
+
+__global__ __launch_bounds__(256) void sample_init_kernel(const uint32_t* __restrict__ seeds, uint32_t N, uint64_t lps,
+                                                          uint32_t* __restrict__ data) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i < N) data[(uint64_t)i * lps] = seeds[i];
+}
+
+int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds) {
+  hipStream_t st = g->stream;
+  std::vector<uint64_t> width(hops), off(hops), loff(hops, 0);
+  uint64_t lps = 0, slen = 0, wd = 1;
+  for (uint32_t h = 0; h < hops; ++h) {
+    wd *= fanout[h];
+    width[h] = wd;
+    off[h] = lps;
+    lps += wd;
+    if (h + 1 < hops) {
+      loff[h] = slen;
+      slen += wd;
+    }
+  }
+  if ((uint64_t)N * lps > (1ull << 40)) return fail(SKY_ERR_LIMIT, "sample: output too large");
+
+  unsigned long long* d_sampled = nullptr;
+  uint32_t *bitmap = nullptr, *list = nullptr, *d_count = nullptr;
+  const uint32_t words = (g->V + 31) / 32;
+  auto cleanup = [&]() {
+    if (d_sampled) (void)hipFree(d_sampled);
+    if (bitmap) (void)hipFree(bitmap);
+    if (list) (void)hipFree(list);
+    if (d_count) (void)hipFree(d_count);
+  };
+  auto body = [&]() -> int {
+    SKY_HIP(hipMalloc((void**)&d_sampled, 8));
+    SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
+    if (N && slen) SKY_HIP(hipMemsetAsync(sample_lengths, 0, (size_t)N * slen * 4, st));
+    if (online) {
+      SKY_TRY(ensure_table_storage(g));
+      SKY_TRY(prepare_build_scratch(g->V));
+      SKY_HIP(hipMalloc((void**)&bitmap, (size_t)words * 4 + 16));
+      SKY_HIP(hipMalloc((void**)&list, (size_t)g->V * 4 + 16));
+      SKY_HIP(hipMalloc((void**)&d_count, 4));
+    }
+    EventTimer tm(st);
+    SKY_TRY(tm.mark("start", 0));
+    if (online) SKY_HIP(hipMemsetAsync(bitmap, 0, (size_t)words * 4, st));
+    if (N) hipLaunchKernelGGL(sample_init_kernel, dim3((N + 255) / 256), dim3(256), 0, st, seeds, N, lps, data);
+    for (uint32_t h = 0; h + 1 < hops && N; ++h) {
+      HopGeom hg;
+      hg.h = h;
+      hg.k = fanout[h + 1];
+      hg.fan_h = fanout[h];
+      hg.width = width[h];
+      hg.off = off[h];
+      hg.off_next = off[h + 1];
+      hg.loff = loff[h];
+      hg.loff_prev = h ? loff[h - 1] : 0;
+      hg.lps = lps;
+      hg.slen = slen;
+      if (online) {
+        const uint64_t slots = (uint64_t)N * hg.width;
+        SKY_HIP(hipMemsetAsync(d_count, 0, 4, st));
+        hipLaunchKernelGGL(frontier_collect_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, st, data,
+                           sample_lengths, slots, hg, bitmap, list, d_count);
+        uint32_t cnt = 0;
+        SKY_HIP(hipMemcpyAsync(&cnt, d_count, 4, hipMemcpyDeviceToHost, st));
+        SKY_HIP(hipStreamSynchronize(st));
+        SKY_TRY(build_rows(g, list, cnt, nullptr));
+      }
+      const uint64_t total = (uint64_t)N * hg.width * hg.k;
+      if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");
+      hipLaunchKernelGGL(sample_hop_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, g->xadj,
+                         g->adjncy, g->prob, g->alias, total, hg, seed, data, sample_lengths, d_sampled);
+    }
+    SKY_TRY(tm.mark("sample", 0));
+    SKY_TRY(tm.finish(nullptr, seconds));
+    unsigned long long hcount = 0;
+    SKY_HIP(hipMemcpy(&hcount, d_sampled, 8, hipMemcpyDeviceToHost));
+    if (sampled) *sampled = hcount;
+    return SKY_OK;
+  };
+  const int rc = body();
+  cleanup();
+  return rc;
+}
+
+}  // namespace sky

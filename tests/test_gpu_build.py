@@ -1,0 +1,102 @@
+"""Offline alias build on the GPU (through the C-ABI) against the CPU oracle: bit-exact tables,
+and the reconstruction invariant on every row."""
+import numpy as np
+import pytest
+
+from helpers import graph_from_degrees
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-6
+
+# degrees that straddle every dispatch class boundary of the build
+EDGE_DEGREES = [0, 1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 63, 64, 65, 66, 67, 68, 127, 253, 254, 255, 256, 257, 1021,
+                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 8189, 8190, 8191, 8192, 8193, 20000, 70001]
+
+
+def build_and_compare(orc, xadj, adjncy, w, label):
+    from skywalker_amd import capi
+    print("case", label, "V", len(xadj) - 1, "E", len(w), flush=True)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    prob, alias, valid = g.tables()
+    g.free()
+    oprob, oalias, ovalid = orc.alias_build(xadj, w)
+    st = orc.alias_check(xadj, w, prob, alias, valid)
+    assert st["bad_valid"] == 0 and st["bad_range"] == 0 and st["bad_invalid"] == 0, st
+    assert st["max_rel_err"] < TOL, st
+    bad = np.flatnonzero((prob != oprob) | (alias != oalias))
+    if len(bad):
+        v = int(np.searchsorted(xadj, bad[0], side="right") - 1)
+        raise AssertionError("%s: %d entries differ from the oracle, first at slot %d (vertex %d, degree %d)" %
+                             (label, len(bad), bad[0], v, xadj[v + 1] - xadj[v]))
+    assert np.array_equal(valid, ovalid)
+
+
+@pytest.mark.parametrize("dist", ["lognormal", "uniform", "unit", "lognormal2", "equal", "nearequal", "sparse"])
+def test_every_degree_class(orc, dist):
+    rng = np.random.default_rng(11)
+    degs = EDGE_DEGREES + list(rng.integers(1, 300, 400)) + list(rng.integers(300, 6000, 30))
+    rng.shuffle(degs)
+    xadj, adjncy, w = graph_from_degrees(degs, rng, dist, V=len(degs) + 7)
+    build_and_compare(orc, xadj, adjncy, w, "classes/" + dist)
+
+
+def test_unaligned_row_starts(orc):
+    # rows of every residue mod 4 in front of each LDS-class row
+    rng = np.random.default_rng(5)
+    degs = []
+    for d in (70, 254, 700, 1021, 3000, 4093, 8000, 8189, 9000):
+        for pad in (1, 2, 3, 5):
+            degs += [pad, d]
+    xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal")
+    build_and_compare(orc, xadj, adjncy, w, "unaligned")
+
+
+def test_all_zero_and_empty_rows(orc):
+    rng = np.random.default_rng(2)
+    degs = [0, 5, 0, 40, 100, 1, 2, 3000, 9000, 0]
+    xadj, adjncy, w = graph_from_degrees(degs, rng, "uniform")
+    for v in (1, 3, 4, 5, 6, 7, 8):
+        if v % 2 == 1 or v == 8:
+            w[xadj[v]:xadj[v + 1]] = 0.0
+    build_and_compare(orc, xadj, adjncy, w, "zero rows")
+
+
+def test_hub_row(orc):
+    rng = np.random.default_rng(3)
+    xadj, adjncy, w = graph_from_degrees([1_200_000, 3, 90_000], rng, "lognormal2", V=4096)
+    build_and_compare(orc, xadj, adjncy, w, "hub")
+
+
+def test_config1_rmat_s16(orc):
+    xadj, adjncy = orc.rmat_csr(16, 16, 42)
+    w = orc.gen_weights(orc.W_UNIFORM, 42, len(adjncy), 1.0, 100.0)
+    build_and_compare(orc, xadj, adjncy, w, "config1")
+
+
+def test_rebuild_is_idempotent(orc):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 8, 9)
+    w = orc.gen_weights(orc.W_UNIT, 9, len(adjncy))
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    a = g.tables()
+    g.build_tables()
+    b = g.tables()
+    g.free()
+    for x, y in zip(a, b):
+        assert np.array_equal(x, y)
+
+
+def test_bad_arguments_are_reported(orc):
+    from skywalker_amd import capi
+    xadj = np.array([0, 2, 1], np.uint32)  # not monotone
+    with pytest.raises(capi.SkyError):
+        capi.Graph.upload(xadj, np.zeros(1, np.uint32), np.ones(1, np.float32))
+    xadj = np.array([0, 1], np.uint32)
+    with pytest.raises(capi.SkyError):
+        capi.Graph.upload(xadj, np.array([5], np.uint32), np.ones(1, np.float32))  # neighbour out of range
+    g = capi.Graph.upload(np.array([0, 1, 1], np.uint32), np.array([1], np.uint32), np.ones(1, np.float32))
+    with pytest.raises(capi.SkyError):
+        g.walk_offline(np.array([0], np.uint32), 4, 0.0, 1)  # tables not built
+    g.free()

@@ -1,0 +1,69 @@
+"""k-hop neighbour sampling on the GPU against the oracle: bit-exact blocks and counts."""
+import numpy as np
+import pytest
+
+from helpers import chi_square_p, graph_from_degrees
+
+pytestmark = pytest.mark.gpu
+
+
+def test_layout_closed_form():
+    from skywalker_amd import capi
+    assert capi.sample_layout([1, 25, 10]) == (276, 26)
+    assert capi.sample_layout([1, 2, 2]) == (7, 3)
+    assert capi.sample_layout([1, 20, 20]) == (421, 21)
+
+
+@pytest.mark.parametrize("fanout", [[1, 25, 10], [1, 3, 2, 2], [1, 5]])
+def test_offline_and_online_match_oracle(orc, fanout):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(13, 8, 21)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 21, len(adjncy), 0.0, 1.0)
+    seeds = orc.gen_seeds(4, 1 << 13, 1500)
+    lps, slen = capi.sample_layout(fanout)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    d_on, sl_on, s_on, _ = g.sample_online(seeds, fanout, 17)
+    on = (d_on.to_host((1500, lps)), sl_on.to_host((1500, slen)))
+    g.build_tables()
+    prob, alias, valid = g.tables()
+    d_off, sl_off, s_off, _ = g.sample_offline(seeds, fanout, 17)
+    off = (d_off.to_host((1500, lps)), sl_off.to_host((1500, slen)))
+    g.free()
+    odata, osl, osampled = orc.sample_offline(xadj, adjncy, prob, alias, seeds, fanout, 17)
+    assert np.array_equal(off[1], osl) and np.array_equal(off[0], odata) and s_off == osampled
+    assert np.array_equal(on[0], off[0]) and np.array_equal(on[1], off[1]) and s_on == s_off
+    o2data, o2sl, o2sampled = orc.sample_online(xadj, adjncy, w, seeds, fanout, 17)
+    assert np.array_equal(on[0], o2data) and np.array_equal(on[1], o2sl) and s_on == o2sampled
+    assert osampled == int(osl.sum())
+
+
+def test_exact_count_when_every_degree_exceeds_fanout(orc):
+    from skywalker_amd import capi
+    rng = np.random.default_rng(6)
+    V = 500
+    xadj, adjncy, w = graph_from_degrees(rng.integers(30, 60, V), rng, "uniform", V=V)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    seeds = rng.integers(0, V, 300, dtype=np.uint32)
+    data, sl, sampled, _ = g.sample_offline(seeds, [1, 25, 10], 3)
+    g.free()
+    assert sampled == 300 * (25 + 250)
+    assert not np.any(data.to_host() == 0xFFFFFFFF)
+
+
+def test_per_parent_draw_frequencies(orc):
+    from skywalker_amd import capi
+    rng = np.random.default_rng(9)
+    d = 40
+    xadj = np.zeros(d + 2, np.uint32)
+    xadj[1:] = d
+    adjncy = np.arange(1, d + 1, dtype=np.uint32)
+    w = rng.lognormal(0, 1, d).astype(np.float32)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    N = 20000
+    data, sl, sampled, _ = g.sample_offline(np.zeros(N, np.uint32), [1, 10], 5)
+    g.free()
+    draws = data.to_host((N, 11))[:, 1:].ravel()
+    assert sampled == N * 10
+    assert chi_square_p(np.bincount(draws, minlength=d + 1)[1:], w.astype(np.float64) / w.sum(dtype=np.float64)) > 0.01

@@ -1,0 +1,107 @@
+"""Walks on the GPU against the oracle: bit-exact paths for the same Philox stream and tables."""
+import numpy as np
+import pytest
+
+from helpers import chi_square_p, graph_from_degrees
+
+pytestmark = pytest.mark.gpu
+
+
+def run_offline(orc, xadj, adjncy, w, seeds, length, stop, seed):
+    from skywalker_amd import capi
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    prob, alias, valid = g.tables()
+    paths_d, len_d, sampled, sec = g.walk_offline(seeds, length, stop, seed)
+    paths, lengths = paths_d.to_host((len(seeds), length + 1)), len_d.to_host()
+    g.free()
+    opaths, olengths, osampled = orc.walk_offline(xadj, adjncy, prob, alias, seeds, length, stop, seed)
+    return (paths, lengths, sampled), (opaths, olengths, osampled), (prob, alias, valid)
+
+
+def test_config1_deepwalk_bit_exact(orc):
+    xadj, adjncy = orc.rmat_csr(16, 16, 42)
+    w = orc.gen_weights(orc.W_UNIFORM, 42, len(adjncy), 1.0, 100.0)
+    seeds = orc.gen_seeds(42, 1 << 16, 4096)
+    got, want, _ = run_offline(orc, xadj, adjncy, w, seeds, 80, 0.0, 42)
+    assert np.array_equal(got[1], want[1])
+    assert np.array_equal(got[0], want[0])
+    assert got[2] == want[2] == int(want[1].sum())
+
+
+def test_ppr_bit_exact_and_length_law(orc):
+    # every vertex has out-edges so only the stop test ends a walk
+    rng = np.random.default_rng(4)
+    V = 2000
+    xadj, adjncy, w = graph_from_degrees(rng.integers(1, 40, V), rng, "lognormal", V=V)
+    seeds = rng.integers(0, V, 60000, dtype=np.uint32)
+    tp, L = 0.15, 100
+    got, want, _ = run_offline(orc, xadj, adjncy, w, seeds, L, tp, 7)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]) and got[2] == want[2]
+    lengths = got[1].astype(np.float64)
+    mean = (1 - (1 - tp) ** L) / tp - 1 + (1 - tp) ** L  # E[min(G, L)] with G ~ Geometric(tp) counting failures
+    assert abs(lengths.mean() - mean) < 4 * np.sqrt((1 - tp) / tp**2 / len(seeds))
+    k = np.arange(0, 30)
+    cnt = np.array([(lengths == x).sum() for x in k])
+    pk = tp * (1 - tp) ** k
+    assert chi_square_p(np.append(cnt, len(seeds) - cnt.sum()), np.append(pk, 1 - pk.sum())) > 0.01
+
+
+def test_dead_ends_and_zero_weight_rows(orc):
+    # path graph 0 -> 1 -> 2 -> 3 (3 has no out-edge); vertex 4 has one zero-weight edge; 5 loops on itself
+    xadj = np.array([0, 1, 2, 3, 3, 4, 5], np.uint32)
+    adjncy = np.array([1, 2, 3, 0, 5], np.uint32)
+    w = np.array([1, 1, 1, 0, 2], np.float32)
+    seeds = np.array([0, 1, 2, 3, 4, 5], np.uint32)
+    got, want, _ = run_offline(orc, xadj, adjncy, w, seeds, 6, 0.0, 1)
+    assert got[1].tolist() == [3, 2, 1, 0, 0, 6]
+    assert got[0][0, :4].tolist() == [0, 1, 2, 3] and np.all(got[0][0, 4:] == 0xFFFFFFFF)
+    assert np.all(got[0][5] == 5)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+
+def test_next_hop_frequencies_chi_square(orc):
+    # star: hub 0 with 50 weighted spokes; one step from the hub must follow w / sum(w)
+    rng = np.random.default_rng(8)
+    d = 50
+    xadj = np.zeros(d + 2, np.uint32)
+    xadj[1:] = d
+    adjncy = np.arange(1, d + 1, dtype=np.uint32)
+    w = rng.lognormal(0, 1, d).astype(np.float32)
+    N = 200000
+    seeds = np.zeros(N, np.uint32)
+    got, want, _ = run_offline(orc, xadj, adjncy, w, seeds, 1, 0.0, 3)
+    assert np.array_equal(got[0], want[0])
+    counts = np.bincount(got[0][:, 1], minlength=d + 1)[1:]
+    assert chi_square_p(counts, w.astype(np.float64) / w.astype(np.float64).sum()) > 0.01
+
+
+def test_walk_does_not_depend_on_batch_composition(orc):
+    # walker i's path is a function of (seed, i, start vertex) only
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 8, 5)
+    w = orc.gen_weights(orc.W_UNIT, 5, len(adjncy))
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    seeds = orc.gen_seeds(1, 1 << 12, 3000)
+    full = g.walk_offline(seeds, 20, 0.0, 9)[0].to_host((3000, 21))
+    part = g.walk_offline(seeds[:1000], 20, 0.0, 9)[0].to_host((1000, 21))
+    g.free()
+    assert np.array_equal(full[:1000], part)
+
+
+def test_online_static_walk_equals_offline_and_oracle(orc):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(13, 8, 6)
+    w = orc.gen_weights(orc.W_UNIFORM, 6, len(adjncy), 1.0, 100.0)
+    seeds = orc.gen_seeds(3, 1 << 13, 2000)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    p_on, l_on, s_on, _ = g.walk_online(capi.BIAS_STATIC, 1.0, 1.0, seeds, 30, 0.1, 5)
+    on = (p_on.to_host((2000, 31)), l_on.to_host())
+    g.build_tables()
+    p_off, l_off, s_off, _ = g.walk_offline(seeds, 30, 0.1, 5)
+    off = (p_off.to_host((2000, 31)), l_off.to_host())
+    g.free()
+    assert np.array_equal(on[0], off[0]) and np.array_equal(on[1], off[1]) and s_on == s_off
+    opaths, olengths, osampled = orc.walk_online(xadj, adjncy, w, 0, 1.0, 1.0, seeds, 30, 0.1, 5)
+    assert np.array_equal(on[0], opaths) and np.array_equal(on[1], olengths) and s_on == osampled
