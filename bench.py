@@ -1,0 +1,162 @@
+#!/usr/bin/env python3
+"""Benchmark of the alias-method hot path on one MI355X.
+
+A step = one pass of the hot path over one batch of synthetic input that is already resident in HBM:
+offline alias tables for every vertex (sky_alias_build_all), then a biased DeepWalk of length 80 from the
+batch of start vertices (sky_walk_offline), and for the large configuration also PPR (stop 0.15, max 100).
+Prints ONE JSON line.  Only one GPU is ever used.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X published
+
+# name -> (scale, edge_factor, weight kind, wa, wb, graph seed, walkers, walk length, ppr)
+CONFIGS = {
+    "c1": dict(scale=16, ef=16, wkind="uniform", wa=1.0, wb=100.0, seed=42, walkers=4096, length=80, ppr=False),
+    "c2": dict(scale=20, ef=16, wkind="unit", wa=0.0, wb=0.0, seed=1, walkers=40000, length=80, ppr=False),
+    "c5": dict(scale=26, ef=28, wkind="lognormal", wa=0.0, wb=2.0, seed=5, walkers=1000000, length=80, ppr=True),
+}
+KERNEL_OF = {  # build_profile entry -> kernel symbol
+    "bin": "bin_count_kernel+bin_scatter_kernel", "sub4": "build_subwave_kernel<4>", "sub8": "build_subwave_kernel<8>",
+    "sub16": "build_subwave_kernel<16>", "sub32": "build_subwave_kernel<32>", "wave64": "build_subwave_kernel<64>",
+    "lds_w1": "build_lds_kernel<64,1>", "lds_w4": "build_lds_kernel<64,4>", "lds_b4": "build_lds_kernel<256,4>",
+    "lds_x2": "build_lds_kernel<1024,2>", "huge": "huge_prefix_kernel+build_huge_kernel",
+}
+
+
+def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=400_000_000, walk_sample=65536):
+    """Oracle timed on the host cores, on a bounded sample of the same workload."""
+    import numpy as np
+    V, E = g.V, g.E
+    xadj, adjncy, w = g.download()
+    # build sample: the leading vertex range holding at most budget_edges edges
+    vs = int(np.searchsorted(xadj, min(E, budget_edges), side="right") - 1)
+    vs = max(vs, 1)
+    es = int(xadj[vs])
+    t0 = time.perf_counter()
+    orc.alias_build(np.ascontiguousarray(xadj[:vs + 1]), np.ascontiguousarray(w[:es]))
+    t_build = time.perf_counter() - t0
+    prob, alias, _ = g.tables()
+    seeds = seeds_d.to_host()[:walk_sample]
+    t0 = time.perf_counter()
+    _, _, sampled = orc.walk_offline(xadj, adjncy, prob, alias, seeds, cfg["length"], 0.0, cfg["seed"])
+    t_walk = time.perf_counter() - t0
+    value = (es + sampled) / (t_build + t_walk)
+    return {
+        "value": value, "unit": "edges/s", "cores": orc.num_threads(), "kind": "port",
+        "sample": "oracle (C++/OpenMP) on the same graph: alias build of vertices [0,%d) = %d edges in %.3f s "
+                  "(%.3e edges/s); DeepWalk L=%d of the first %d walkers = %d steps in %.3f s (%.3e steps/s)" %
+                  (vs, es, t_build, es / t_build, cfg["length"], len(seeds), sampled, t_walk, sampled / t_walk),
+        "build_edges_per_s": es / t_build, "walk_seps": sampled / t_walk,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", default="c5", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the multi-GPU path of the reference is out of scope); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch  # device synchronisation brackets only
+    from skywalker_amd import capi
+    import numpy as np
+
+    cfg = CONFIGS[args.config]
+    wk = {"uniform": capi.W_UNIFORM, "unit": capi.W_UNIT, "lognormal": capi.W_LOGNORMAL}[cfg["wkind"]]
+    name, cus = capi.device_name()
+    t_gen = time.perf_counter()
+    g = capi.Graph.rmat(cfg["scale"], cfg["ef"], cfg["seed"], wk, cfg["wa"], cfg["wb"], cfg["seed"])
+    t_gen = time.perf_counter() - t_gen
+    V, E, N, L = g.V, g.E, cfg["walkers"], cfg["length"]
+    seeds = g.gen_seeds(cfg["seed"], N)
+    paths = capi.DeviceArray(N * (L + 1), np.uint32, fill=capi.FILL)
+    lengths = capi.DeviceArray(N, np.uint32, fill=0)
+    if cfg["ppr"]:
+        ppr_paths = capi.DeviceArray(N * 101, np.uint32, fill=capi.FILL)
+        ppr_lengths = capi.DeviceArray(N, np.uint32, fill=0)
+
+    def sync():
+        torch.cuda.synchronize()
+        capi.synchronize()
+
+    rec = []
+
+    def step():
+        r = {}
+        r["build_s"] = g.build_tables()
+        r["profile"] = g.build_profile()
+        _, _, r["walk_edges"], r["walk_s"] = g.walk_offline(seeds, L, 0.0, cfg["seed"], out=(paths, lengths))
+        if cfg["ppr"]:
+            _, _, r["ppr_edges"], r["ppr_s"] = g.walk_offline(seeds, 100, 0.15, cfg["seed"] + 1,
+                                                              out=(ppr_paths, ppr_lengths))
+        return r
+
+    for _ in range(args.warmup):
+        step()
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        rec.append(step())
+    sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    mean = lambda k: sum(r[k] for r in rec) / len(rec)
+    build_s, walk_s, walk_edges = mean("build_s"), mean("walk_s"), rec[-1]["walk_edges"]
+    work = E + walk_edges + (rec[-1]["ppr_edges"] if cfg["ppr"] else 0)
+    build_bytes = 12 * E + 5 * V
+    # dominant kernel of the step, from the per-kernel HIP-event brackets of the build
+    prof = {}
+    for r in rec:
+        for nm, ms, edges in r["profile"]:
+            p = prof.setdefault(nm, [0.0, edges])
+            p[0] += ms / len(rec)
+    dom = max(prof, key=lambda k: prof[k][0])
+    dom_ms, dom_edges = prof[dom]
+    dom_bytes = 12 * dom_edges  # read w, write prob and alias of the class's rows; xadj/valid are per vertex and small
+    out = {
+        "metric": "edges/sec over the hot path (alias-table build edges + sampled walk edges) on 1 MI355X",
+        "value": work / (ms_per_step * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 tables, u64 fixed-point ledger, u32 indices", "data": "synthetic",
+        "config": {"workload": "%s: R-MAT scale %d ef %d (%d V, %d E), %s weights; offline alias build of all vertices "
+                               "+ biased DeepWalk L=%d from %d start vertices%s" %
+                               (args.config, cfg["scale"], cfg["ef"], V, E, cfg["wkind"], L, N,
+                                " + PPR(0.15, max 100)" if cfg["ppr"] else ""),
+                   "device": name, "compute_units": cus, "graph_generation_s": t_gen},
+        "build": {"edges_per_s": E / build_s, "ms": build_s * 1e3, "algorithmic_bytes": build_bytes,
+                  "hbm_frac": build_bytes / build_s / HBM_PEAK,
+                  "kernels_ms": {KERNEL_OF.get(k, k): round(v[0], 4) for k, v in prof.items()}},
+        "walk": {"seps": walk_edges / walk_s, "ms": walk_s * 1e3, "steps": walk_edges,
+                 "algorithmic_bytes": 24 * walk_edges, "hbm_frac": 24 * walk_edges / walk_s / HBM_PEAK},
+        "roofline": {"bound": "hbm", "kernel": KERNEL_OF.get(dom, dom), "achieved": dom_bytes / (dom_ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK,
+                     "traffic": None, "launch_ms": dom_ms, "algorithmic_bytes_per_launch": dom_bytes},
+    }
+    if cfg["ppr"]:
+        ppr_s, ppr_edges = mean("ppr_s"), rec[-1]["ppr_edges"]
+        out["ppr"] = {"seps": ppr_edges / ppr_s, "ms": ppr_s * 1e3, "steps": ppr_edges}
+    if not args.no_cpu:
+        from oracle import orc
+        out["cpu_baseline"] = cpu_baseline(capi, orc, g, cfg, seeds)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -63,17 +63,27 @@ __device__ __forceinline__ uint32_t first_greater(const uint64_t* a, uint32_t lo
 // `src` lists the vertices to bin (n of them); a null src means vertices 0..n-1.
 __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restrict__ xadj,
                                                         const uint32_t* __restrict__ src, uint32_t n,
-                                                        uint32_t* __restrict__ counts) {
+                                                        uint32_t* __restrict__ counts,
+                                                        unsigned long long* __restrict__ class_edges) {
   __shared__ uint32_t s_cnt[CLS_COUNT];
-  if (threadIdx.x < CLS_COUNT) s_cnt[threadIdx.x] = 0;
+  __shared__ unsigned long long s_edges[CLS_COUNT];
+  if (threadIdx.x < CLS_COUNT) {
+    s_cnt[threadIdx.x] = 0;
+    s_edges[threadIdx.x] = 0;
+  }
   __syncthreads();
   for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += gridDim.x * 256u) {
     const uint32_t v = src ? src[i] : i;
-    const int c = degree_class(xadj[v + 1] - xadj[v]);
+    const uint32_t d = xadj[v + 1] - xadj[v];
+    const int c = degree_class(d);
     if (c >= CLS_SUB4) atomicAdd(&s_cnt[c], 1u);
+    if (c >= CLS_TINY) atomicAdd(&s_edges[c], (unsigned long long)d);
   }
   __syncthreads();
-  if (threadIdx.x < CLS_COUNT && s_cnt[threadIdx.x]) atomicAdd(&counts[threadIdx.x], s_cnt[threadIdx.x]);
+  if (threadIdx.x < CLS_COUNT) {
+    if (s_cnt[threadIdx.x]) atomicAdd(&counts[threadIdx.x], s_cnt[threadIdx.x]);
+    if (s_edges[threadIdx.x]) atomicAdd(&class_edges[threadIdx.x], s_edges[threadIdx.x]);
+  }
 }
 
 constexpr int BIN_ITEMS = 4;  // vertices per thread in the scatter pass
@@ -517,9 +527,11 @@ __global__ __launch_bounds__(1024) void huge_prefix_kernel(const uint32_t* __res
 // ---------------------------------------------------------------- host driver
 namespace {
 
+constexpr size_t COUNTER_BYTES = 2 * CLS_COUNT * 4 + CLS_COUNT * 8;
+
 struct BuildScratch {
   uint32_t* vlist = nullptr;     // [vcap]
-  uint32_t* counters = nullptr;  // [2*CLS_COUNT] counts then cursors
+  uint32_t* counters = nullptr;  // [2*CLS_COUNT] counts then cursors, then CLS_COUNT 64-bit edge totals
   uint64_t* huge_off = nullptr;  // [huge_cap + 1], last = total
   uint64_t* huge_scratch = nullptr;
   uint32_t vcap = 0, huge_cap = 0;
@@ -580,7 +592,7 @@ int prepare_build_scratch(uint32_t max_rows) {
     SKY_HIP(hipMalloc((void**)&sc.vlist, (size_t)max_rows * 4 + 16));
     sc.vcap = max_rows;
   }
-  if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, 2 * CLS_COUNT * 4));
+  if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, COUNTER_BYTES));
   if (!sc.lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<64, 4>, 64 * 4 * 4 * 16));
     SKY_TRY(enable_big_lds(build_lds_kernel<256, 4>, 256 * 4 * 4 * 16));
@@ -596,12 +608,19 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   hipStream_t st = g->stream;
   BuildScratch& sc = g_scratch;
   uint32_t counts[CLS_COUNT] = {0}, starts[CLS_COUNT] = {0};
+  struct {
+    uint32_t counts[2 * CLS_COUNT];
+    unsigned long long edges[CLS_COUNT];
+  } host = {};
+  static_assert(sizeof(host) == COUNTER_BYTES, "counter block layout");
   if (n > 0) {
-    SKY_HIP(hipMemsetAsync(sc.counters, 0, 2 * CLS_COUNT * 4, st));
+    SKY_HIP(hipMemsetAsync(sc.counters, 0, COUNTER_BYTES, st));
     const uint32_t grid = std::min<uint32_t>((n + 255) / 256, 256 * 8);
-    hipLaunchKernelGGL(bin_count_kernel, dim3(grid), dim3(256), 0, st, g->xadj, src, n, sc.counters);
-    SKY_HIP(hipMemcpyAsync(counts, sc.counters, sizeof(counts), hipMemcpyDeviceToHost, st));
+    hipLaunchKernelGGL(bin_count_kernel, dim3(grid), dim3(256), 0, st, g->xadj, src, n, sc.counters,
+                       reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
+    SKY_HIP(hipMemcpyAsync(&host, sc.counters, COUNTER_BYTES, hipMemcpyDeviceToHost, st));
     SKY_HIP(hipStreamSynchronize(st));
+    for (int c = 0; c < CLS_COUNT; ++c) counts[c] = host.counts[c];
     uint32_t acc = 0;
     for (int c = 0; c < CLS_COUNT; ++c) {
       starts[c] = acc;
@@ -611,7 +630,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     hipLaunchKernelGGL(bin_scatter_kernel, dim3((n + 256 * BIN_ITEMS - 1) / (256 * BIN_ITEMS)), dim3(256), 0, st,
                        g->xadj, g->adjwgt, src, n, sc.counters + CLS_COUNT, sc.vlist, g->prob, g->alias, g->valid);
   }
-  if (tm) SKY_TRY(tm->mark("bin", 0));
+  if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
   uint32_t* const vlist = sc.vlist;
 
   auto sub = [&](int cls, auto kernel, int G, const char* name) -> int {
@@ -621,7 +640,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, st, vlist + starts[cls],
                          cnt, g->xadj, g->adjwgt, g->prob, g->alias, g->valid);
     }
-    return tm ? tm->mark(name, cnt) : SKY_OK;
+    return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
   SKY_TRY(sub(CLS_SUB4, build_subwave_kernel<4>, 4, "sub4"));
   SKY_TRY(sub(CLS_SUB8, build_subwave_kernel<8>, 8, "sub8"));
@@ -636,7 +655,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
                          g->prob, g->alias, g->valid);
     }
-    return tm ? tm->mark(name, cnt) : SKY_OK;
+    return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
   SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
   SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<64, 4>, 64, 4, "lds_w4"));
@@ -668,7 +687,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
                        sc.vlist + starts[CLS_HUGE], cnt, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch, g->prob,
                        g->alias, g->valid);
   }
-  if (tm) SKY_TRY(tm->mark("huge", counts[CLS_HUGE]));
+  if (tm) SKY_TRY(tm->mark("huge", host.edges[CLS_HUGE]));
   return SKY_OK;
 }
 

@@ -122,9 +122,9 @@ int generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int
   void* temp = nullptr;
   size_t temp_bytes = 0;
   auto cleanup = [&]() {
-    if (keys_a) hipFree(keys_a);
-    if (keys_b) hipFree(keys_b);
-    if (temp) hipFree(temp);
+    if (keys_a) (void)hipFree(keys_a);
+    if (keys_b) (void)hipFree(keys_b);
+    if (temp) (void)hipFree(temp);
   };
 #define GEN_HIP(expr)                                                                              \
   do {                                                                                             \

@@ -64,8 +64,8 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   SKY_HIP(hipGetLastError());
   float ms = 0;
   SKY_HIP(hipEventElapsedTime(&ms, e0, e1));
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
   unsigned long long h = 0;
   SKY_HIP(hipMemcpy(&h, d_sampled, 8, hipMemcpyDeviceToHost));
   SKY_HIP(hipFree(d_sampled));
