@@ -132,9 +132,259 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
   return rc;
 }
 
-int walk_online_node2vec(sky_graph*, float, float, const uint32_t*, uint32_t, uint32_t, float, uint64_t, uint32_t*,
-                         uint32_t*, uint64_t*, double*) {
-  return fail(SKY_ERR_STATE, "sky_walk_online: node2vec bias is not available in this build");
+// ---------------------------------------------------------------- node2vec
+// One workgroup per (walker, step).  Only entry `col` of the step's table is ever read, so the
+// kernel evaluates that entry alone, from the same prefix-sum definition the offline build uses:
+//   pass 1  exact sum of the second-order weights -> ledger, class of entry col
+//           (a light col whose own share accepts the draw needs nothing more)
+//   pass 2  prefix of deficits (or surpluses) up to col
+//   pass 3  first slot whose running prefix crosses it (and the last / next heavy)
+// The result is bit for bit the draw from the fully built table.
+constexpr int N2V_T = 256;
+constexpr uint32_t N2V_CACHE = 4096;  // second-order weights of rows up to this degree stay in LDS between passes
+
+__device__ __forceinline__ bool row_contains(const uint32_t* __restrict__ row, uint32_t n, uint32_t key) {
+  uint32_t lo = 0, len = n;
+  while (len > 0) {
+    const uint32_t half = len >> 1;
+    const uint32_t x = row[lo + half];
+    if (x == key) return true;
+    if (x < key) {
+      lo += half + 1;
+      len -= half + 1;
+    } else {
+      len = half;
+    }
+  }
+  return false;
+}
+
+struct N2vRow {
+  const float* w;
+  const uint32_t* nbr;
+  const uint32_t* prow;
+  uint32_t pdeg, prev;
+  bool has_prev;
+  float p, q;
+  // weight of the edge in slot k after the second-order factor (src/api/bias_node2vec.cu:15-27)
+  __device__ __forceinline__ float operator()(uint32_t k) const {
+    float x = w[k];
+    if (has_prev) {
+      const uint32_t t = nbr[k];
+      if (t == prev) x = __fdiv_rn(x, p);
+      else if (!row_contains(prow, pdeg, t)) x = __fdiv_rn(x, q);
+    }
+    return clamp_weight(x);
+  }
+};
+
+template <class T>
+__device__ __forceinline__ T block_bcast_min(T v, T* s_tmp) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const T o = (T)shfl_xor_u64((uint64_t)v, m);
+    v = o < v ? o : v;
+  }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = v;
+  __syncthreads();
+  T r = s_tmp[0];
+  for (int i = 1; i < N2V_T / 64; ++i) r = s_tmp[i] < r ? s_tmp[i] : r;
+  return r;
+}
+__device__ __forceinline__ uint64_t block_bcast_sum(uint64_t v, uint64_t* s_tmp) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_u64(v, m);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = v;
+  __syncthreads();
+  uint64_t r = 0;
+  for (int i = 0; i < N2V_T / 64; ++i) r += s_tmp[i];
+  return r;
+}
+
+__global__ __launch_bounds__(N2V_T) void n2v_step_kernel(const uint32_t* __restrict__ xadj,
+                                                         const uint32_t* __restrict__ adjncy,
+                                                         const float* __restrict__ wgt, uint32_t len, uint32_t s,
+                                                         float p, float q, float stop_prob, uint64_t seed,
+                                                         uint32_t* __restrict__ paths,
+                                                         uint32_t* __restrict__ lengths) {
+  __shared__ float s_w[N2V_CACHE];
+  __shared__ uint64_t s_tmp[N2V_T / 64];
+  __shared__ u128 s_sum[N2V_T / 64];
+  const uint32_t i = blockIdx.x;
+  const int tid = threadIdx.x;
+  if (lengths[i] != len) return;  // stopped at an earlier step
+  const u32x4 r = philox(seed, i, s, 0, DOM_WALK);
+  uint32_t* path = paths + (size_t)i * (len + 1);
+  const uint32_t v = path[s];
+  const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+  if ((stop_prob > 0.0f && u24(r.z) < stop_prob) || d == 0) {
+    if (tid == 0) lengths[i] = s;
+    return;
+  }
+  N2vRow row;
+  row.w = wgt + off;
+  row.nbr = adjncy + off;
+  row.has_prev = s > 0;
+  row.prev = s > 0 ? path[s - 1] : 0;
+  row.prow = adjncy + xadj[row.prev];
+  row.pdeg = xadj[row.prev + 1] - xadj[row.prev];
+  row.p = p;
+  row.q = q;
+  const bool cached = d <= N2V_CACHE;
+  auto weight = [&](uint32_t k) -> float { return cached ? s_w[k] : row(k); };
+
+  // pass 1: exact total
+  u128 sum{0, 0};
+  for (uint32_t k = tid; k < d; k += N2V_T) {
+    const float x = row(k);
+    if (cached) s_w[k] = x;
+    sum = add128(sum, weight_fixed(x));
+  }
+  sum = group_sum_u128<64>(sum);
+  if ((tid & 63) == 0) s_sum[tid >> 6] = sum;
+  __syncthreads();
+  sum = s_sum[0];
+  for (int k = 1; k < N2V_T / 64; ++k) sum = add128(sum, s_sum[k]);
+  if ((sum.lo | sum.hi) == 0) {
+    if (tid == 0) lengths[i] = s;
+    return;
+  }
+  const Ledger L = make_ledger(d, sum);
+  const uint32_t col = __umulhi(r.x, d);
+  const float u = u24(r.y);
+  const Entry ec = classify(weight(col), L);
+  if (!ec.heavy && u < (float)ec.p) {  // the light keeps the draw: its alias is never read
+    if (tid == 0) path[s + 1] = row.nbr[col];
+    return;
+  }
+
+  // pass 2: prefix up to col of the amounts of col's own kind (exclusive for a light, inclusive for a heavy)
+  uint64_t part = 0;
+  const uint32_t upto = ec.heavy ? col + 1 : col;
+  for (uint32_t k = tid; k < upto; k += N2V_T) {
+    const Entry e = classify(weight(k), L);
+    if (e.heavy == ec.heavy) part += e.amount;
+  }
+  const uint64_t key = block_bcast_sum(part, s_tmp);  // x of a light, y of a heavy
+
+  // pass 3: running prefix of the other kind until it crosses the key
+  uint32_t cand;
+  if (!ec.heavy) {
+    // first heavy m with SH(m) > x; the last heavy if none; col itself if the row has no heavy
+    uint64_t carry = 0;
+    uint32_t found = 0xFFFFFFFFu, last_heavy = 0xFFFFFFFFu;
+    for (uint32_t base = 0; base < d && found == 0xFFFFFFFFu; base += N2V_T) {
+      const uint32_t k = base + tid;
+      uint64_t amt = 0;
+      bool heavy = false;
+      if (k < d) {
+        const Entry e = classify(weight(k), L);
+        heavy = e.heavy;
+        amt = heavy ? e.amount : 0;
+      }
+      const uint64_t inc = group_scan_u64<64>(amt);
+      __syncthreads();
+      if ((tid & 63) == 63) s_tmp[tid >> 6] = inc;
+      __syncthreads();
+      uint64_t before = carry, total = 0;
+      for (int wv = 0; wv < N2V_T / 64; ++wv) {
+        if (wv == (tid >> 6)) before += total;
+        total += s_tmp[wv];
+      }
+      const uint32_t hit = (heavy && before + inc > key) ? k : 0xFFFFFFFFu;
+      const uint32_t lh = heavy ? ~k : 0xFFFFFFFFu;  // min of ~k = max of k
+      found = block_bcast_min<uint32_t>(hit, reinterpret_cast<uint32_t*>(s_tmp));
+      const uint32_t lhm = block_bcast_min<uint32_t>(lh, reinterpret_cast<uint32_t*>(s_tmp));
+      if (lhm != 0xFFFFFFFFu) last_heavy = ~lhm;
+      carry += total;
+    }
+    cand = found != 0xFFFFFFFFu ? found : (last_heavy != 0xFFFFFFFFu ? last_heavy : col);
+  } else {
+    // next heavy after col (none: col is the last heavy and keeps the draw), then the first light l
+    // with SL(l) >= y: prob = (one + y - SL(l)) / one
+    uint32_t nxt = 0xFFFFFFFFu;
+    for (uint32_t base = col + 1; base < d && nxt == 0xFFFFFFFFu; base += N2V_T) {
+      const uint32_t k = base + tid;
+      uint32_t hit = 0xFFFFFFFFu;
+      if (k < d && classify(weight(k), L).heavy) hit = k;
+      nxt = block_bcast_min<uint32_t>(hit, reinterpret_cast<uint32_t*>(s_tmp));
+    }
+    cand = col;
+    if (nxt != 0xFFFFFFFFu) {
+      uint64_t carry = 0, best = ~0ull;  // best = (index << 0) encoded below
+      uint32_t li = 0xFFFFFFFFu;
+      uint64_t sl_at = 0;
+      for (uint32_t base = 0; base < d && li == 0xFFFFFFFFu; base += N2V_T) {
+        const uint32_t k = base + tid;
+        uint64_t amt = 0;
+        bool light = false;
+        if (k < d) {
+          const Entry e = classify(weight(k), L);
+          light = !e.heavy;
+          amt = light ? e.amount : 0;
+        }
+        const uint64_t inc = group_scan_u64<64>(amt);
+        __syncthreads();
+        if ((tid & 63) == 63) s_tmp[tid >> 6] = inc;
+        __syncthreads();
+        uint64_t before = carry, total = 0;
+        for (int wv = 0; wv < N2V_T / 64; ++wv) {
+          if (wv == (tid >> 6)) before += total;
+          total += s_tmp[wv];
+        }
+        const uint64_t mine = before + inc;
+        const uint32_t hit = (light && mine >= key) ? k : 0xFFFFFFFFu;
+        li = block_bcast_min<uint32_t>(hit, reinterpret_cast<uint32_t*>(s_tmp));
+        if (li != 0xFFFFFFFFu) {
+          // the owner of slot li publishes its prefix
+          __syncthreads();
+          if (k == li) s_tmp[0] = mine;
+          __syncthreads();
+          sl_at = s_tmp[0];
+        }
+        carry += total;
+      }
+      (void)best;
+      if (li != 0xFFFFFFFFu) {
+        const float pr = residual_prob(L.one + key - sl_at, L);
+        cand = u < pr ? col : nxt;
+      }
+    }
+  }
+  if (tid == 0) path[s + 1] = row.nbr[cand];
+}
+
+int walk_online_node2vec(sky_graph* g, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
+                         float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
+                         double* seconds) {
+  hipStream_t st = g->stream;
+  unsigned long long* d_sampled = nullptr;
+  auto body = [&]() -> int {
+    SKY_HIP(hipMalloc((void**)&d_sampled, 8));
+    SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
+    EventTimer tm(st);
+    SKY_TRY(tm.mark("start", 0));
+    if (N) {
+      const uint32_t blocks = (N + 255) / 256;
+      hipLaunchKernelGGL(walk_init_kernel, dim3(blocks), dim3(256), 0, st, seeds, N, len, paths, lengths);
+      for (uint32_t s = 0; s < len; ++s)
+        hipLaunchKernelGGL(n2v_step_kernel, dim3(N), dim3(N2V_T), 0, st, g->xadj, g->adjncy, g->adjwgt, len, s, p, q,
+                           stop_prob, seed, paths, lengths);
+      hipLaunchKernelGGL(sum_lengths_kernel, dim3(std::min<uint32_t>(blocks, 1024)), dim3(256), 0, st, lengths, N,
+                         d_sampled);
+    }
+    SKY_TRY(tm.mark("walk", 0));
+    SKY_TRY(tm.finish(nullptr, seconds));
+    unsigned long long h = 0;
+    SKY_HIP(hipMemcpy(&h, d_sampled, 8, hipMemcpyDeviceToHost));
+    if (sampled) *sampled = h;
+    return SKY_OK;
+  };
+  const int rc = body();
+  if (d_sampled) (void)hipFree(d_sampled);
+  return rc;
 }
 
 }  // namespace sky

@@ -105,3 +105,43 @@ def test_online_static_walk_equals_offline_and_oracle(orc):
     assert np.array_equal(on[0], off[0]) and np.array_equal(on[1], off[1]) and s_on == s_off
     opaths, olengths, osampled = orc.walk_online(xadj, adjncy, w, 0, 1.0, 1.0, seeds, 30, 0.1, 5)
     assert np.array_equal(on[0], opaths) and np.array_equal(on[1], olengths) and s_on == osampled
+
+
+@pytest.mark.parametrize("scale,ef,stop", [(11, 8, 0.0), (13, 16, 0.05)])
+def test_node2vec_bit_exact(orc, scale, ef, stop):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(scale, ef, 31)
+    w = orc.gen_weights(orc.W_UNIFORM, 31, len(adjncy), 1.0, 100.0)
+    seeds = orc.gen_seeds(2, 1 << scale, 1500)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    paths, lengths, sampled, _ = g.walk_online(capi.BIAS_NODE2VEC, 2.0, 0.5, seeds, 20, stop, 13)
+    got = (paths.to_host((1500, 21)), lengths.to_host())
+    g.free()
+    opaths, olengths, osampled = orc.walk_online(xadj, adjncy, w, 1, 2.0, 0.5, seeds, 20, stop, 13)
+    assert np.array_equal(got[1], olengths)
+    assert np.array_equal(got[0], opaths)
+    assert sampled == osampled
+
+
+def test_node2vec_hub_rows_beyond_the_weight_cache(orc):
+    # a hub of degree 6000 (more than the kernel keeps in LDS) reached from and returning to small rows
+    from skywalker_amd import capi
+    rng = np.random.default_rng(12)
+    V = 6001
+    hub = np.arange(1, V, dtype=np.uint32)
+    xadj = np.zeros(V + 1, np.uint32)
+    xadj[1] = V - 1
+    spokes = []
+    for v in range(1, V):
+        nb = sorted({0, int(rng.integers(1, V)), int(rng.integers(1, V))} - {v})
+        spokes.append(nb)
+        xadj[v + 1] = xadj[v] + len(nb)
+    adjncy = np.concatenate([hub] + [np.array(s, np.uint32) for s in spokes])
+    w = rng.lognormal(0, 1, len(adjncy)).astype(np.float32)
+    seeds = rng.integers(0, V, 600, dtype=np.uint32)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    paths, lengths, sampled, _ = g.walk_online(capi.BIAS_NODE2VEC, 2.0, 0.5, seeds, 12, 0.0, 4)
+    got = (paths.to_host((600, 13)), lengths.to_host())
+    g.free()
+    opaths, olengths, osampled = orc.walk_online(xadj, adjncy, w, 1, 2.0, 0.5, seeds, 12, 0.0, 4)
+    assert np.array_equal(got[0], opaths) and np.array_equal(got[1], olengths) and sampled == osampled
