@@ -1,0 +1,108 @@
+"""Host-side logic of the drop-in surface: the gflags-compatible parser and the Galois .gr reader
+(CPU only), and the `skywalker` command line end to end (GPU)."""
+import os
+import re
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST = os.path.join(ROOT, "skywalker_amd", "host")
+
+
+def write_gr(path, xadj, adjncy, weights_u32=None):
+    """Galois .gr v1: header, V row-end offsets (u64), E destinations (u32), pad, E weights (u32)."""
+    V, E = len(xadj) - 1, len(adjncy)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<4Q", 1, 0 if weights_u32 is None else 4, V, E))
+        f.write(np.asarray(xadj[1:], np.uint64).tobytes())
+        f.write(np.asarray(adjncy, np.uint32).tobytes())
+        if weights_u32 is not None:
+            if E % 2:
+                f.write(b"\0\0\0\0")
+            f.write(np.asarray(weights_u32, np.uint32).tobytes())
+
+
+def run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    return r.returncode, r.stdout, r.stderr
+
+
+def test_flag_forms():
+    tool = os.path.join(HOST, "gr_tool")
+    rc, out, _ = run([tool, "flags", "--input=/x/y.gr", "-n", "40000", "--tp", "0.15", "--ol=1", "--nobias", "-v"])
+    assert rc == 0 and out.strip() == "input=/x/y.gr n=40000 tp=0.15 ol=1 bias=0 v=1"
+    rc, out, _ = run([tool, "flags", "--ol", "--bias=false", "-n=7"])
+    assert rc == 0 and "n=7" in out and "ol=1" in out and "bias=0" in out
+    rc, _, err = run([tool, "flags", "--nosuchflag"])
+    assert rc == 1 and "unknown command line flag" in err
+    rc, _, err = run([tool, "flags", "-n", "abc"])
+    assert rc == 1 and "illegal value" in err
+
+
+@pytest.mark.parametrize("odd", [False, True])
+def test_gr_reader_round_trip(tmp_path, orc, odd):
+    xadj, adjncy = orc.rmat_csr(8, 5, 3)
+    if odd:  # an odd edge count exercises the 4-byte pad in front of the weights
+        adjncy = adjncy[:-1]
+        xadj = np.minimum(xadj, len(adjncy)).astype(np.uint32)
+    w = (np.arange(len(adjncy)) % 97 + 1).astype(np.uint32)
+    p = str(tmp_path / "g.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    rc, out, _ = run([os.path.join(HOST, "gr_tool"), "info", p])
+    assert rc == 0
+    V, E, md, sa, sw = out.split()[-5:]
+    assert int(V) == len(xadj) - 1 and int(E) == len(adjncy)
+    assert int(md) == int(np.diff(xadj.astype(np.int64)).max())
+    assert int(sa) == int(adjncy.astype(np.int64).sum()) and float(sw) == float(w.sum())
+
+
+@pytest.mark.gpu
+def test_cli_offline_deepwalk_matches_oracle(tmp_path, orc):
+    xadj, adjncy = orc.rmat_csr(12, 8, 11)
+    w = (orc.gen_weights(orc.W_UNIFORM, 11, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "rmat12.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--bias=1", "--ol=0", "--input", p, "-n", "600",
+                        "--d", "20", "--printresult", "--seed", "5"])
+    assert rc == 0, err
+    lines = out.splitlines()
+    assert lines[0] == "rmat12.w.gr"
+    prob, alias, valid = orc.alias_build(xadj, w.astype(np.float32))
+    seeds = np.arange(600, dtype=np.uint32)
+    paths, lengths, sampled = orc.walk_offline(xadj, adjncy, prob, alias, seeds, 20, 0.0, 5)
+    for j in range(3):
+        i = lines.index("%drd path len %d " % (j, lengths[j]))
+        got = [int(x) for x in lines[i + 1].split()]
+        assert got == paths[j, :min(lengths[j], 21)].tolist()
+    # last three lines: table ms, sample ms, MSEPS (src/main.cu:406-419)
+    table_ms, sample_ms, mseps = (float(l.strip()) for l in lines[-3:])
+    assert table_ms > 0 and sample_ms > 0
+    assert abs(mseps - sampled / (sample_ms * 1e-3) / 1e6) <= 0.02 * mseps + 0.02
+
+
+@pytest.mark.gpu
+def test_cli_online_sage_and_csv(tmp_path, orc):
+    xadj, adjncy = orc.rmat_csr(11, 8, 2)
+    w = (orc.gen_weights(orc.W_UNIFORM, 2, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "s.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--sage", "--bias=1", "--ol=1", "--input", p, "-n", "300",
+                        "--csv", "--printresult"])
+    assert rc == 0, err
+    data, sl, sampled = orc.sample_online(xadj, adjncy, w.astype(np.float32), np.arange(300, dtype=np.uint32),
+                                          [1, 25, 10], 0)
+    m = re.search(r"0th sample src: (\d+), 1-hop len: (\d+)", out)
+    assert m and int(m.group(1)) == 0 and int(m.group(2)) == sl[0, 0]
+    hop1 = [int(x) for x in out.split("1-hop : ")[1].splitlines()[0].split()]
+    assert hop1 == data[0, 1:1 + sl[0, 0]].tolist()
+    last = out.strip().splitlines()[-1]
+    assert last.startswith("s.w.gr,") or re.match(r"^[\d.]+,\t[\d.]+,$", last)
+
+
+@pytest.mark.gpu
+def test_cli_rejects_multi_gpu(tmp_path):
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--ngpu", "2", "--input", "/nonexistent"])
+    assert rc == 1 and "one GPU" in err
