@@ -23,7 +23,7 @@ EXPORTS = [
     "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
     "sky_alias_build_all", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
     "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_philox_selftest",
-    "sky_last_build_profile",
+    "sky_last_build_profile", "sky_set_option",
 ]
 
 
@@ -235,6 +235,10 @@ class Graph:
             self.free()
         except Exception:
             pass
+
+
+def set_option(name, value):
+    _ck(lib().sky_set_option(name.encode(), C.c_long(value)))
 
 
 def philox_selftest(ctr, key):

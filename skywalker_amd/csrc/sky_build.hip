@@ -44,21 +44,6 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   return CLS_HUGE;
 }
 
-// first m in [lo, n) with a[m] > key, else n
-__device__ __forceinline__ uint32_t first_greater(const uint64_t* a, uint32_t lo, uint32_t n, uint64_t key) {
-  uint32_t len = n - lo;
-  while (len > 0) {
-    const uint32_t half = len >> 1;
-    if (a[lo + half] <= key) {
-      lo += half + 1;
-      len -= half + 1;
-    } else {
-      len = half;
-    }
-  }
-  return lo;
-}
-
 // ---------------------------------------------------------------- binning
 // `src` lists the vertices to bin (n of them); a null src means vertices 0..n-1.
 __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restrict__ xadj,
@@ -402,7 +387,12 @@ __device__ __forceinline__ u128 block_sum_u128(u128 v, u128* s_tmp) {
   return r;
 }
 
+__device__ __forceinline__ bool streaming_row(uint32_t off, uint32_t d, uint32_t max_tiles) {
+  return ((off & 3u) + d + 4095u) / 4096u > max_tiles;  // rows the tile-parallel path leaves alone
+}
+
 __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+                                                            uint32_t max_tiles,
                                                             const uint64_t* __restrict__ scratch_off,
                                                             const uint32_t* __restrict__ xadj,
                                                             const float* __restrict__ wgt,
@@ -416,6 +406,7 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __re
   for (uint32_t r = blockIdx.x; r < count; r += gridDim.x) {
     const uint32_t v = vlist[r];
     const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+    if (!streaming_row(off, d, max_tiles)) continue;
     const float* wr = wgt + off;
     uint64_t* g_sl = scratch + 2 * scratch_off[r];
     uint64_t* g_sh = g_sl + d;
@@ -496,7 +487,7 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __re
 // Exclusive prefix sum of the degrees of the huge rows (a few thousand at most per launch of
 // 1024 threads; longer lists are walked in chunks by the same block).
 __global__ __launch_bounds__(1024) void huge_prefix_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
-                                                           const uint32_t* __restrict__ xadj,
+                                                           uint32_t max_tiles, const uint32_t* __restrict__ xadj,
                                                            uint64_t* __restrict__ scratch_off,
                                                            uint64_t* __restrict__ total) {
   __shared__ uint64_t s_w[16];
@@ -508,6 +499,7 @@ __global__ __launch_bounds__(1024) void huge_prefix_kernel(const uint32_t* __res
     if (r < count) {
       const uint32_t v = vlist[r];
       d = xadj[v + 1] - xadj[v];
+      if (!streaming_row(xadj[v], (uint32_t)d, max_tiles)) d = 0;
     }
     const uint64_t inc = group_scan_u64<64>(d);
     __syncthreads();
@@ -664,28 +656,33 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
 
   if (counts[CLS_HUGE]) {
     const uint32_t cnt = counts[CLS_HUGE];
-    if (sc.huge_cap < cnt) {
-      if (sc.huge_off) SKY_HIP(hipFree(sc.huge_off));
-      sc.huge_off = nullptr;
-      sc.huge_cap = 0;
-      SKY_HIP(hipMalloc((void**)&sc.huge_off, ((size_t)cnt + 1) * 8));
-      sc.huge_cap = cnt;
+    uint32_t skipped = 0;
+    SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_HUGE], cnt, &skipped));
+    if (skipped) {  // rows with more tiles than the tile-parallel path takes: one workgroup streams each
+      const uint32_t max_tiles = tiled_max_tiles();
+      if (sc.huge_cap < cnt) {
+        if (sc.huge_off) SKY_HIP(hipFree(sc.huge_off));
+        sc.huge_off = nullptr;
+        sc.huge_cap = 0;
+        SKY_HIP(hipMalloc((void**)&sc.huge_off, ((size_t)cnt + 1) * 8));
+        sc.huge_cap = cnt;
+      }
+      hipLaunchKernelGGL(huge_prefix_kernel, dim3(1), dim3(1024), 0, st, vlist + starts[CLS_HUGE], cnt, max_tiles,
+                         g->xadj, sc.huge_off, sc.huge_off + cnt);
+      uint64_t total = 0;
+      SKY_HIP(hipMemcpyAsync(&total, sc.huge_off + cnt, 8, hipMemcpyDeviceToHost, st));
+      SKY_HIP(hipStreamSynchronize(st));
+      if (sc.huge_scratch_cap < total) {
+        if (sc.huge_scratch) SKY_HIP(hipFree(sc.huge_scratch));
+        sc.huge_scratch = nullptr;
+        sc.huge_scratch_cap = 0;
+        SKY_HIP(hipMalloc((void**)&sc.huge_scratch, total * 16));
+        sc.huge_scratch_cap = total;
+      }
+      hipLaunchKernelGGL(build_huge_kernel, dim3(std::min<uint32_t>(cnt, 512)), dim3(HUGE_T), 0, st,
+                         vlist + starts[CLS_HUGE], cnt, max_tiles, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch,
+                         g->prob, g->alias, g->valid);
     }
-    hipLaunchKernelGGL(huge_prefix_kernel, dim3(1), dim3(1024), 0, st, sc.vlist + starts[CLS_HUGE], cnt, g->xadj,
-                       sc.huge_off, sc.huge_off + cnt);
-    uint64_t total = 0;
-    SKY_HIP(hipMemcpyAsync(&total, sc.huge_off + cnt, 8, hipMemcpyDeviceToHost, st));
-    SKY_HIP(hipStreamSynchronize(st));
-    if (sc.huge_scratch_cap < total) {
-      if (sc.huge_scratch) SKY_HIP(hipFree(sc.huge_scratch));
-      sc.huge_scratch = nullptr;
-      sc.huge_scratch_cap = 0;
-      SKY_HIP(hipMalloc((void**)&sc.huge_scratch, total * 16));
-      sc.huge_scratch_cap = total;
-    }
-    hipLaunchKernelGGL(build_huge_kernel, dim3(std::min<uint32_t>(cnt, 512)), dim3(HUGE_T), 0, st,
-                       sc.vlist + starts[CLS_HUGE], cnt, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch, g->prob,
-                       g->alias, g->valid);
   }
   if (tm) SKY_TRY(tm->mark("huge", host.edges[CLS_HUGE]));
   return SKY_OK;

@@ -1,0 +1,677 @@
+// Alias tables of rows too long for one workgroup's LDS, built tile by tile by the whole GPU.
+//
+// A row is cut into tiles of 4096 slots counted from its 16-byte aligned start.  The table is the
+// same pure function of the weights as everywhere else (see sky_build.hip); only the evaluation
+// order changes:
+//   tiled_sum_kernel      per tile   exact 128-bit partial sum of the weights
+//   tiled_ledger_kernel   per row    total -> scale and fraction bits
+//   tiled_totals_kernel   per tile   sum of deficits, sum of surpluses, first and last heavy
+//   tiled_scan_kernel     per row    exclusive prefix of the tile totals (BL, BH), next heavy after each tile
+//   tiled_emit_kernel     per tile   every entry of the tile
+// In the last step a light with exclusive deficit prefix x needs the first slot whose surplus prefix
+// exceeds x.  The tile holding that slot ("partner") follows from BH; its per-slot prefix is
+// recomputed from the weights into LDS and searched there.  Heavies look up their retiring
+// light the same way against BL.  Lights and heavies of a tile are monotone in their keys, so the
+// partners of one tile are a contiguous run and the total number of (tile, partner) pairs of a row
+// is at most twice its tile count: no per-slot scratch in global memory, O(1) passes over the weights.
+#include <algorithm>
+
+#include "sky_graph.h"
+
+namespace sky {
+
+constexpr int TL_T = 256;                // threads per tile
+constexpr int TL_Q = 4;                  // float4 quads per thread
+constexpr int TILE = TL_T * 4 * TL_Q;    // 4096 slots
+constexpr uint32_t NONE32 = 0xFFFFFFFFu;
+constexpr uint32_t TILED_MAX_TILES = 2047;  // tile prefixes of one row must fit the emit kernel's LDS
+
+struct TiledRow {
+  uint32_t v, off, d, base, lead, span, ntiles, tile0;  // tile0: first global tile id; prefix arrays start at tile0 + row
+  double scale, fs, inv_fs;
+  uint64_t one, total_h;
+  uint32_t ok, last_heavy;  // last_heavy: span index
+};
+struct TileTotals {
+  uint64_t d, u;
+  uint32_t first_heavy, last_heavy;  // span indices, NONE32 when the tile has no heavy
+};
+
+__device__ __forceinline__ Ledger row_ledger(const TiledRow& r) {
+  Ledger L;
+  L.scale = r.scale;
+  L.fs = r.fs;
+  L.inv_fs = r.inv_fs;
+  L.one = r.one;
+  return L;
+}
+
+// Weights of tile `t` of a row: quad q of thread tid covers span slots 4*(q*TL_T + tid) + t*TILE ...+3.
+__device__ __forceinline__ void load_tile(const float* __restrict__ wgt, const TiledRow& r, uint32_t t, int tid,
+                                          float (&w)[TL_Q][4]) {
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q) {
+    const uint32_t pos = t * TILE + 4u * (q * TL_T + tid);
+    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pos < r.span) x = *reinterpret_cast<const float4*>(wgt + r.base + pos);
+    const float xs[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = pos + k;
+      w[q][k] = (idx >= r.lead && idx < r.span) ? clamp_weight(xs[k]) : 0.0f;
+    }
+  }
+}
+__device__ __forceinline__ bool in_row(const TiledRow& r, uint32_t idx) { return idx >= r.lead && idx < r.span; }
+
+// ---------------------------------------------------------------- row and tile bookkeeping
+// One block: geometry of every row and the exclusive prefix of the tile counts.  Rows with more
+// than TILED_MAX_TILES tiles get no tiles here (they are left to the streaming kernel).
+__global__ __launch_bounds__(1024) void tiled_rows_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+                                                          const uint32_t* __restrict__ xadj, uint32_t max_tiles,
+                                                          TiledRow* __restrict__ rows,
+                                                          uint32_t* __restrict__ totals /* [0] tiles, [1] skipped rows */) {
+  __shared__ uint32_t s_w[16];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  uint32_t carry = 0, skipped = 0;
+  for (uint32_t chunk = 0; chunk < count; chunk += 1024) {
+    const uint32_t r = chunk + tid;
+    TiledRow row = {};
+    uint32_t nt = 0;
+    if (r < count) {
+      row.v = vlist[r];
+      row.off = xadj[row.v];
+      row.d = xadj[row.v + 1] - row.off;
+      row.base = row.off & ~3u;
+      row.lead = row.off - row.base;
+      row.span = row.lead + row.d;
+      nt = (row.span + TILE - 1) / TILE;
+      if (nt > max_tiles) {
+        nt = 0;
+        ++skipped;
+      }
+      row.ntiles = nt;
+    }
+    const uint32_t inc = group_scan_u32<64>(nt);
+    __syncthreads();
+    if (lane == 63) s_w[wave] = inc;
+    __syncthreads();
+    uint32_t b = carry, t = 0;
+    for (int k = 0; k < 16; ++k) {
+      if (k == wave) b += t;
+      t += s_w[k];
+    }
+    if (r < count) {
+      row.tile0 = b + inc - nt;
+      rows[r] = row;
+    }
+    carry += t;
+  }
+  // skipped rows: sum over the block
+  for (int m = 32; m >= 1; m >>= 1) skipped += __shfl_xor((int)skipped, m, 64);
+  __syncthreads();
+  if (lane == 0) s_w[wave] = skipped;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t s = 0;
+    for (int k = 0; k < 16; ++k) s += s_w[k];
+    totals[0] = carry;
+    totals[1] = s;
+  }
+}
+
+__global__ __launch_bounds__(256) void tiled_map_kernel(const TiledRow* __restrict__ rows, uint32_t count,
+                                                        uint32_t* __restrict__ tile2row) {
+  const uint32_t r = blockIdx.x;
+  if (r >= count) return;
+  const uint32_t t0 = rows[r].tile0, nt = rows[r].ntiles;
+  for (uint32_t t = threadIdx.x; t < nt; t += 256) tile2row[t0 + t] = r;
+}
+
+// ---------------------------------------------------------------- pass 1: exact sums
+__global__ __launch_bounds__(TL_T) void tiled_sum_kernel(const uint32_t* __restrict__ tile2row,
+                                                         const TiledRow* __restrict__ rows,
+                                                         const float* __restrict__ wgt, u128* __restrict__ tsum) {
+  __shared__ u128 s_w[TL_T / 64];
+  const uint32_t tile = blockIdx.x;
+  const TiledRow r = rows[tile2row[tile]];
+  const int tid = threadIdx.x;
+  float w[TL_Q][4];
+  load_tile(wgt, r, tile - r.tile0, tid, w);
+  u128 sum{0, 0};
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) sum = add128(sum, weight_fixed(w[q][k]));
+  sum = group_sum_u128<64>(sum);
+  if ((tid & 63) == 0) s_w[tid >> 6] = sum;
+  __syncthreads();
+  if (tid == 0) {
+    u128 s = s_w[0];
+    for (int i = 1; i < TL_T / 64; ++i) s = add128(s, s_w[i]);
+    tsum[tile] = s;
+  }
+}
+
+__global__ __launch_bounds__(64) void tiled_ledger_kernel(TiledRow* __restrict__ rows, uint32_t count,
+                                                          const u128* __restrict__ tsum) {
+  const uint32_t r = blockIdx.x;
+  if (r >= count) return;
+  const uint32_t t0 = rows[r].tile0, nt = rows[r].ntiles, d = rows[r].d;
+  if (nt == 0) return;
+  u128 sum{0, 0};
+  for (uint32_t t = threadIdx.x; t < nt; t += 64) sum = add128(sum, tsum[t0 + t]);
+  sum = group_sum_u128<64>(sum);
+  if (threadIdx.x == 0) {
+    const bool ok = (sum.lo | sum.hi) != 0;
+    rows[r].ok = ok;
+    if (ok) {
+      const Ledger L = make_ledger(d, sum);
+      rows[r].scale = L.scale;
+      rows[r].fs = L.fs;
+      rows[r].inv_fs = L.inv_fs;
+      rows[r].one = L.one;
+    }
+  }
+}
+
+// ---------------------------------------------------------------- pass 2: tile totals
+__global__ __launch_bounds__(TL_T) void tiled_totals_kernel(const uint32_t* __restrict__ tile2row,
+                                                            const TiledRow* __restrict__ rows,
+                                                            const float* __restrict__ wgt,
+                                                            TileTotals* __restrict__ ttot) {
+  __shared__ uint64_t s_d[TL_T / 64], s_u[TL_T / 64];
+  __shared__ uint32_t s_f[TL_T / 64], s_l[TL_T / 64];
+  const uint32_t tile = blockIdx.x;
+  const TiledRow r = rows[tile2row[tile]];
+  const int tid = threadIdx.x;
+  if (!r.ok) return;
+  const Ledger L = row_ledger(r);
+  const uint32_t t = tile - r.tile0;
+  float w[TL_Q][4];
+  load_tile(wgt, r, t, tid, w);
+  uint64_t sd = 0, su = 0;
+  uint32_t fh = NONE32, lh = 0;  // lh holds idx + 1 so that 0 means none
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = t * TILE + 4u * (q * TL_T + tid) + k;
+      if (!in_row(r, idx)) continue;
+      const Entry e = classify(w[q][k], L);
+      if (e.heavy) {
+        su += e.amount;
+        fh = min(fh, idx);
+        lh = max(lh, idx + 1);
+      } else {
+        sd += e.amount;
+      }
+    }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    sd += shfl_xor_u64(sd, m);
+    su += shfl_xor_u64(su, m);
+    fh = min(fh, (uint32_t)__shfl_xor((int)fh, m, 64));
+    lh = max(lh, (uint32_t)__shfl_xor((int)lh, m, 64));
+  }
+  if ((tid & 63) == 0) {
+    s_d[tid >> 6] = sd;
+    s_u[tid >> 6] = su;
+    s_f[tid >> 6] = fh;
+    s_l[tid >> 6] = lh;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    TileTotals o{0, 0, NONE32, 0};
+    for (int i = 0; i < TL_T / 64; ++i) {
+      o.d += s_d[i];
+      o.u += s_u[i];
+      o.first_heavy = min(o.first_heavy, s_f[i]);
+      o.last_heavy = max(o.last_heavy, s_l[i]);
+    }
+    o.last_heavy = o.last_heavy ? o.last_heavy - 1 : NONE32;
+    ttot[tile] = o;
+  }
+}
+
+// Per row: BL[t], BH[t] = deficits / surpluses before tile t (t = 0..ntiles, the last entry is the
+// row total), stored at index tile0 + row + t; nfh[tile] = first heavy in any later tile.
+__global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ rows, uint32_t count,
+                                                        const TileTotals* __restrict__ ttot,
+                                                        uint64_t* __restrict__ BL, uint64_t* __restrict__ BH,
+                                                        uint32_t* __restrict__ nfh) {
+  const uint32_t r = blockIdx.x;
+  if (r >= count) return;
+  const uint32_t t0 = rows[r].tile0, nt = rows[r].ntiles;
+  if (nt == 0 || !rows[r].ok) return;
+  const int lane = threadIdx.x;
+  const uint32_t b0 = t0 + r;
+  uint64_t cl = 0, ch = 0;
+  uint32_t last = NONE32;
+  for (uint32_t c = 0; c < nt; c += 64) {
+    const uint32_t t = c + lane;
+    uint64_t d = 0, u = 0;
+    uint32_t lh = 0;
+    if (t < nt) {
+      const TileTotals x = ttot[t0 + t];
+      d = x.d;
+      u = x.u;
+      lh = x.last_heavy == NONE32 ? 0 : x.last_heavy + 1;
+    }
+    const uint64_t il = group_scan_u64<64>(d), ih = group_scan_u64<64>(u);
+    if (t < nt) {
+      BL[b0 + t] = cl + il - d;
+      BH[b0 + t] = ch + ih - u;
+    }
+    cl += shfl_u64(il, 63);
+    ch += shfl_u64(ih, 63);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) lh = max(lh, (uint32_t)__shfl_xor((int)lh, m, 64));
+    if (lh) last = lh - 1;
+  }
+  // next first heavy: walk the tiles backwards
+  uint32_t carry = NONE32;
+  for (int32_t c = (int32_t)((nt - 1) / 64 * 64); c >= 0; c -= 64) {
+    const uint32_t t = (uint32_t)c + lane;
+    uint32_t fh = t < nt ? ttot[t0 + t].first_heavy : NONE32;
+    // exclusive suffix minimum over lanes
+    uint32_t suf = fh;
+#pragma unroll
+    for (int dlt = 1; dlt < 64; dlt <<= 1) {
+      const uint32_t o = (uint32_t)__shfl_down((int)suf, dlt, 64);
+      if (lane + dlt < 64) suf = min(suf, o);
+    }
+    uint32_t excl = (uint32_t)__shfl_down((int)suf, 1, 64);
+    if (lane == 63) excl = NONE32;
+    if (t < nt) nfh[t0 + t] = min(excl, carry);
+    carry = min(carry, (uint32_t)__shfl((int)suf, 0, 64));
+  }
+  if (lane == 0) {
+    BL[b0 + nt] = cl;
+    BH[b0 + nt] = ch;
+    rows[r].total_h = ch;
+    rows[r].last_heavy = last;
+  }
+}
+
+// ---------------------------------------------------------------- pass 3: every entry of a tile
+// Inclusive prefix of `val` over the slots of one tile in slot order (quad q of thread tid before quad
+// q of thread tid+1, sub-tile q before q+1), starting from `base`.
+struct TileScan {
+  uint64_t* s_wave;  // [TL_T/64]
+  __device__ __forceinline__ void run(const uint64_t (&val)[TL_Q][4], uint64_t base, uint64_t (&out)[TL_Q][4]) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    uint64_t carry = base;
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q) {
+      uint64_t run = 0, loc[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        run += val[q][k];
+        loc[k] = run;
+      }
+      const uint64_t inc = group_scan_u64<64>(run);
+      __syncthreads();
+      if (lane == 63) s_wave[wave] = inc;
+      __syncthreads();
+      uint64_t before = carry + inc - run, tot = 0;
+#pragma unroll
+      for (int i = 0; i < TL_T / 64; ++i) {
+        if (i == wave) before += tot;
+        tot += s_wave[i];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) out[q][k] = before + loc[k];
+      carry += tot;
+    }
+  }
+};
+
+// first j in [0, TILE) with P[j] > key (TILE if none), four keys at a time
+__device__ __forceinline__ void search4(const uint64_t* __restrict__ P, const uint64_t (&key)[4], uint32_t (&pos)[4]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) pos[k] = 0;
+#pragma unroll
+  for (uint32_t step = TILE / 2; step >= 1; step >>= 1) {
+    uint64_t v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = P[pos[k] + step - 1];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (v[k] <= key[k]) pos[k] += step;
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    if (P[pos[k]] <= key[k]) pos[k] += 1;
+}
+
+// first t in [0, nt) with B[t + 1] > key (nt if none)
+__device__ __forceinline__ uint32_t first_tile_above(const uint64_t* B, uint32_t nt, uint64_t key) {
+  return first_greater(B + 1, 0, nt, key);
+}
+
+__global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __restrict__ tile2row,
+                                                          const TiledRow* __restrict__ rows,
+                                                          const float* __restrict__ wgt,
+                                                          const uint64_t* __restrict__ gBL,
+                                                          const uint64_t* __restrict__ gBH,
+                                                          const uint32_t* __restrict__ nfh, float* __restrict__ prob,
+                                                          uint32_t* __restrict__ alias,
+                                                          int8_t* __restrict__ valid) {
+  extern __shared__ uint64_t smem[];
+  uint64_t* P = smem;                  // [TILE] per-slot prefix of the current partner tile
+  uint64_t* s_BL = smem + TILE;        // [nt + 1]
+  __shared__ uint64_t s_wave[TL_T / 64];
+  __shared__ uint32_t s_first[TL_Q][TL_T / 64];
+  const uint32_t tile = blockIdx.x;
+  const uint32_t ri = tile2row[tile];
+  const TiledRow r = rows[ri];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t T = tile - r.tile0, nt = r.ntiles;
+  uint64_t* s_BH = s_BL + nt + 1;
+
+  float w[TL_Q][4];
+  load_tile(wgt, r, T, tid, w);
+  if (!r.ok) {
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t idx = T * TILE + 4u * (q * TL_T + tid) + k;
+        if (in_row(r, idx)) {
+          prob[r.base + idx] = 0.0f;
+          alias[r.base + idx] = SKY_INVALID;
+        }
+      }
+    if (T == 0 && tid == 0) valid[r.v] = 0;
+    return;
+  }
+  const Ledger L = row_ledger(r);
+  const uint32_t b0 = r.tile0 + ri;
+  for (uint32_t i = tid; i <= nt; i += TL_T) {
+    s_BL[i] = gBL[b0 + i];
+    s_BH[i] = gBH[b0 + i];
+  }
+
+  // own tile: class, amount, prefix of the own kind -> key (x of a light, y of a heavy)
+  uint64_t dl[TL_Q][4], dh[TL_Q][4], key[TL_Q][4];
+  float op[TL_Q][4];
+  uint32_t oa[TL_Q][4];
+  uint32_t heavy_mask = 0, live_mask = 0;
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = T * TILE + 4u * (q * TL_T + tid) + k;
+      const Entry e = classify(w[q][k], L);
+      const bool in = in_row(r, idx);
+      dl[q][k] = (in && !e.heavy) ? e.amount : 0;
+      dh[q][k] = (in && e.heavy) ? e.amount : 0;
+      op[q][k] = e.heavy ? 1.0f : (float)e.p;
+      if (in) live_mask |= 1u << (q * 4 + k);
+      if (in && e.heavy) heavy_mask |= 1u << (q * 4 + k);
+    }
+  __syncthreads();  // s_BL / s_BH are complete
+  TileScan scan{s_wave};
+  {
+    uint64_t sl[TL_Q][4], sh[TL_Q][4];
+    scan.run(dl, s_BL[T], sl);
+    scan.run(dh, s_BH[T], sh);
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) key[q][k] = (heavy_mask >> (q * 4 + k)) & 1 ? sh[q][k] : sl[q][k] - dl[q][k];
+  }
+
+  // next heavy after each own heavy (span index), NONE32 for the last heavy of the row
+  uint32_t nh_after_quad[TL_Q];
+  {
+    uint32_t qfirst[TL_Q];
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q) {
+      const uint32_t m = (heavy_mask >> (q * 4)) & 15u;
+      qfirst[q] = m ? T * TILE + 4u * (q * TL_T + tid) + (uint32_t)(__ffs((int)m) - 1) : NONE32;
+      uint32_t suf = qfirst[q];
+#pragma unroll
+      for (int dlt = 1; dlt < 64; dlt <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_down((int)suf, dlt, 64);
+        if (lane + dlt < 64) suf = min(suf, o);
+      }
+      uint32_t excl = (uint32_t)__shfl_down((int)suf, 1, 64);
+      if (lane == 63) excl = NONE32;
+      nh_after_quad[q] = excl;
+      if (lane == 0) s_first[q][wave] = suf;
+    }
+    __syncthreads();
+    const uint32_t later_tiles = nfh[tile];
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q) {
+      uint32_t m = later_tiles;
+      for (int wv = 0; wv < TL_T / 64; ++wv) {
+        if (wv > wave) m = min(m, s_first[q][wv]);
+#pragma unroll
+        for (int q2 = q + 1; q2 < TL_Q; ++q2) m = min(m, s_first[q2][wv]);
+      }
+      nh_after_quad[q] = min(nh_after_quad[q], m);
+    }
+  }
+  uint32_t nh[TL_Q][4];
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q) {
+    uint32_t nxt = nh_after_quad[q];
+#pragma unroll
+    for (int k = 3; k >= 0; --k) {
+      nh[q][k] = nxt;
+      if ((heavy_mask >> (q * 4 + k)) & 1) nxt = T * TILE + 4u * (q * TL_T + tid) + k;
+    }
+  }
+  // defaults: a light without donor takes the last heavy (itself if the row has none);
+  // a heavy that is last, or that no light retires, keeps {1, itself}
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = T * TILE + 4u * (q * TL_T + tid) + k;
+      const bool heavy = (heavy_mask >> (q * 4 + k)) & 1;
+      oa[q][k] = (!heavy && r.total_h) ? r.last_heavy - r.lead : idx - r.lead;
+    }
+
+  // ---- lights against the surplus prefix of their partner tiles
+  {
+    const uint32_t t_lo = first_tile_above(s_BH, nt, s_BL[T]);
+    const uint32_t t_hi = min(first_tile_above(s_BH, nt, s_BL[T + 1]), nt - 1);
+    for (uint32_t pt = t_lo; pt <= t_hi && pt < nt; ++pt) {
+      const uint64_t lo = s_BH[pt], hi = s_BH[pt + 1];
+      if (hi == lo) continue;
+      float pw[TL_Q][4];
+      load_tile(wgt, r, pt, tid, pw);
+      uint64_t pv[TL_Q][4], ps[TL_Q][4];
+#pragma unroll
+      for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t idx = pt * TILE + 4u * (q * TL_T + tid) + k;
+          const Entry e = classify(pw[q][k], L);
+          pv[q][k] = (in_row(r, idx) && e.heavy) ? e.amount : 0;
+        }
+      scan.run(pv, lo, ps);
+      __syncthreads();  // previous partner's searches are done
+#pragma unroll
+      for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) P[4u * (q * TL_T + tid) + k] = ps[q][k];
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < TL_Q; ++q) {
+        bool mine[4], any = false;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int b = q * 4 + k;
+          mine[k] = ((live_mask >> b) & 1) && !((heavy_mask >> b) & 1) && key[q][k] >= lo && key[q][k] < hi;
+          any |= mine[k];
+        }
+        if (!any) continue;
+        uint32_t pos[4];
+        search4(P, key[q], pos);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (mine[k]) oa[q][k] = pt * TILE + pos[k] - r.lead;
+      }
+    }
+  }
+  // ---- heavies against the deficit prefix of their partner tiles
+  {
+    const uint32_t t_lo = first_tile_above(s_BL, nt, s_BH[T]);  // first t with BL[t+1] >= BH[T] + 1
+    const uint32_t t_hi = min(s_BH[T + 1] ? first_tile_above(s_BL, nt, s_BH[T + 1] - 1) : 0u, nt - 1);
+    const bool any_heavy = s_BH[T + 1] != s_BH[T];
+    for (uint32_t pt = t_lo; any_heavy && pt <= t_hi && pt < nt; ++pt) {
+      const uint64_t lo = s_BL[pt], hi = s_BL[pt + 1];
+      if (hi == lo) continue;
+      float pw[TL_Q][4];
+      load_tile(wgt, r, pt, tid, pw);
+      uint64_t pv[TL_Q][4], ps[TL_Q][4];
+#pragma unroll
+      for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t idx = pt * TILE + 4u * (q * TL_T + tid) + k;
+          const Entry e = classify(pw[q][k], L);
+          pv[q][k] = (in_row(r, idx) && !e.heavy) ? e.amount : 0;
+        }
+      scan.run(pv, lo, ps);
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) P[4u * (q * TL_T + tid) + k] = ps[q][k];
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < TL_Q; ++q) {
+        bool mine[4], any = false;
+        uint64_t km1[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int b = q * 4 + k;
+          // a heavy retires in this partner iff lo < y <= hi; the last heavy of the row never retires
+          mine[k] = ((heavy_mask >> b) & 1) && nh[q][k] != NONE32 && key[q][k] > lo && key[q][k] <= hi;
+          km1[k] = key[q][k] - 1;
+          any |= mine[k];
+        }
+        if (!any) continue;
+        uint32_t pos[4];
+        search4(P, km1, pos);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (mine[k]) {
+            op[q][k] = residual_prob(L.one + key[q][k] - P[pos[k]], L);
+            oa[q][k] = nh[q][k] - r.lead;
+          }
+      }
+    }
+  }
+  // ---- store
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q) {
+    const uint32_t pos = T * TILE + 4u * (q * TL_T + tid);
+    if (pos >= r.span) continue;
+    if (pos >= r.lead && pos + 4 <= r.span) {
+      *reinterpret_cast<float4*>(prob + r.base + pos) = make_float4(op[q][0], op[q][1], op[q][2], op[q][3]);
+      *reinterpret_cast<uint4*>(alias + r.base + pos) = make_uint4(oa[q][0], oa[q][1], oa[q][2], oa[q][3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (in_row(r, pos + k)) {
+          prob[r.base + pos + k] = op[q][k];
+          alias[r.base + pos + k] = oa[q][k];
+        }
+    }
+  }
+  if (T == 0 && tid == 0) valid[r.v] = 1;
+}
+
+// ---------------------------------------------------------------- host driver
+namespace {
+struct TiledScratch {
+  TiledRow* rows = nullptr;
+  uint32_t* totals = nullptr;  // [2]
+  uint32_t* tile2row = nullptr;
+  u128* tsum = nullptr;
+  TileTotals* ttot = nullptr;
+  uint64_t *BL = nullptr, *BH = nullptr;
+  uint32_t* nfh = nullptr;
+  uint32_t row_cap = 0, tile_cap = 0;
+  bool lds_enabled = false;
+};
+TiledScratch g_tiled;
+uint32_t g_tiled_max_tiles = TILED_MAX_TILES;
+}  // namespace
+
+uint32_t tiled_max_tiles() { return g_tiled_max_tiles; }
+void set_tiled_max_tiles(uint32_t n) { g_tiled_max_tiles = std::min<uint32_t>(std::max<uint32_t>(n, 1), TILED_MAX_TILES); }
+
+// Builds the rows of `rows_list` (device, n entries) that have at most the configured number of
+// tiles; *skipped receives how many rows were left for the streaming kernel.
+int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped) {
+  hipStream_t st = g->stream;
+  TiledScratch& sc = g_tiled;
+  *skipped = 0;
+  if (n == 0) return SKY_OK;
+  if (sc.row_cap < n) {
+    if (sc.rows) SKY_HIP(hipFree(sc.rows));
+    sc.rows = nullptr;
+    sc.row_cap = 0;
+    SKY_HIP(hipMalloc((void**)&sc.rows, (size_t)n * sizeof(TiledRow)));
+    sc.row_cap = n;
+  }
+  if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, 8));
+  if (!sc.lds_enabled) {
+    SKY_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_emit_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)((TILE + 2 * (TILED_MAX_TILES + 1)) * 8)));
+    sc.lds_enabled = true;
+  }
+  hipLaunchKernelGGL(tiled_rows_kernel, dim3(1), dim3(1024), 0, st, rows_list, n, g->xadj, g_tiled_max_tiles, sc.rows,
+                     sc.totals);
+  uint32_t totals[2] = {0, 0};
+  SKY_HIP(hipMemcpyAsync(totals, sc.totals, 8, hipMemcpyDeviceToHost, st));
+  SKY_HIP(hipStreamSynchronize(st));
+  const uint32_t ntiles = totals[0];
+  *skipped = totals[1];
+  if (ntiles == 0) return SKY_OK;
+  if (sc.tile_cap < ntiles) {
+    void* olds[] = {sc.tile2row, sc.tsum, sc.ttot, sc.BL, sc.BH, sc.nfh};
+    for (void* p : olds)
+      if (p) SKY_HIP(hipFree(p));
+    sc.tile2row = nullptr; sc.tsum = nullptr; sc.ttot = nullptr; sc.BL = nullptr; sc.BH = nullptr; sc.nfh = nullptr;
+    sc.tile_cap = 0;
+    const size_t cap = (size_t)ntiles + ntiles / 4 + 1024;
+    SKY_HIP(hipMalloc((void**)&sc.tile2row, cap * 4));
+    SKY_HIP(hipMalloc((void**)&sc.tsum, cap * sizeof(u128)));
+    SKY_HIP(hipMalloc((void**)&sc.ttot, cap * sizeof(TileTotals)));
+    SKY_HIP(hipMalloc((void**)&sc.nfh, cap * 4));
+    sc.tile_cap = (uint32_t)cap;
+  }
+  // prefix arrays hold ntiles + one extra entry per row
+  static size_t b_cap = 0;
+  const size_t b_need = (size_t)ntiles + n;
+  if (b_cap < b_need) {
+    if (sc.BL) SKY_HIP(hipFree(sc.BL));
+    if (sc.BH) SKY_HIP(hipFree(sc.BH));
+    sc.BL = sc.BH = nullptr;
+    b_cap = 0;
+    SKY_HIP(hipMalloc((void**)&sc.BL, (b_need + b_need / 4 + 1024) * 8));
+    SKY_HIP(hipMalloc((void**)&sc.BH, (b_need + b_need / 4 + 1024) * 8));
+    b_cap = b_need + b_need / 4 + 1024;
+  }
+  hipLaunchKernelGGL(tiled_map_kernel, dim3(n), dim3(256), 0, st, sc.rows, n, sc.tile2row);
+  hipLaunchKernelGGL(tiled_sum_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.tsum);
+  hipLaunchKernelGGL(tiled_ledger_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.tsum);
+  hipLaunchKernelGGL(tiled_totals_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.ttot);
+  hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh);
+  const size_t lds = (size_t)(TILE + 2 * (g_tiled_max_tiles + 1)) * 8;
+  hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), lds, st, sc.tile2row, sc.rows, g->adjwgt, sc.BL,
+                     sc.BH, sc.nfh, g->prob, g->alias, g->valid);
+  return SKY_OK;
+}
+
+}  // namespace sky

@@ -286,6 +286,16 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
   return philox_selftest(ctr_host, key_host, n, out_host);
 }
 
+int sky_set_option(const char* name, long value) {
+  if (!name) return fail(SKY_ERR_ARG, "sky_set_option: null name");
+  if (!strcmp(name, "tiled_max_tiles")) {
+    if (value < 1) return fail(SKY_ERR_ARG, "sky_set_option: tiled_max_tiles must be >= 1");
+    set_tiled_max_tiles((uint32_t)value);
+    return SKY_OK;
+  }
+  return fail(SKY_ERR_ARG, std::string("sky_set_option: unknown option ") + name);
+}
+
 int sky_last_build_profile(const sky_graph* g, const char** names, float* ms, uint64_t* edges, int max_entries) {
   if (!g) return 0;
   int n = 0;

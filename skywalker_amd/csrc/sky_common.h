@@ -133,6 +133,21 @@ __device__ __forceinline__ float residual_prob(uint64_t r_units, const Ledger& L
   return (float)((double)r_units * L.inv_fs);
 }
 
+// first m in [lo, n) with a[m] > key, else n
+__device__ __forceinline__ uint32_t first_greater(const uint64_t* a, uint32_t lo, uint32_t n, uint64_t key) {
+  uint32_t len = n - lo;
+  while (len > 0) {
+    const uint32_t half = len >> 1;
+    if (a[lo + half] <= key) {
+      lo += half + 1;
+      len -= half + 1;
+    } else {
+      len = half;
+    }
+  }
+  return lo;
+}
+
 // ---------------------------------------------------------------- wave64 primitives
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 

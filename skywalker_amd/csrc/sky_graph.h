@@ -62,6 +62,10 @@ int ensure_table_storage(sky_graph* g);
 int prepare_build_scratch(uint32_t max_rows);
 int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm);
 int build_all_tables(sky_graph* g, double* seconds);
+// rows of more than 8189 entries: tile-parallel path, and how many tiles per row it accepts
+int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped);
+void set_tiled_max_tiles(uint32_t n);
+uint32_t tiled_max_tiles();
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
                  uint32_t* paths, uint32_t* lengths, uint64_t* sampled, double* seconds);
 int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,

@@ -100,3 +100,30 @@ def test_bad_arguments_are_reported(orc):
     with pytest.raises(capi.SkyError):
         g.walk_offline(np.array([0], np.uint32), 4, 0.0, 1)  # tables not built
     g.free()
+
+
+@pytest.mark.parametrize("dist", ["lognormal2", "nearequal", "sparse", "fewlights", "fewheavies"])
+def test_rows_built_tile_by_tile(orc, dist):
+    # rows beyond one workgroup's LDS: 3 to 80 tiles of 4096, starts of every alignment
+    from helpers import weights
+    rng = np.random.default_rng(21)
+    degs = [8190, 1, 8193, 2, 12288, 3, 12289, 40000, 5, 100001, 330000]
+    xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=4096)
+    if dist == "fewlights":      # almost every entry barely heavy, 1 % very light: a light tile spans many partners
+        w = np.where(rng.random(len(w)) < 0.01, 0.01, 1.01).astype(np.float32)
+    elif dist == "fewheavies":   # 0.1 % of the entries carry almost all the mass
+        w = np.where(rng.random(len(w)) < 0.001, 1000.0, 0.5).astype(np.float32)
+    else:
+        w = weights(len(w), rng, dist)
+    build_and_compare(orc, xadj, adjncy, w, "tiled/" + dist)
+
+
+def test_streaming_kernel_for_rows_with_too_many_tiles(orc):
+    from skywalker_amd import capi
+    rng = np.random.default_rng(22)
+    xadj, adjncy, w = graph_from_degrees([9000, 20000, 3, 70000], rng, "lognormal2", V=4096)
+    capi.set_option("tiled_max_tiles", 3)  # 9000 stays tile-parallel, the other two are streamed
+    try:
+        build_and_compare(orc, xadj, adjncy, w, "streaming")
+    finally:
+        capi.set_option("tiled_max_tiles", 2047)
