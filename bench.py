@@ -140,7 +140,9 @@ def main():
                    "device": name, "compute_units": cus, "graph_generation_s": t_gen},
         "build": {"edges_per_s": E / build_s, "ms": build_s * 1e3, "algorithmic_bytes": build_bytes,
                   "hbm_frac": build_bytes / build_s / HBM_PEAK,
-                  "kernels_ms": {KERNEL_OF.get(k, k): round(v[0], 4) for k, v in prof.items()}},
+                  "kernels": {KERNEL_OF.get(k, k): {"ms": round(v[0], 4), "edges": v[1],
+                                                    "GBps": round(12 * v[1] / (v[0] * 1e-3) / 1e9, 1) if v[0] > 0 else 0}
+                              for k, v in prof.items()}},
         "walk": {"seps": walk_edges / walk_s, "ms": walk_s * 1e3, "steps": walk_edges,
                  "algorithmic_bytes": 24 * walk_edges, "hbm_frac": 24 * walk_edges / walk_s / HBM_PEAK},
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF.get(dom, dom), "achieved": dom_bytes / (dom_ms * 1e-3) / 1e9,

@@ -211,9 +211,84 @@ __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __re
 }
 
 // ---------------------------------------------------------------- one row per workgroup, prefix arrays in LDS
-// ROWT threads cooperate on one row of at most ROWT*4*T slots (counted from the row's
-// 16-byte aligned start).  Weights are read once as aligned float4 quads and stay in
-// registers; SL and SH of every slot live in LDS for the searches.
+// ROWT threads cooperate on one row of at most ROWT*4*T slots (counted from the row's 16-byte
+// aligned start).  Weights are read once as aligned float4 quads; every entry is classified once
+// and keeps its search key in registers; SL and SH of every slot live in LDS.  Each entry then
+// does exactly one binary search, lights in SH and heavies in SL, four searches interleaved; the
+// next heavy after each heavy and the last heavy of the row come from a suffix scan, not a search.
+constexpr uint32_t NONE32 = 0xFFFFFFFFu;
+
+// Inclusive prefixes of two quantities over the slots of a tile held as [Q][4] per thread (slot order:
+// quad q of thread tid, then thread tid + 1; sub-tile q before q + 1).  One barrier.
+template <int ROWT, int Q>
+__device__ __forceinline__ void block_scan2(const uint64_t (&a)[Q][4], const uint64_t (&b)[Q][4],
+                                            uint64_t* __restrict__ s_ex /* [2 * Q * ROWT/64] */,
+                                            uint64_t (&oa)[Q][4], uint64_t (&ob)[Q][4], uint64_t& tot_a,
+                                            uint64_t& tot_b) {
+  constexpr int NW = ROWT / 64;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  uint64_t ia[Q], ib[Q];
+#pragma unroll
+  for (int q = 0; q < Q; ++q) {
+    uint64_t ra = 0, rb = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      ra += a[q][k];
+      rb += b[q][k];
+      oa[q][k] = ra;
+      ob[q][k] = rb;
+    }
+    ia[q] = group_scan_u64<64>(ra);
+    ib[q] = group_scan_u64<64>(rb);
+    if (lane == 63) {
+      s_ex[(q * NW + wave) * 2] = ia[q];
+      s_ex[(q * NW + wave) * 2 + 1] = ib[q];
+    }
+    ia[q] -= ra;  // exclusive over the lanes of this wave
+    ib[q] -= rb;
+  }
+  __syncthreads();
+  uint64_t run_a = 0, run_b = 0;
+#pragma unroll
+  for (int q = 0; q < Q; ++q) {
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      if (w == wave) {
+        ia[q] += run_a;
+        ib[q] += run_b;
+      }
+      run_a += s_ex[(q * NW + w) * 2];
+      run_b += s_ex[(q * NW + w) * 2 + 1];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      oa[q][k] += ia[q];
+      ob[q][k] += ib[q];
+    }
+  }
+  tot_a = run_a;
+  tot_b = run_b;
+}
+
+// For four keys at once: number of leading entries of a_k[0..n) that are <= key_k (n if all are).
+__device__ __forceinline__ void search4(const uint64_t* const (&a)[4], const uint64_t (&key)[4], uint32_t n,
+                                        uint32_t (&pos)[4]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) pos[k] = 0;
+  for (uint32_t step = 1u << (31 - __clz((int)n)); step; step >>= 1) {
+    uint64_t v[4];
+    uint32_t t[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      t[k] = pos[k] + step;
+      v[k] = a[k][min(t[k], n) - 1];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (t[k] <= n && v[k] <= key[k]) pos[k] = t[k];
+  }
+}
+
 template <int ROWT, int T>
 __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restrict__ vlist,
                                                          const uint32_t* __restrict__ xadj,
@@ -225,7 +300,8 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   uint64_t* s_sl = smem;
   uint64_t* s_sh = smem + CAP;
   __shared__ u128 s_wsum[NW];
-  __shared__ uint64_t s_wl[NW], s_wh[NW];
+  __shared__ uint64_t s_ex[2 * T * NW];
+  __shared__ uint32_t s_fh[T][NW], s_lh[T][NW];
 
   const uint32_t v = vlist[blockIdx.x];
   const uint32_t off = xadj[v], d = xadj[v + 1] - off;
@@ -234,6 +310,7 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
 
   float w[T][4];
   u128 sum{0, 0};
+  uint32_t live = 0;  // bit q*4+k: slot belongs to the row
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const uint32_t pos = 4u * (t * ROWT + tid);
@@ -243,7 +320,9 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const uint32_t idx = pos + k;
-      w[t][k] = (idx >= lead && idx < span) ? clamp_weight(xs[k]) : 0.0f;
+      const bool in = idx >= lead && idx < span;
+      if (in) live |= 1u << (t * 4 + k);
+      w[t][k] = in ? clamp_weight(xs[k]) : 0.0f;
       sum = add128(sum, weight_fixed(w[t][k]));
     }
   }
@@ -257,115 +336,130 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   }
   if ((sum.lo | sum.hi) == 0) {
 #pragma unroll
-    for (int t = 0; t < T; ++t) {
-      const uint32_t pos = 4u * (t * ROWT + tid);
+    for (int t = 0; t < T; ++t)
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const uint32_t idx = pos + k;
-        if (idx >= lead && idx < span) {
+      for (int k = 0; k < 4; ++k)
+        if ((live >> (t * 4 + k)) & 1) {
+          const uint32_t idx = 4u * (t * ROWT + tid) + k;
           prob[base + idx] = 0.0f;
           alias[base + idx] = SKY_INVALID;
         }
-      }
-    }
     if (tid == 0) valid[v] = 0;
     return;
   }
   const Ledger L = make_ledger(d, sum);
 
-  uint64_t carry_l = 0, carry_h = 0;
+  // classify once; amounts -> prefix sums; first / last heavy of every (sub-tile, wave)
+  uint64_t dl[T][4], dh[T][4], sl[T][4], sh[T][4];
+  float op[T][4];
+  uint32_t heavy = 0;
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int b = t * 4 + k;
+      const Entry e = classify(w[t][k], L);
+      const bool in = (live >> b) & 1;
+      dl[t][k] = (in && !e.heavy) ? e.amount : 0;
+      dh[t][k] = (in && e.heavy) ? e.amount : 0;
+      op[t][k] = e.heavy ? 1.0f : (float)e.p;
+      if (in && e.heavy) heavy |= 1u << b;
+    }
+    const uint32_t m = (heavy >> (t * 4)) & 15u;
+    const uint32_t q0 = 4u * (t * ROWT + tid);
+    uint32_t fh = m ? q0 + (uint32_t)(__ffs((int)m) - 1) : NONE32;
+    uint32_t lh = m ? q0 + (uint32_t)(31 - __clz((int)m)) + 1 : 0;  // index + 1, 0 = none
+#pragma unroll
+    for (int x = 32; x >= 1; x >>= 1) {
+      fh = min(fh, (uint32_t)__shfl_xor((int)fh, x, 64));
+      lh = max(lh, (uint32_t)__shfl_xor((int)lh, x, 64));
+    }
+    if (lane == 0) {
+      s_fh[t][wave] = fh;
+      s_lh[t][wave] = lh;
+    }
+  }
+  uint64_t total_l, total_h;
+  block_scan2<ROWT, T>(dl, dh, s_ex, sl, sh, total_l, total_h);  // its barrier also publishes s_fh / s_lh
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const uint32_t pos = 4u * (t * ROWT + tid);
-    uint64_t l[4], h[4], rl = 0, rh = 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const uint32_t idx = pos + k;
-      const Entry e = classify(w[t][k], L);
-      const bool in = idx >= lead && idx < span;
-      rl += (in && !e.heavy) ? e.amount : 0;
-      rh += (in && e.heavy) ? e.amount : 0;
-      l[k] = rl;
-      h[k] = rh;
-    }
-    const uint64_t il = group_scan_u64<64>(rl), ih = group_scan_u64<64>(rh);
-    uint64_t base_l = carry_l + il - rl, base_h = carry_h + ih - rh;
-    if (NW > 1) {
-      if (t > 0) __syncthreads();  // previous tile's wave totals have been consumed
-      if (lane == 63) { s_wl[wave] = il; s_wh[wave] = ih; }
-      __syncthreads();
-      uint64_t tl = 0, th = 0;
-#pragma unroll
-      for (int i = 0; i < NW; ++i) {
-        if (i == wave) { base_l += tl; base_h += th; }
-        tl += s_wl[i];
-        th += s_wh[i];
-      }
-      carry_l += tl;
-      carry_h += th;
-    } else {
-      carry_l += shfl_u64(il, 63);
-      carry_h += shfl_u64(ih, 63);
-    }
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      s_sl[pos + k] = base_l + l[k];
-      s_sh[pos + k] = base_h + h[k];
+      s_sl[pos + k] = sl[t][k];
+      s_sh[pos + k] = sh[t][k];
     }
   }
-  __syncthreads();
-  const uint64_t total_h = carry_h;
+  // next heavy after each quad: later lanes of the wave, later waves of the sub-tile, later sub-tiles
+  uint32_t last_heavy = 0;
+  uint32_t nh_after[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const uint32_t m = (heavy >> (t * 4)) & 15u;
+    uint32_t suf = m ? 4u * (t * ROWT + tid) + (uint32_t)(__ffs((int)m) - 1) : NONE32;
+#pragma unroll
+    for (int dlt = 1; dlt < 64; dlt <<= 1) {
+      const uint32_t o = (uint32_t)__shfl_down((int)suf, dlt, 64);
+      if (lane + dlt < 64) suf = min(suf, o);
+    }
+    uint32_t nx = (uint32_t)__shfl_down((int)suf, 1, 64);
+    if (lane == 63) nx = NONE32;
+#pragma unroll
+    for (int wv = 0; wv < NW; ++wv) {
+      if (wv > wave) nx = min(nx, s_fh[t][wv]);
+#pragma unroll
+      for (int t2 = t + 1; t2 < T; ++t2) nx = min(nx, s_fh[t2][wv]);
+      last_heavy = max(last_heavy, s_lh[t][wv]);
+    }
+    nh_after[t] = nx;
+  }
+  __syncthreads();  // s_sl / s_sh are complete
 
+  const uint64_t* a_l = s_sl + lead;
+  const uint64_t* a_h = s_sh + lead;
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const uint32_t pos = 4u * (t * ROWT + tid);
     if (pos >= span) continue;
-    float op[4];
-    uint32_t oa[4];
+    const uint64_t* arr[4];
+    uint64_t key[4];
+    uint32_t nh[4], oa[4], at[4];
+    uint32_t nxt = nh_after[t];
+#pragma unroll
+    for (int k = 3; k >= 0; --k) {
+      nh[k] = nxt;
+      if ((heavy >> (t * 4 + k)) & 1) nxt = pos + k;
+    }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const uint32_t idx = pos + k;
-      op[k] = 0.0f;
-      oa[k] = 0;
-      if (idx < lead || idx >= span) continue;
-      const Entry e = classify(w[t][k], L);
-      const uint32_t self = idx - lead;
-      if (!e.heavy) {
-        const uint64_t x = s_sl[idx] - e.amount;
-        const uint32_t m = first_greater(s_sh, lead, span, x);
-        op[k] = (float)e.p;
-        if (m < span) {
-          oa[k] = m - lead;
-        } else if (total_h) {
-          oa[k] = first_greater(s_sh, lead, span, total_h - 1) - lead;  // the last heavy
-        } else {
-          oa[k] = self;
-        }
+      const bool hv = (heavy >> (t * 4 + k)) & 1;
+      arr[k] = hv ? a_l : a_h;                              // a heavy looks for its retiring light in SL
+      key[k] = hv ? sh[t][k] - 1 : sl[t][k] - dl[t][k];      // first SL >= y  <=>  first SL > y - 1
+    }
+    search4(arr, key, d, at);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool hv = (heavy >> (t * 4 + k)) & 1;
+      const uint32_t self = pos + k - lead;
+      if (!hv) {
+        oa[k] = at[k] < d ? at[k] : (last_heavy ? last_heavy - 1 - lead : self);
+      } else if (nh[k] != NONE32 && at[k] < d) {
+        op[t][k] = residual_prob(L.one + sh[t][k] - a_l[at[k]], L);
+        oa[k] = nh[k] - lead;
       } else {
-        const uint64_t y = s_sh[idx];
-        const uint32_t nxt = first_greater(s_sh, idx + 1, span, y);
-        const uint32_t li = nxt < span ? first_greater(s_sl, lead, span, y - 1) : span;
-        if (li < span) {
-          op[k] = residual_prob(L.one + y - s_sl[li], L);
-          oa[k] = nxt - lead;
-        } else {
-          op[k] = 1.0f;
-          oa[k] = self;
-        }
+        oa[k] = self;  // op is already 1
       }
     }
     if (pos >= lead && pos + 4 <= span) {
-      *reinterpret_cast<float4*>(prob + base + pos) = make_float4(op[0], op[1], op[2], op[3]);
+      *reinterpret_cast<float4*>(prob + base + pos) = make_float4(op[t][0], op[t][1], op[t][2], op[t][3]);
       *reinterpret_cast<uint4*>(alias + base + pos) = make_uint4(oa[0], oa[1], oa[2], oa[3]);
     } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const uint32_t idx = pos + k;
-        if (idx >= lead && idx < span) {
-          prob[base + idx] = op[k];
-          alias[base + idx] = oa[k];
+      for (int k = 0; k < 4; ++k)
+        if ((live >> (t * 4 + k)) & 1) {
+          prob[base + pos + k] = op[t][k];
+          alias[base + pos + k] = oa[k];
         }
-      }
     }
   }
   if (tid == 0) valid[v] = 1;

@@ -166,37 +166,85 @@ __device__ __forceinline__ uint64_t shfl_up_u64(uint64_t v, int delta) {
   const uint32_t hi = __shfl_up((int)(uint32_t)(v >> 32), delta, 64);
   return ((uint64_t)hi << 32) | lo;
 }
-// Sum over aligned groups of G lanes; every lane of the group receives the total.
-template <int G>
-__device__ __forceinline__ u128 group_sum_u128(u128 v) {
-#pragma unroll
-  for (int m = 1; m < G; m <<= 1) {
-    u128 o;
-    o.lo = shfl_xor_u64(v.lo, m);
-    o.hi = shfl_xor_u64(v.hi, m);
-    v = add128(v, o);
-  }
-  return v;
+// ---- DPP building blocks.  A wave is four rows of 16 lanes; row_shr:n moves data n lanes up inside a
+// row, row_bcast15 / row_bcast31 carry the last lane of a row (of the first half) to the next row(s).
+// Lanes without a source, and rows masked off, receive 0.  Callers must be convergent (all 64 lanes
+// active): a DPP read from a disabled lane is not defined.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp0(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xF, true);
 }
-// Inclusive prefix sum over aligned groups of G lanes.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t dpp0_u64(uint64_t v) {
+  const uint32_t lo = dpp0<CTRL, ROW_MASK>((uint32_t)v), hi = dpp0<CTRL, ROW_MASK>((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+constexpr int DPP_ROW_SHR1 = 0x111, DPP_ROW_SHR2 = 0x112, DPP_ROW_SHR4 = 0x114, DPP_ROW_SHR8 = 0x118;
+constexpr int DPP_ROW_BCAST15 = 0x142, DPP_ROW_BCAST31 = 0x143;
+constexpr int DPP_QUAD_XOR1 = 0xB1 /* quad_perm [1,0,3,2] */, DPP_QUAD_XOR2 = 0x4E /* quad_perm [2,3,0,1] */;
+constexpr int DPP_ROW_HALF_MIRROR = 0x141, DPP_ROW_MIRROR = 0x140;
+
+// Inclusive prefix sum over aligned groups of G lanes (G = 4, 8, 16, 32, 64).
 template <int G>
 __device__ __forceinline__ uint64_t group_scan_u64(uint64_t v) {
   const int gl = lane_id() & (G - 1);
-#pragma unroll
-  for (int d = 1; d < G; d <<= 1) {
-    const uint64_t o = shfl_up_u64(v, d);
-    if (gl >= d) v += o;
+  if (G >= 16) {
+    v += dpp0_u64<DPP_ROW_SHR1, 0xF>(v);
+    v += dpp0_u64<DPP_ROW_SHR2, 0xF>(v);
+    v += dpp0_u64<DPP_ROW_SHR4, 0xF>(v);
+    v += dpp0_u64<DPP_ROW_SHR8, 0xF>(v);
+    if (G >= 32) v += dpp0_u64<DPP_ROW_BCAST15, 0xA>(v);
+    if (G >= 64) v += dpp0_u64<DPP_ROW_BCAST31, 0xC>(v);
+  } else {
+    uint64_t o = dpp0_u64<DPP_ROW_SHR1, 0xF>(v);
+    v += gl >= 1 ? o : 0;
+    o = dpp0_u64<DPP_ROW_SHR2, 0xF>(v);
+    v += gl >= 2 ? o : 0;
+    if (G >= 8) {
+      o = dpp0_u64<DPP_ROW_SHR4, 0xF>(v);
+      v += gl >= 4 ? o : 0;
+    }
   }
   return v;
 }
 template <int G>
 __device__ __forceinline__ uint32_t group_scan_u32(uint32_t v) {
   const int gl = lane_id() & (G - 1);
-#pragma unroll
-  for (int d = 1; d < G; d <<= 1) {
-    const uint32_t o = __shfl_up((int)v, d, 64);
-    if (gl >= d) v += o;
+  if (G >= 16) {
+    v += dpp0<DPP_ROW_SHR1, 0xF>(v);
+    v += dpp0<DPP_ROW_SHR2, 0xF>(v);
+    v += dpp0<DPP_ROW_SHR4, 0xF>(v);
+    v += dpp0<DPP_ROW_SHR8, 0xF>(v);
+    if (G >= 32) v += dpp0<DPP_ROW_BCAST15, 0xA>(v);
+    if (G >= 64) v += dpp0<DPP_ROW_BCAST31, 0xC>(v);
+  } else {
+    uint32_t o = dpp0<DPP_ROW_SHR1, 0xF>(v);
+    v += gl >= 1 ? o : 0;
+    o = dpp0<DPP_ROW_SHR2, 0xF>(v);
+    v += gl >= 2 ? o : 0;
+    if (G >= 8) {
+      o = dpp0<DPP_ROW_SHR4, 0xF>(v);
+      v += gl >= 4 ? o : 0;
+    }
   }
+  return v;
+}
+// Sum over aligned groups of G lanes; every lane of the group receives the total.
+// Butterfly inside a row of 16 by DPP (xor 1, xor 2, half mirror, mirror), then across rows.
+template <int G>
+__device__ __forceinline__ u128 group_sum_u128(u128 v) {
+  auto mix = [&](auto get) {
+    u128 o;
+    o.lo = get(v.lo);
+    o.hi = get(v.hi);
+    v = add128(v, o);
+  };
+  mix([](uint64_t x) { return dpp0_u64<DPP_QUAD_XOR1, 0xF>(x); });
+  mix([](uint64_t x) { return dpp0_u64<DPP_QUAD_XOR2, 0xF>(x); });
+  if (G >= 8) mix([](uint64_t x) { return dpp0_u64<DPP_ROW_HALF_MIRROR, 0xF>(x); });
+  if (G >= 16) mix([](uint64_t x) { return dpp0_u64<DPP_ROW_MIRROR, 0xF>(x); });
+  if (G >= 32) mix([](uint64_t x) { return shfl_xor_u64(x, 16); });
+  if (G >= 64) mix([](uint64_t x) { return shfl_xor_u64(x, 32); });
   return v;
 }
 
