@@ -36,8 +36,8 @@
 //   scale= (double)deg / Sd ;  p_i = (double)w'_i * scale
 //   F    = 40 if deg < 2^22, else 62 - floor(log2(deg))    (fraction bits of the integer ledger)
 //   t_i  = (p_i - 1.0) * 2^F
-//   heavy iff t_i >= 0.5, with surplus U_i = floor(t_i + 0.5) >= 1                 (64-bit unsigned)
-//   light otherwise, with deficit D_i = floor(-t_i + 0.5)
+//   heavy iff t_i >= 0.5, with surplus U_i = max(rint(t_i), 1)                     (64-bit unsigned,
+//   light otherwise, with deficit D_i = rint(-t_i)                                  rint = nearest, ties to even)
 //   lights and heavies are taken in CSR slot order.  A sweep lets heavy j fill
 //   lights while its residual r (units of 2^-F) exceeds 2^F; when r <= 2^F the
 //   heavy becomes a bucket {prob = r*2^-F, alias = next heavy} and the next
@@ -237,7 +237,10 @@ static int alias_row_sweep(uint32_t deg, GetW getw, float* prob, uint32_t* alias
     if (excess(i) >= 0.5) heavy.push_back(i);
   }
   const size_t nH = heavy.size();
-  auto surplus = [&](uint32_t j) -> uint64_t { return (uint64_t)std::floor(excess(heavy[j]) + 0.5); };
+  auto surplus = [&](uint32_t j) -> uint64_t {
+    const uint64_t u = (uint64_t)std::nearbyint(excess(heavy[j]));  // default rounding mode: ties to even
+    return u ? u : 1;
+  };
   const uint64_t ONE = 1ull << F;
   if (nH == 0) {
     for (uint32_t i = 0; i < deg; ++i) { prob[i] = (float)p[i]; alias[i] = i; }
@@ -254,7 +257,7 @@ static int alias_row_sweep(uint32_t deg, GetW getw, float* prob, uint32_t* alias
       r += surplus(j + 1);
       ++j;
     }
-    const uint64_t D = (uint64_t)std::floor(-excess(i) + 0.5);
+    const uint64_t D = (uint64_t)std::nearbyint(-excess(i));
     prob[i] = (float)p[i];
     alias[i] = heavy[j];  // the last heavy also absorbs lights left without a donor
     // a heavy that is not the last has r > 2^32 > D here; the last heavy's r is never read again

@@ -7,8 +7,8 @@
 // parallelises:
 //   S     = sum floor(w_i 2^64)  (128 bit)        scale = deg / double(S)      p_i = w_i * scale
 //   F     = 40 fraction bits (62 - floor(log2 deg) for rows of 2^22 entries and more)
-//   t_i   = (p_i - 1) 2^F  ;  heavy iff t_i >= 0.5 : surplus U_i = floor(t_i + .5)
-//                             light otherwise      : deficit D_i = floor(-t_i + .5)
+//   t_i   = (p_i - 1) 2^F  ;  heavy iff t_i >= 0.5 : surplus U_i = max(rint(t_i), 1)
+//                             light otherwise      : deficit D_i = rint(-t_i)      (ties to even)
 //   SL(i) = inclusive prefix sum of deficits over slots <= i,  SH(i) likewise of surpluses
 //   light i : prob = float(p_i), alias = first slot m with SH(m) > SL(i) - D_i
 //             (the last heavy if there is none; itself if the row has no heavy)
@@ -37,8 +37,11 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 16) return CLS_SUB16;
   if (d <= 32) return CLS_SUB32;
   if (d <= 64) return CLS_WAVE;
+  if (d <= 125) return CLS_LDS_H1;
   if (d <= 253) return CLS_LDS_W1;
+  if (d <= 509) return CLS_LDS_W2;
   if (d <= 1021) return CLS_LDS_W4;
+  if (d <= 2045) return CLS_LDS_B2;
   if (d <= 4093) return CLS_LDS_B4;
   if (d <= 8189) return CLS_LDS_X2;
   return CLS_HUGE;
@@ -270,23 +273,28 @@ __device__ __forceinline__ void block_scan2(const uint64_t (&a)[Q][4], const uin
   tot_b = run_b;
 }
 
-// For four keys at once: number of leading entries of a_k[0..n) that are <= key_k (n if all are).
-__device__ __forceinline__ void search4(const uint64_t* const (&a)[4], const uint64_t (&key)[4], uint32_t n,
-                                        uint32_t (&pos)[4]) {
+// For four keys at once: number of entries of the sorted array that starts `base_k` bytes into the LDS
+// block `s` and has n >= 1 entries that are <= key_k.  The first probe narrows the answer to a window
+// of hb = 2^floor(log2 n) entries that ends inside the array, so no later probe needs a bound check.
+// Everything is kept as 32-bit byte offsets from `s` so that the probes stay LDS reads.
+__device__ __forceinline__ uint64_t lds_u64(const uint64_t* s, uint32_t byte_off) {
+  return *reinterpret_cast<const uint64_t*>(reinterpret_cast<const char*>(s) + byte_off);
+}
+__device__ __forceinline__ void search4(const uint64_t* s, const uint32_t (&base)[4], const uint64_t (&key)[4],
+                                        uint32_t n, uint32_t (&pos)[4]) {
+  const uint32_t hb = 1u << (31 - __clz((int)n));
+  uint32_t cur[4];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) pos[k] = 0;
-  for (uint32_t step = 1u << (31 - __clz((int)n)); step; step >>= 1) {
+  for (int k = 0; k < 4; ++k) cur[k] = base[k] + (lds_u64(s, base[k] + (hb - 1) * 8u) <= key[k] ? (n - hb) * 8u : 0u);
+  for (uint32_t step = hb * 4u; step >= 8u; step >>= 1) {  // step in bytes: hb/2 entries first
     uint64_t v[4];
-    uint32_t t[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      t[k] = pos[k] + step;
-      v[k] = a[k][min(t[k], n) - 1];
-    }
+    for (int k = 0; k < 4; ++k) v[k] = lds_u64(s, cur[k] + step - 8u);
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-      if (t[k] <= n && v[k] <= key[k]) pos[k] = t[k];
+    for (int k = 0; k < 4; ++k) cur[k] = v[k] <= key[k] ? cur[k] + step : cur[k];
   }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) pos[k] = (cur[k] - base[k]) / 8u + (lds_u64(s, cur[k]) <= key[k] ? 1u : 0u);
 }
 
 template <int ROWT, int T>
@@ -353,6 +361,7 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   uint64_t dl[T][4], dh[T][4], sl[T][4], sh[T][4];
   float op[T][4];
   uint32_t heavy = 0;
+  uint64_t hb_mask[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) {
 #pragma unroll
@@ -365,14 +374,18 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
       op[t][k] = e.heavy ? 1.0f : (float)e.p;
       if (in && e.heavy) heavy |= 1u << b;
     }
+    // first and last heavy slot of this (sub-tile, wave), from a ballot over the quads that hold a heavy
     const uint32_t m = (heavy >> (t * 4)) & 15u;
-    const uint32_t q0 = 4u * (t * ROWT + tid);
-    uint32_t fh = m ? q0 + (uint32_t)(__ffs((int)m) - 1) : NONE32;
-    uint32_t lh = m ? q0 + (uint32_t)(31 - __clz((int)m)) + 1 : 0;  // index + 1, 0 = none
-#pragma unroll
-    for (int x = 32; x >= 1; x >>= 1) {
-      fh = min(fh, (uint32_t)__shfl_xor((int)fh, x, 64));
-      lh = max(lh, (uint32_t)__shfl_xor((int)lh, x, 64));
+    const uint64_t bal = __ballot(m != 0);
+    hb_mask[t] = bal;
+    // readlane must see every lane's m: keep it out of divergent code
+    uint32_t fh = NONE32, lh = 0;  // lh holds index + 1, 0 = none
+    if (bal) {
+      const int l0 = __ffsll((unsigned long long)bal) - 1, l1 = 63 - __clzll((long long)bal);
+      const uint32_t m0 = (uint32_t)__builtin_amdgcn_readlane((int)m, l0);
+      const uint32_t m1 = (uint32_t)__builtin_amdgcn_readlane((int)m, l1);
+      fh = 4u * (t * ROWT + wave * 64 + l0) + (uint32_t)(__ffs((int)m0) - 1);
+      lh = 4u * (t * ROWT + wave * 64 + l1) + (uint32_t)(31 - __clz((int)m1)) + 1;
     }
     if (lane == 0) {
       s_fh[t][wave] = fh;
@@ -395,15 +408,12 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   uint32_t nh_after[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) {
+    // next quad of this wave that holds a heavy: first ballot bit above this lane
     const uint32_t m = (heavy >> (t * 4)) & 15u;
-    uint32_t suf = m ? 4u * (t * ROWT + tid) + (uint32_t)(__ffs((int)m) - 1) : NONE32;
-#pragma unroll
-    for (int dlt = 1; dlt < 64; dlt <<= 1) {
-      const uint32_t o = (uint32_t)__shfl_down((int)suf, dlt, 64);
-      if (lane + dlt < 64) suf = min(suf, o);
-    }
-    uint32_t nx = (uint32_t)__shfl_down((int)suf, 1, 64);
-    if (lane == 63) nx = NONE32;
+    const uint64_t above = hb_mask[t] & ~((2ull << lane) - 1);
+    const int ln = above ? __ffsll((unsigned long long)above) - 1 : lane;
+    const uint32_t mn = (uint32_t)__shfl((int)m, ln, 64);
+    uint32_t nx = above ? 4u * (t * ROWT + wave * 64 + ln) + (uint32_t)(__ffs((int)mn) - 1) : NONE32;
 #pragma unroll
     for (int wv = 0; wv < NW; ++wv) {
       if (wv > wave) nx = min(nx, s_fh[t][wv]);
@@ -416,12 +426,12 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   __syncthreads();  // s_sl / s_sh are complete
 
   const uint64_t* a_l = s_sl + lead;
-  const uint64_t* a_h = s_sh + lead;
+  const uint32_t off_l = lead * 8u, off_h = (CAP + lead) * 8u;  // byte offsets of the row inside smem
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const uint32_t pos = 4u * (t * ROWT + tid);
     if (pos >= span) continue;
-    const uint64_t* arr[4];
+    uint32_t arr[4];
     uint64_t key[4];
     uint32_t nh[4], oa[4], at[4];
     uint32_t nxt = nh_after[t];
@@ -433,10 +443,10 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const bool hv = (heavy >> (t * 4 + k)) & 1;
-      arr[k] = hv ? a_l : a_h;                              // a heavy looks for its retiring light in SL
+      arr[k] = hv ? off_l : off_h;                          // a heavy looks for its retiring light in SL
       key[k] = hv ? sh[t][k] - 1 : sl[t][k] - dl[t][k];      // first SL >= y  <=>  first SL > y - 1
     }
-    search4(arr, key, d, at);
+    search4(smem, arr, key, d, at);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const bool hv = (heavy >> (t * 4 + k)) & 1;
@@ -743,8 +753,11 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
+  SKY_TRY(lds(CLS_LDS_H1, build_lds_kernel<64, 1>, 64, 1, "lds_h1"));
   SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
+  SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
   SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<64, 4>, 64, 4, "lds_w4"));
+  SKY_TRY(lds(CLS_LDS_B2, build_lds_kernel<256, 2>, 256, 2, "lds_b2"));
   SKY_TRY(lds(CLS_LDS_B4, build_lds_kernel<256, 4>, 256, 4, "lds_b4"));
   SKY_TRY(lds(CLS_LDS_X2, build_lds_kernel<1024, 2>, 1024, 2, "lds_x2"));
 

@@ -115,18 +115,25 @@ __device__ __forceinline__ Ledger make_ledger(uint32_t deg, u128 sum) {
   L.inv_fs = 1.0 / L.fs;
   return L;
 }
-// Per-entry classification: t = (p - 1) * 2^F; heavy iff t >= 0.5.
+// Per-entry classification: t = (p - 1) * 2^F; heavy iff t >= 0.5; amount = max(rint(|t|), 1 if heavy).
 struct Entry {
   double p;
   uint64_t amount;  // surplus (heavy) or deficit (light), units of 2^-F
   bool heavy;
 };
+// |t| rounded to the nearest integer, ties to even.  Below 2^52 adding 2^52 leaves the rounded integer in
+// the low mantissa bits (two instructions); from 2^52 on a double is an integer already.
+__device__ __forceinline__ uint64_t round_to_u64(double x) {
+  if (x < 4503599627370496.0) return (uint64_t)__double_as_longlong(x + 4503599627370496.0) - 0x4330000000000000ull;
+  return (uint64_t)x;
+}
 __device__ __forceinline__ Entry classify(float w, const Ledger& L) {
   Entry e;
   e.p = (double)w * L.scale;
   const double t = (e.p - 1.0) * L.fs;
   e.heavy = t >= 0.5;
-  e.amount = (uint64_t)floor((e.heavy ? t : -t) + 0.5);
+  e.amount = round_to_u64(fmax(e.heavy ? t : -t, 0.0));  // a light with 0 < t < 0.5 has deficit 0
+  if (e.heavy && e.amount == 0) e.amount = 1;  // t = 0.5 exactly rounds to even 0: a heavy always has surplus >= 1
   return e;
 }
 __device__ __forceinline__ float residual_prob(uint64_t r_units, const Ledger& L) {

@@ -37,12 +37,15 @@ enum BuildClass : int {
   CLS_SUB16 = 4,   // deg 9..16
   CLS_SUB32 = 5,   // deg 17..32
   CLS_WAVE = 6,    // deg 33..64       one wavefront, one entry per lane
-  CLS_LDS_W1 = 7,  // deg <= 253       one wavefront, LDS prefix arrays, 4 entries per lane
-  CLS_LDS_W4 = 8,  // deg <= 1021      one wavefront, 16 entries per lane
-  CLS_LDS_B4 = 9,  // deg <= 4093      256 threads
-  CLS_LDS_X2 = 10, // deg <= 8189      1024 threads, 128 KB of LDS
-  CLS_HUGE = 11,   // above            1024 threads streaming through a global scratch
-  CLS_COUNT = 12
+  CLS_LDS_H1 = 7,  // deg <= 125       one wavefront, LDS prefix arrays, 4 entries per lane (half the lanes idle)
+  CLS_LDS_W1 = 8,  // deg <= 253       one wavefront, 4 entries per lane
+  CLS_LDS_W2 = 9,  // deg <= 509       one wavefront, 8 entries per lane
+  CLS_LDS_W4 = 10, // deg <= 1021      one wavefront, 16 entries per lane
+  CLS_LDS_B2 = 11, // deg <= 2045      256 threads, 8 entries per thread
+  CLS_LDS_B4 = 12, // deg <= 4093      256 threads, 16 entries per thread
+  CLS_LDS_X2 = 13, // deg <= 8189      1024 threads, 128 KB of LDS
+  CLS_HUGE = 14,   // above            built tile by tile by the whole GPU
+  CLS_COUNT = 15
 };
 
 // Sequence of HIP events on one stream; consecutive marks bracket one kernel (or group).
