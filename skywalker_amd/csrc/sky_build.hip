@@ -25,6 +25,7 @@
 // and 1024 threads streaming through a global scratch for rows beyond 128 KB of LDS.
 #include <algorithm>
 
+#include "sky_build_common.h"
 #include "sky_graph.h"
 
 namespace sky {
@@ -219,84 +220,6 @@ __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __re
 // and keeps its search key in registers; SL and SH of every slot live in LDS.  Each entry then
 // does exactly one binary search, lights in SH and heavies in SL, four searches interleaved; the
 // next heavy after each heavy and the last heavy of the row come from a suffix scan, not a search.
-constexpr uint32_t NONE32 = 0xFFFFFFFFu;
-
-// Inclusive prefixes of two quantities over the slots of a tile held as [Q][4] per thread (slot order:
-// quad q of thread tid, then thread tid + 1; sub-tile q before q + 1).  One barrier.
-template <int ROWT, int Q>
-__device__ __forceinline__ void block_scan2(const uint64_t (&a)[Q][4], const uint64_t (&b)[Q][4],
-                                            uint64_t* __restrict__ s_ex /* [2 * Q * ROWT/64] */,
-                                            uint64_t (&oa)[Q][4], uint64_t (&ob)[Q][4], uint64_t& tot_a,
-                                            uint64_t& tot_b) {
-  constexpr int NW = ROWT / 64;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  uint64_t ia[Q], ib[Q];
-#pragma unroll
-  for (int q = 0; q < Q; ++q) {
-    uint64_t ra = 0, rb = 0;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      ra += a[q][k];
-      rb += b[q][k];
-      oa[q][k] = ra;
-      ob[q][k] = rb;
-    }
-    ia[q] = group_scan_u64<64>(ra);
-    ib[q] = group_scan_u64<64>(rb);
-    if (lane == 63) {
-      s_ex[(q * NW + wave) * 2] = ia[q];
-      s_ex[(q * NW + wave) * 2 + 1] = ib[q];
-    }
-    ia[q] -= ra;  // exclusive over the lanes of this wave
-    ib[q] -= rb;
-  }
-  __syncthreads();
-  uint64_t run_a = 0, run_b = 0;
-#pragma unroll
-  for (int q = 0; q < Q; ++q) {
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      if (w == wave) {
-        ia[q] += run_a;
-        ib[q] += run_b;
-      }
-      run_a += s_ex[(q * NW + w) * 2];
-      run_b += s_ex[(q * NW + w) * 2 + 1];
-    }
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      oa[q][k] += ia[q];
-      ob[q][k] += ib[q];
-    }
-  }
-  tot_a = run_a;
-  tot_b = run_b;
-}
-
-// For four keys at once: number of entries of the sorted array that starts `base_k` bytes into the LDS
-// block `s` and has n >= 1 entries that are <= key_k.  The first probe narrows the answer to a window
-// of hb = 2^floor(log2 n) entries that ends inside the array, so no later probe needs a bound check.
-// Everything is kept as 32-bit byte offsets from `s` so that the probes stay LDS reads.
-__device__ __forceinline__ uint64_t lds_u64(const uint64_t* s, uint32_t byte_off) {
-  return *reinterpret_cast<const uint64_t*>(reinterpret_cast<const char*>(s) + byte_off);
-}
-__device__ __forceinline__ void search4(const uint64_t* s, const uint32_t (&base)[4], const uint64_t (&key)[4],
-                                        uint32_t n, uint32_t (&pos)[4]) {
-  const uint32_t hb = 1u << (31 - __clz((int)n));
-  uint32_t cur[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) cur[k] = base[k] + (lds_u64(s, base[k] + (hb - 1) * 8u) <= key[k] ? (n - hb) * 8u : 0u);
-  for (uint32_t step = hb * 4u; step >= 8u; step >>= 1) {  // step in bytes: hb/2 entries first
-    uint64_t v[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] = lds_u64(s, cur[k] + step - 8u);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) cur[k] = v[k] <= key[k] ? cur[k] + step : cur[k];
-  }
-#pragma unroll
-  for (int k = 0; k < 4; ++k) pos[k] = (cur[k] - base[k]) / 8u + (lds_u64(s, cur[k]) <= key[k] ? 1u : 0u);
-}
-
 template <int ROWT, int T>
 __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restrict__ vlist,
                                                          const uint32_t* __restrict__ xadj,

@@ -16,6 +16,7 @@
 // is at most twice its tile count: no per-slot scratch in global memory, O(1) passes over the weights.
 #include <algorithm>
 
+#include "sky_build_common.h"
 #include "sky_graph.h"
 
 namespace sky {
@@ -23,7 +24,6 @@ namespace sky {
 constexpr int TL_T = 256;                // threads per tile
 constexpr int TL_Q = 4;                  // float4 quads per thread
 constexpr int TILE = TL_T * 4 * TL_Q;    // 4096 slots
-constexpr uint32_t NONE32 = 0xFFFFFFFFu;
 constexpr uint32_t TILED_MAX_TILES = 2047;  // tile prefixes of one row must fit the emit kernel's LDS
 
 struct TiledRow {
@@ -70,10 +70,10 @@ __device__ __forceinline__ bool in_row(const TiledRow& r, uint32_t idx) { return
 __global__ __launch_bounds__(1024) void tiled_rows_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
                                                           const uint32_t* __restrict__ xadj, uint32_t max_tiles,
                                                           TiledRow* __restrict__ rows,
-                                                          uint32_t* __restrict__ totals /* [0] tiles, [1] skipped rows */) {
+                                                          uint32_t* __restrict__ totals /* [0] tiles, [1] skipped rows, [2] most tiles in a row */) {
   __shared__ uint32_t s_w[16];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  uint32_t carry = 0, skipped = 0;
+  uint32_t carry = 0, skipped = 0, most = 0;
   for (uint32_t chunk = 0; chunk < count; chunk += 1024) {
     const uint32_t r = chunk + tid;
     TiledRow row = {};
@@ -91,6 +91,7 @@ __global__ __launch_bounds__(1024) void tiled_rows_kernel(const uint32_t* __rest
         ++skipped;
       }
       row.ntiles = nt;
+      most = max(most, nt);
     }
     const uint32_t inc = group_scan_u32<64>(nt);
     __syncthreads();
@@ -108,15 +109,26 @@ __global__ __launch_bounds__(1024) void tiled_rows_kernel(const uint32_t* __rest
     carry += t;
   }
   // skipped rows: sum over the block
-  for (int m = 32; m >= 1; m >>= 1) skipped += __shfl_xor((int)skipped, m, 64);
+  for (int m = 32; m >= 1; m >>= 1) {
+    skipped += __shfl_xor((int)skipped, m, 64);
+    most = max(most, (uint32_t)__shfl_xor((int)most, m, 64));
+  }
+  __shared__ uint32_t s_most[16];
   __syncthreads();
-  if (lane == 0) s_w[wave] = skipped;
+  if (lane == 0) {
+    s_w[wave] = skipped;
+    s_most[wave] = most;
+  }
   __syncthreads();
   if (tid == 0) {
-    uint32_t s = 0;
-    for (int k = 0; k < 16; ++k) s += s_w[k];
+    uint32_t s = 0, mm = 0;
+    for (int k = 0; k < 16; ++k) {
+      s += s_w[k];
+      mm = max(mm, s_most[k]);
+    }
     totals[0] = carry;
     totals[1] = s;
+    totals[2] = mm;
   }
 }
 
@@ -295,59 +307,75 @@ __global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ r
 }
 
 // ---------------------------------------------------------------- pass 3: every entry of a tile
-// Inclusive prefix of `val` over the slots of one tile in slot order (quad q of thread tid before quad
-// q of thread tid+1, sub-tile q before q+1), starting from `base`.
-struct TileScan {
-  uint64_t* s_wave;  // [TL_T/64]
-  __device__ __forceinline__ void run(const uint64_t (&val)[TL_Q][4], uint64_t base, uint64_t (&out)[TL_Q][4]) {
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    uint64_t carry = base;
-#pragma unroll
-    for (int q = 0; q < TL_Q; ++q) {
-      uint64_t run = 0, loc[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        run += val[q][k];
-        loc[k] = run;
-      }
-      const uint64_t inc = group_scan_u64<64>(run);
-      __syncthreads();
-      if (lane == 63) s_wave[wave] = inc;
-      __syncthreads();
-      uint64_t before = carry + inc - run, tot = 0;
-#pragma unroll
-      for (int i = 0; i < TL_T / 64; ++i) {
-        if (i == wave) before += tot;
-        tot += s_wave[i];
-      }
-#pragma unroll
-      for (int k = 0; k < 4; ++k) out[q][k] = before + loc[k];
-      carry += tot;
-    }
-  }
-};
-
-// first j in [0, TILE) with P[j] > key (TILE if none), four keys at a time
-__device__ __forceinline__ void search4(const uint64_t* __restrict__ P, const uint64_t (&key)[4], uint32_t (&pos)[4]) {
-#pragma unroll
-  for (int k = 0; k < 4; ++k) pos[k] = 0;
-#pragma unroll
-  for (uint32_t step = TILE / 2; step >= 1; step >>= 1) {
-    uint64_t v[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] = P[pos[k] + step - 1];
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-      if (v[k] <= key[k]) pos[k] += step;
-  }
-#pragma unroll
-  for (int k = 0; k < 4; ++k)
-    if (P[pos[k]] <= key[k]) pos[k] += 1;
-}
-
 // first t in [0, nt) with B[t + 1] > key (nt if none)
 __device__ __forceinline__ uint32_t first_tile_above(const uint64_t* B, uint32_t nt, uint64_t key) {
   return first_greater(B + 1, 0, nt, key);
+}
+
+// One pass over the partner tiles of one kind.  OWN_HEAVY = false: own lights (key = exclusive deficit
+// prefix x) against the surplus prefix of the tiles whose range [B[pt], B[pt+1]) holds x.
+// OWN_HEAVY = true: own heavies (key = y - 1) against the deficit prefix, same range test.
+template <bool OWN_HEAVY>
+__device__ __forceinline__ void partner_pass(const TiledRow& r, const Ledger& L, const float* __restrict__ wgt,
+                                             const uint64_t* s_B, uint32_t t_lo, uint32_t t_hi, uint64_t* smem,
+                                             uint64_t* s_ex, uint32_t heavy_mask, uint32_t live_mask,
+                                             const uint32_t (&nh_after)[TL_Q], uint32_t T,
+                                             const uint64_t (&key)[TL_Q][4], float (&op)[TL_Q][4],
+                                             uint32_t (&oa)[TL_Q][4]) {
+  const int tid = threadIdx.x;
+  const uint32_t nt = r.ntiles;
+  for (uint32_t pt = t_lo; pt <= t_hi && pt < nt; ++pt) {
+    const uint64_t lo = s_B[pt], hi = s_B[pt + 1];
+    if (hi == lo) continue;
+    float pw[TL_Q][4];
+    load_tile(wgt, r, pt, tid, pw);
+    uint64_t pv[TL_Q][4], ps[TL_Q][4];
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t idx = pt * TILE + 4u * (q * TL_T + tid) + k;
+        const Entry e = classify(pw[q][k], L);
+        pv[q][k] = (in_row(r, idx) && e.heavy != OWN_HEAVY) ? e.amount : 0;
+      }
+    __syncthreads();  // searches of the previous partner are done: s_ex and P may be overwritten
+    block_scan1<TL_T, TL_Q>(pv, s_ex, lo, ps);
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) smem[4u * (q * TL_T + tid) + k] = ps[q][k];
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q) {
+      uint32_t mine = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int b = q * 4 + k;
+        const bool kind = ((live_mask >> b) & 1) && (((heavy_mask >> b) & 1) != 0) == OWN_HEAVY;
+        if (kind && key[q][k] >= lo && key[q][k] < hi) mine |= 1u << k;
+      }
+      if (!mine) continue;
+      const uint32_t base[4] = {0, 0, 0, 0};
+      uint32_t pos[4];
+      search4(smem, base, key[q], (uint32_t)TILE, pos);
+      if (OWN_HEAVY) {
+        // next heavy after each slot of the quad; the row's last heavy never retires
+        uint32_t nxt = nh_after[q];
+#pragma unroll
+        for (int k = 3; k >= 0; --k) {
+          if (((mine >> k) & 1) && nxt != NONE32) {
+            op[q][k] = residual_prob(L.one + key[q][k] + 1 - smem[pos[k]], L);
+            oa[q][k] = nxt - r.lead;
+          }
+          if ((heavy_mask >> (q * 4 + k)) & 1) nxt = T * TILE + 4u * (q * TL_T + tid) + k;
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if ((mine >> k) & 1) oa[q][k] = pt * TILE + pos[k] - r.lead;
+      }
+    }
+  }
 }
 
 __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __restrict__ tile2row,
@@ -358,11 +386,11 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
                                                           const uint32_t* __restrict__ nfh, float* __restrict__ prob,
                                                           uint32_t* __restrict__ alias,
                                                           int8_t* __restrict__ valid) {
-  extern __shared__ uint64_t smem[];
-  uint64_t* P = smem;                  // [TILE] per-slot prefix of the current partner tile
+  constexpr int NW = TL_T / 64;
+  extern __shared__ uint64_t smem[];   // [TILE] per-slot prefix of the current partner tile, then BL, BH
   uint64_t* s_BL = smem + TILE;        // [nt + 1]
-  __shared__ uint64_t s_wave[TL_T / 64];
-  __shared__ uint32_t s_first[TL_Q][TL_T / 64];
+  __shared__ uint64_t s_ex[2 * TL_Q * NW];
+  __shared__ uint32_t s_fh[TL_Q][NW];
   const uint32_t tile = blockIdx.x;
   const uint32_t ri = tile2row[tile];
   const TiledRow r = rows[ri];
@@ -393,76 +421,65 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
     s_BH[i] = gBH[b0 + i];
   }
 
-  // own tile: class, amount, prefix of the own kind -> key (x of a light, y of a heavy)
-  uint64_t dl[TL_Q][4], dh[TL_Q][4], key[TL_Q][4];
+  // own tile: class and amount of every slot, prefix of the own kind -> search key
+  uint64_t key[TL_Q][4];
   float op[TL_Q][4];
   uint32_t oa[TL_Q][4];
   uint32_t heavy_mask = 0, live_mask = 0;
-#pragma unroll
-  for (int q = 0; q < TL_Q; ++q)
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const uint32_t idx = T * TILE + 4u * (q * TL_T + tid) + k;
-      const Entry e = classify(w[q][k], L);
-      const bool in = in_row(r, idx);
-      dl[q][k] = (in && !e.heavy) ? e.amount : 0;
-      dh[q][k] = (in && e.heavy) ? e.amount : 0;
-      op[q][k] = e.heavy ? 1.0f : (float)e.p;
-      if (in) live_mask |= 1u << (q * 4 + k);
-      if (in && e.heavy) heavy_mask |= 1u << (q * 4 + k);
-    }
-  __syncthreads();  // s_BL / s_BH are complete
-  TileScan scan{s_wave};
+  uint64_t hb_mask[TL_Q];
   {
-    uint64_t sl[TL_Q][4], sh[TL_Q][4];
-    scan.run(dl, s_BL[T], sl);
-    scan.run(dh, s_BH[T], sh);
+    uint64_t dl[TL_Q][4], dh[TL_Q][4], sl[TL_Q][4], sh[TL_Q][4];
+#pragma unroll
+    for (int q = 0; q < TL_Q; ++q) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t idx = T * TILE + 4u * (q * TL_T + tid) + k;
+        const Entry e = classify(w[q][k], L);
+        const bool in = in_row(r, idx);
+        dl[q][k] = (in && !e.heavy) ? e.amount : 0;
+        dh[q][k] = (in && e.heavy) ? e.amount : 0;
+        op[q][k] = e.heavy ? 1.0f : (float)e.p;
+        if (in) live_mask |= 1u << (q * 4 + k);
+        if (in && e.heavy) heavy_mask |= 1u << (q * 4 + k);
+      }
+      const uint32_t m = (heavy_mask >> (q * 4)) & 15u;
+      const uint64_t bal = __ballot(m != 0);
+      hb_mask[q] = bal;
+      uint32_t fh = NONE32;
+      if (bal) {
+        const int l0 = __ffsll((unsigned long long)bal) - 1;
+        const uint32_t m0 = (uint32_t)__builtin_amdgcn_readlane((int)m, l0);
+        fh = T * TILE + 4u * (q * TL_T + wave * 64 + l0) + (uint32_t)(__ffs((int)m0) - 1);
+      }
+      if (lane == 0) s_fh[q][wave] = fh;
+    }
+    uint64_t tl, th;
+    block_scan2<TL_T, TL_Q>(dl, dh, s_ex, sl, sh, tl, th);  // its barrier also publishes s_BL / s_BH / s_fh
+    const uint64_t bl = s_BL[T], bh = s_BH[T];
 #pragma unroll
     for (int q = 0; q < TL_Q; ++q)
 #pragma unroll
-      for (int k = 0; k < 4; ++k) key[q][k] = (heavy_mask >> (q * 4 + k)) & 1 ? sh[q][k] : sl[q][k] - dl[q][k];
+      for (int k = 0; k < 4; ++k)
+        key[q][k] = ((heavy_mask >> (q * 4 + k)) & 1) ? bh + sh[q][k] - 1 : bl + sl[q][k] - dl[q][k];
   }
-
-  // next heavy after each own heavy (span index), NONE32 for the last heavy of the row
-  uint32_t nh_after_quad[TL_Q];
+  // next heavy after each quad (span index): later lanes, later waves, later sub-tiles, later tiles
+  uint32_t nh_after[TL_Q];
   {
-    uint32_t qfirst[TL_Q];
-#pragma unroll
-    for (int q = 0; q < TL_Q; ++q) {
-      const uint32_t m = (heavy_mask >> (q * 4)) & 15u;
-      qfirst[q] = m ? T * TILE + 4u * (q * TL_T + tid) + (uint32_t)(__ffs((int)m) - 1) : NONE32;
-      uint32_t suf = qfirst[q];
-#pragma unroll
-      for (int dlt = 1; dlt < 64; dlt <<= 1) {
-        const uint32_t o = (uint32_t)__shfl_down((int)suf, dlt, 64);
-        if (lane + dlt < 64) suf = min(suf, o);
-      }
-      uint32_t excl = (uint32_t)__shfl_down((int)suf, 1, 64);
-      if (lane == 63) excl = NONE32;
-      nh_after_quad[q] = excl;
-      if (lane == 0) s_first[q][wave] = suf;
-    }
-    __syncthreads();
     const uint32_t later_tiles = nfh[tile];
 #pragma unroll
     for (int q = 0; q < TL_Q; ++q) {
-      uint32_t m = later_tiles;
-      for (int wv = 0; wv < TL_T / 64; ++wv) {
-        if (wv > wave) m = min(m, s_first[q][wv]);
+      const uint32_t m = (heavy_mask >> (q * 4)) & 15u;
+      const uint64_t above = hb_mask[q] & ~((2ull << lane) - 1);
+      const int ln = above ? __ffsll((unsigned long long)above) - 1 : lane;
+      const uint32_t mn = (uint32_t)__shfl((int)m, ln, 64);
+      uint32_t nx = above ? T * TILE + 4u * (q * TL_T + wave * 64 + ln) + (uint32_t)(__ffs((int)mn) - 1) : later_tiles;
 #pragma unroll
-        for (int q2 = q + 1; q2 < TL_Q; ++q2) m = min(m, s_first[q2][wv]);
+      for (int wv = 0; wv < NW; ++wv) {
+        if (wv > wave) nx = min(nx, s_fh[q][wv]);
+#pragma unroll
+        for (int q2 = q + 1; q2 < TL_Q; ++q2) nx = min(nx, s_fh[q2][wv]);
       }
-      nh_after_quad[q] = min(nh_after_quad[q], m);
-    }
-  }
-  uint32_t nh[TL_Q][4];
-#pragma unroll
-  for (int q = 0; q < TL_Q; ++q) {
-    uint32_t nxt = nh_after_quad[q];
-#pragma unroll
-    for (int k = 3; k >= 0; --k) {
-      nh[q][k] = nxt;
-      if ((heavy_mask >> (q * 4 + k)) & 1) nxt = T * TILE + 4u * (q * TL_T + tid) + k;
+      nh_after[q] = nx;
     }
   }
   // defaults: a light without donor takes the last heavy (itself if the row has none);
@@ -476,100 +493,16 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
       oa[q][k] = (!heavy && r.total_h) ? r.last_heavy - r.lead : idx - r.lead;
     }
 
-  // ---- lights against the surplus prefix of their partner tiles
-  {
-    const uint32_t t_lo = first_tile_above(s_BH, nt, s_BL[T]);
-    const uint32_t t_hi = min(first_tile_above(s_BH, nt, s_BL[T + 1]), nt - 1);
-    for (uint32_t pt = t_lo; pt <= t_hi && pt < nt; ++pt) {
-      const uint64_t lo = s_BH[pt], hi = s_BH[pt + 1];
-      if (hi == lo) continue;
-      float pw[TL_Q][4];
-      load_tile(wgt, r, pt, tid, pw);
-      uint64_t pv[TL_Q][4], ps[TL_Q][4];
-#pragma unroll
-      for (int q = 0; q < TL_Q; ++q)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const uint32_t idx = pt * TILE + 4u * (q * TL_T + tid) + k;
-          const Entry e = classify(pw[q][k], L);
-          pv[q][k] = (in_row(r, idx) && e.heavy) ? e.amount : 0;
-        }
-      scan.run(pv, lo, ps);
-      __syncthreads();  // previous partner's searches are done
-#pragma unroll
-      for (int q = 0; q < TL_Q; ++q)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) P[4u * (q * TL_T + tid) + k] = ps[q][k];
-      __syncthreads();
-#pragma unroll
-      for (int q = 0; q < TL_Q; ++q) {
-        bool mine[4], any = false;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int b = q * 4 + k;
-          mine[k] = ((live_mask >> b) & 1) && !((heavy_mask >> b) & 1) && key[q][k] >= lo && key[q][k] < hi;
-          any |= mine[k];
-        }
-        if (!any) continue;
-        uint32_t pos[4];
-        search4(P, key[q], pos);
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (mine[k]) oa[q][k] = pt * TILE + pos[k] - r.lead;
-      }
-    }
-  }
-  // ---- heavies against the deficit prefix of their partner tiles
-  {
-    const uint32_t t_lo = first_tile_above(s_BL, nt, s_BH[T]);  // first t with BL[t+1] >= BH[T] + 1
-    const uint32_t t_hi = min(s_BH[T + 1] ? first_tile_above(s_BL, nt, s_BH[T + 1] - 1) : 0u, nt - 1);
-    const bool any_heavy = s_BH[T + 1] != s_BH[T];
-    for (uint32_t pt = t_lo; any_heavy && pt <= t_hi && pt < nt; ++pt) {
-      const uint64_t lo = s_BL[pt], hi = s_BL[pt + 1];
-      if (hi == lo) continue;
-      float pw[TL_Q][4];
-      load_tile(wgt, r, pt, tid, pw);
-      uint64_t pv[TL_Q][4], ps[TL_Q][4];
-#pragma unroll
-      for (int q = 0; q < TL_Q; ++q)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const uint32_t idx = pt * TILE + 4u * (q * TL_T + tid) + k;
-          const Entry e = classify(pw[q][k], L);
-          pv[q][k] = (in_row(r, idx) && !e.heavy) ? e.amount : 0;
-        }
-      scan.run(pv, lo, ps);
-      __syncthreads();
-#pragma unroll
-      for (int q = 0; q < TL_Q; ++q)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) P[4u * (q * TL_T + tid) + k] = ps[q][k];
-      __syncthreads();
-#pragma unroll
-      for (int q = 0; q < TL_Q; ++q) {
-        bool mine[4], any = false;
-        uint64_t km1[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int b = q * 4 + k;
-          // a heavy retires in this partner iff lo < y <= hi; the last heavy of the row never retires
-          mine[k] = ((heavy_mask >> b) & 1) && nh[q][k] != NONE32 && key[q][k] > lo && key[q][k] <= hi;
-          km1[k] = key[q][k] - 1;
-          any |= mine[k];
-        }
-        if (!any) continue;
-        uint32_t pos[4];
-        search4(P, km1, pos);
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (mine[k]) {
-            op[q][k] = residual_prob(L.one + key[q][k] - P[pos[k]], L);
-            oa[q][k] = nh[q][k] - r.lead;
-          }
-      }
-    }
-  }
-  // ---- store
+  // lights: partner tiles are those whose surplus range meets [BL[T], BL[T+1]]
+  partner_pass<false>(r, L, wgt, s_BH, first_tile_above(s_BH, nt, s_BL[T]),
+                      min(first_tile_above(s_BH, nt, s_BL[T + 1]), nt - 1), smem, s_ex, heavy_mask, live_mask,
+                      nh_after, T, key, op, oa);
+  // heavies: y in (BH[T], BH[T+1]] retires in the tile whose deficit range (BL[t], BL[t+1]] holds y
+  if (s_BH[T + 1] != s_BH[T])
+    partner_pass<true>(r, L, wgt, s_BL, first_tile_above(s_BL, nt, s_BH[T]),
+                       min(first_tile_above(s_BL, nt, s_BH[T + 1] - 1), nt - 1), smem, s_ex, heavy_mask, live_mask,
+                       nh_after, T, key, op, oa);
+
 #pragma unroll
   for (int q = 0; q < TL_Q; ++q) {
     const uint32_t pos = T * TILE + 4u * (q * TL_T + tid);
@@ -623,7 +556,7 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
     SKY_HIP(hipMalloc((void**)&sc.rows, (size_t)n * sizeof(TiledRow)));
     sc.row_cap = n;
   }
-  if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, 8));
+  if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, 12));
   if (!sc.lds_enabled) {
     SKY_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_emit_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -632,8 +565,8 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
   }
   hipLaunchKernelGGL(tiled_rows_kernel, dim3(1), dim3(1024), 0, st, rows_list, n, g->xadj, g_tiled_max_tiles, sc.rows,
                      sc.totals);
-  uint32_t totals[2] = {0, 0};
-  SKY_HIP(hipMemcpyAsync(totals, sc.totals, 8, hipMemcpyDeviceToHost, st));
+  uint32_t totals[3] = {0, 0, 0};
+  SKY_HIP(hipMemcpyAsync(totals, sc.totals, 12, hipMemcpyDeviceToHost, st));
   SKY_HIP(hipStreamSynchronize(st));
   const uint32_t ntiles = totals[0];
   *skipped = totals[1];
@@ -668,7 +601,7 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
   hipLaunchKernelGGL(tiled_ledger_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.tsum);
   hipLaunchKernelGGL(tiled_totals_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.ttot);
   hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh);
-  const size_t lds = (size_t)(TILE + 2 * (g_tiled_max_tiles + 1)) * 8;
+  const size_t lds = (size_t)(TILE + 2 * (totals[2] + 1)) * 8;  // partner prefix + the longest row's tile prefixes
   hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), lds, st, sc.tile2row, sc.rows, g->adjwgt, sc.BL,
                      sc.BH, sc.nfh, g->prob, g->alias, g->valid);
   return SKY_OK;
