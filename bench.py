@@ -27,9 +27,9 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
     "bin": "bin_count_kernel+bin_scatter_kernel", "sub4": "build_subwave_kernel<4>", "sub8": "build_subwave_kernel<8>",
     "sub16": "build_subwave_kernel<16>", "sub32": "build_subwave_kernel<32>", "wave64": "build_subwave_kernel<64>",
     "lds_h1": "build_lds_kernel<64,1> (deg<=125)", "lds_w1": "build_lds_kernel<64,1>",
-    "lds_w2": "build_lds_kernel<64,2>", "lds_w4": "build_lds_kernel<64,4>", "lds_b2": "build_lds_kernel<256,2>",
-    "lds_b4": "build_lds_kernel<256,4>", "lds_x2": "build_lds_kernel<1024,2>",
-    "huge": "tiled_*_kernel (rows > 8189)",
+    "lds_w2": "build_lds_kernel<64,2>", "lds_w4": "build_lds_kernel<128,2>", "lds_b2": "build_lds_kernel<256,2>",
+    "lds_b4": "build_lds_kernel<512,2>",
+    "huge": "tiled_*_kernel (rows > 4093)",
 }
 
 

@@ -122,8 +122,8 @@ int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, co
  *      ctr_host[4n], key_host[2n] -> out_host[4n]. ---- */
 int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint32_t n, uint32_t* out_host);
 
-/* ---- tuning knobs (no counterpart in the reference).  "tiled_max_tiles": rows of more than 8189 entries are
- *      built tile by tile (4096 entries per tile) up to this many tiles (default and maximum 2047); longer rows
+/* ---- tuning knobs (no counterpart in the reference).  "tiled_max_tiles": rows of more than 4093 entries are
+ *      built tile by tile (1024 entries per tile) up to this many tiles (default: no limit); longer rows
  *      are streamed by one workgroup each.  Tests lower it to exercise the streaming kernel. ---- */
 int sky_set_option(const char* name, long value);
 

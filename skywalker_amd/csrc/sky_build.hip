@@ -21,8 +21,8 @@
 //
 // Dispatch is by degree class (sky_graph.h): one lane per vertex while binning (deg <= 2),
 // 4/8/16/32/64 lanes per vertex with the prefix arrays in a per-wave LDS strip,
-// one wavefront / 256 / 1024 threads per vertex with the row's prefix arrays in LDS,
-// and 1024 threads streaming through a global scratch for rows beyond 128 KB of LDS.
+// 64 to 512 threads per vertex with the row's prefix arrays in LDS (rows up to 4093 entries),
+// and the tile-parallel path of sky_build_tiled.hip for longer rows.
 #include <algorithm>
 
 #include "sky_build_common.h"
@@ -44,7 +44,6 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 1021) return CLS_LDS_W4;
   if (d <= 2045) return CLS_LDS_B2;
   if (d <= 4093) return CLS_LDS_B4;
-  if (d <= 8189) return CLS_LDS_X2;
   return CLS_HUGE;
 }
 
@@ -241,10 +240,17 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
 
   float w[T][4];
   u128 sum{0, 0};
-  uint32_t live = 0;  // bit q*4+k: slot belongs to the row
+  uint32_t live = 0;       // bit q*4+k: slot belongs to the row
+  uint32_t wave_live = 0;  // bit t: some slot of this wave's strip of sub-tile t belongs to the row
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const uint32_t pos = 4u * (t * ROWT + tid);
+    if (4u * (t * ROWT + wave * 64) >= span) {  // wave-uniform: nothing of the row here
+#pragma unroll
+      for (int k = 0; k < 4; ++k) w[t][k] = 0.0f;
+      continue;
+    }
+    wave_live |= 1u << t;
     float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
     if (pos < span) x = *reinterpret_cast<const float4*>(wgt + base + pos);
     const float xs[4] = {x.x, x.y, x.z, x.w};
@@ -287,6 +293,19 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   uint64_t hb_mask[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) {
+    if (!((wave_live >> t) & 1)) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        dl[t][k] = dh[t][k] = 0;
+        op[t][k] = 0.0f;
+      }
+      hb_mask[t] = 0;
+      if (lane == 0) {
+        s_fh[t][wave] = NONE32;
+        s_lh[t][wave] = 0;
+      }
+      continue;
+    }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int b = t * 4 + k;
@@ -316,10 +335,11 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
     }
   }
   uint64_t total_l, total_h;
-  block_scan2<ROWT, T>(dl, dh, s_ex, sl, sh, total_l, total_h);  // its barrier also publishes s_fh / s_lh
+  block_scan2<ROWT, T>(dl, dh, s_ex, sl, sh, total_l, total_h, wave_live);  // its barrier also publishes s_fh / s_lh
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const uint32_t pos = 4u * (t * ROWT + tid);
+    if (!((wave_live >> t) & 1)) continue;  // slots beyond the row are never searched
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       s_sl[pos + k] = sl[t][k];
@@ -415,7 +435,7 @@ __device__ __forceinline__ u128 block_sum_u128(u128 v, u128* s_tmp) {
 }
 
 __device__ __forceinline__ bool streaming_row(uint32_t off, uint32_t d, uint32_t max_tiles) {
-  return ((off & 3u) + d + 4095u) / 4096u > max_tiles;  // rows the tile-parallel path leaves alone
+  return ((off & 3u) + d + TILED_TILE - 1) / TILED_TILE > max_tiles;  // rows the tile-parallel path leaves alone
 }
 
 __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
@@ -613,9 +633,7 @@ int prepare_build_scratch(uint32_t max_rows) {
   }
   if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, COUNTER_BYTES));
   if (!sc.lds_enabled) {
-    SKY_TRY(enable_big_lds(build_lds_kernel<64, 4>, 64 * 4 * 4 * 16));
-    SKY_TRY(enable_big_lds(build_lds_kernel<256, 4>, 256 * 4 * 4 * 16));
-    SKY_TRY(enable_big_lds(build_lds_kernel<1024, 2>, 1024 * 4 * 2 * 16));
+    SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
     sc.lds_enabled = true;
   }
   return SKY_OK;
@@ -679,10 +697,9 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   SKY_TRY(lds(CLS_LDS_H1, build_lds_kernel<64, 1>, 64, 1, "lds_h1"));
   SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
   SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
-  SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<64, 4>, 64, 4, "lds_w4"));
+  SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<128, 2>, 128, 2, "lds_w4"));
   SKY_TRY(lds(CLS_LDS_B2, build_lds_kernel<256, 2>, 256, 2, "lds_b2"));
-  SKY_TRY(lds(CLS_LDS_B4, build_lds_kernel<256, 4>, 256, 4, "lds_b4"));
-  SKY_TRY(lds(CLS_LDS_X2, build_lds_kernel<1024, 2>, 1024, 2, "lds_x2"));
+  SKY_TRY(lds(CLS_LDS_B4, build_lds_kernel<512, 2>, 512, 2, "lds_b4"));
 
   if (counts[CLS_HUGE]) {
     const uint32_t cnt = counts[CLS_HUGE];

@@ -9,16 +9,25 @@ constexpr uint32_t NONE32 = 0xFFFFFFFFu;
 
 // Inclusive prefixes of two quantities over the slots of a tile held as [Q][4] per thread (slot order:
 // quad q of thread tid, then thread tid + 1; sub-tile q before q + 1).  One barrier.
+// Bit q of `wave_live` (wave-uniform) clear means every value of this wave in sub-tile q is zero:
+// the wave then skips that sub-tile's scan.
 template <int ROWT, int Q>
 __device__ __forceinline__ void block_scan2(const uint64_t (&a)[Q][4], const uint64_t (&b)[Q][4],
                                             uint64_t* __restrict__ s_ex /* [2 * Q * ROWT/64] */,
                                             uint64_t (&oa)[Q][4], uint64_t (&ob)[Q][4], uint64_t& tot_a,
-                                            uint64_t& tot_b) {
+                                            uint64_t& tot_b, uint32_t wave_live = 0xFFFFFFFFu) {
   constexpr int NW = ROWT / 64;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   uint64_t ia[Q], ib[Q];
 #pragma unroll
   for (int q = 0; q < Q; ++q) {
+    if (!((wave_live >> q) & 1)) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) oa[q][k] = ob[q][k] = 0;
+      ia[q] = ib[q] = 0;
+      if (lane == 63) s_ex[(q * NW + wave) * 2] = s_ex[(q * NW + wave) * 2 + 1] = 0;
+      continue;
+    }
     uint64_t ra = 0, rb = 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {

@@ -1,6 +1,6 @@
 // Alias tables of rows too long for one workgroup's LDS, built tile by tile by the whole GPU.
 //
-// A row is cut into tiles of 4096 slots counted from its 16-byte aligned start.  The table is the
+// A row is cut into tiles of 1024 slots counted from its 16-byte aligned start.  The table is the
 // same pure function of the weights as everywhere else (see sky_build.hip); only the evaluation
 // order changes:
 //   tiled_sum_kernel      per tile   exact 128-bit partial sum of the weights
@@ -22,9 +22,10 @@
 namespace sky {
 
 constexpr int TL_T = 256;                // threads per tile
-constexpr int TL_Q = 4;                  // float4 quads per thread
-constexpr int TILE = TL_T * 4 * TL_Q;    // 4096 slots
-constexpr uint32_t TILED_MAX_TILES = 2047;  // tile prefixes of one row must fit the emit kernel's LDS
+constexpr int TL_Q = 1;                  // float4 quads per thread
+constexpr int TILE = TL_T * 4 * TL_Q;    // slots per tile
+static_assert(TILE == (int)TILED_TILE, "tile size is part of the dispatch contract");
+constexpr uint32_t TILED_MAX_TILES = 1u << 22;  // rows of more tiles (4G entries) cannot exist with 32-bit offsets
 
 struct TiledRow {
   uint32_t v, off, d, base, lead, span, ntiles, tile0;  // tile0: first global tile id; prefix arrays start at tile0 + row
@@ -246,12 +247,17 @@ __global__ __launch_bounds__(TL_T) void tiled_totals_kernel(const uint32_t* __re
   }
 }
 
+// first t in [0, nt) with B[t + 1] > key (nt if none)
+__device__ __forceinline__ uint32_t first_tile_above(const uint64_t* B, uint32_t nt, uint64_t key) {
+  return first_greater(B + 1, 0, nt, key);
+}
+
 // Per row: BL[t], BH[t] = deficits / surpluses before tile t (t = 0..ntiles, the last entry is the
 // row total), stored at index tile0 + row + t; nfh[tile] = first heavy in any later tile.
 __global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ rows, uint32_t count,
                                                         const TileTotals* __restrict__ ttot,
                                                         uint64_t* __restrict__ BL, uint64_t* __restrict__ BH,
-                                                        uint32_t* __restrict__ nfh) {
+                                                        uint32_t* __restrict__ nfh, uint4* __restrict__ ranges) {
   const uint32_t r = blockIdx.x;
   if (r >= count) return;
   const uint32_t t0 = rows[r].tile0, nt = rows[r].ntiles;
@@ -304,20 +310,76 @@ __global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ r
     rows[r].total_h = ch;
     rows[r].last_heavy = last;
   }
+  // partner tiles of every tile: lights of tile t (keys in [BL[t], BL[t+1]]) meet the tiles whose surplus
+  // range holds those keys; heavies (y in (BH[t], BH[t+1]]) the tiles whose deficit range holds y
+  __threadfence_block();
+  __syncthreads();
+  const uint64_t* rl = BL + b0;
+  const uint64_t* rh = BH + b0;
+  for (uint32_t t = lane; t < nt; t += 64) {
+    uint4 g;
+    g.x = first_tile_above(rh, nt, rl[t]);
+    g.y = min(first_tile_above(rh, nt, rl[t + 1]), nt - 1);
+    if (rh[t + 1] != rh[t]) {
+      g.z = first_tile_above(rl, nt, rh[t]);
+      g.w = min(first_tile_above(rl, nt, rh[t + 1] - 1), nt - 1);
+    } else {
+      g.z = 1;
+      g.w = 0;
+    }
+    ranges[t0 + t] = g;
+  }
 }
 
 // ---------------------------------------------------------------- pass 3: every entry of a tile
-// first t in [0, nt) with B[t + 1] > key (nt if none)
-__device__ __forceinline__ uint32_t first_tile_above(const uint64_t* B, uint32_t nt, uint64_t key) {
-  return first_greater(B + 1, 0, nt, key);
+// Resolves the own entries of one kind whose key lies in [lo, hi) against the per-slot prefix of tile
+// `pt` held in smem[0..TILE).  OWN_HEAVY = false: lights, key = exclusive deficit prefix, prefix = surplus.
+// OWN_HEAVY = true: heavies, key = y - 1, prefix = deficit.
+template <bool OWN_HEAVY>
+__device__ __forceinline__ void resolve_in_tile(const TiledRow& r, const Ledger& L, const uint64_t* smem, uint32_t pt,
+                                                uint64_t lo, uint64_t hi, uint32_t heavy_mask, uint32_t live_mask,
+                                                const uint32_t (&nh_after)[TL_Q], uint32_t T,
+                                                const uint64_t (&key)[TL_Q][4], float (&op)[TL_Q][4],
+                                                uint32_t (&oa)[TL_Q][4]) {
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q) {
+    uint32_t mine = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int b = q * 4 + k;
+      const bool kind = ((live_mask >> b) & 1) && (((heavy_mask >> b) & 1) != 0) == OWN_HEAVY;
+      if (kind && key[q][k] >= lo && key[q][k] < hi) mine |= 1u << k;
+    }
+    if (!mine) continue;
+    const uint32_t base[4] = {0, 0, 0, 0};
+    uint32_t pos[4];
+    search4(smem, base, key[q], (uint32_t)TILE, pos);
+    if (OWN_HEAVY) {
+      // next heavy after each slot of the quad; the row's last heavy never retires
+      uint32_t nxt = nh_after[q];
+#pragma unroll
+      for (int k = 3; k >= 0; --k) {
+        if (((mine >> k) & 1) && nxt != NONE32) {
+          op[q][k] = residual_prob(L.one + key[q][k] + 1 - smem[pos[k]], L);
+          oa[q][k] = nxt - r.lead;
+        }
+        if ((heavy_mask >> (q * 4 + k)) & 1) nxt = T * TILE + 4u * (q * TL_T + tid) + k;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if ((mine >> k) & 1) oa[q][k] = pt * TILE + pos[k] - r.lead;
+    }
+  }
 }
 
-// One pass over the partner tiles of one kind.  OWN_HEAVY = false: own lights (key = exclusive deficit
-// prefix x) against the surplus prefix of the tiles whose range [B[pt], B[pt+1]) holds x.
-// OWN_HEAVY = true: own heavies (key = y - 1) against the deficit prefix, same range test.
+// One pass over the partner tiles of one kind other than the own tile T: their per-slot prefix is
+// recomputed from the weights into LDS.
 template <bool OWN_HEAVY>
 __device__ __forceinline__ void partner_pass(const TiledRow& r, const Ledger& L, const float* __restrict__ wgt,
-                                             const uint64_t* s_B, uint32_t t_lo, uint32_t t_hi, uint64_t* smem,
+                                             const uint64_t* __restrict__ B, uint32_t t_lo, uint32_t t_hi,
+                                             uint64_t* smem,
                                              uint64_t* s_ex, uint32_t heavy_mask, uint32_t live_mask,
                                              const uint32_t (&nh_after)[TL_Q], uint32_t T,
                                              const uint64_t (&key)[TL_Q][4], float (&op)[TL_Q][4],
@@ -325,8 +387,8 @@ __device__ __forceinline__ void partner_pass(const TiledRow& r, const Ledger& L,
   const int tid = threadIdx.x;
   const uint32_t nt = r.ntiles;
   for (uint32_t pt = t_lo; pt <= t_hi && pt < nt; ++pt) {
-    const uint64_t lo = s_B[pt], hi = s_B[pt + 1];
-    if (hi == lo) continue;
+    const uint64_t lo = B[pt], hi = B[pt + 1];
+    if (hi == lo || pt == T) continue;
     float pw[TL_Q][4];
     load_tile(wgt, r, pt, tid, pw);
     uint64_t pv[TL_Q][4], ps[TL_Q][4];
@@ -338,43 +400,14 @@ __device__ __forceinline__ void partner_pass(const TiledRow& r, const Ledger& L,
         const Entry e = classify(pw[q][k], L);
         pv[q][k] = (in_row(r, idx) && e.heavy != OWN_HEAVY) ? e.amount : 0;
       }
-    __syncthreads();  // searches of the previous partner are done: s_ex and P may be overwritten
+    __syncthreads();  // searches of the previous partner are done: s_ex and the prefix may be overwritten
     block_scan1<TL_T, TL_Q>(pv, s_ex, lo, ps);
 #pragma unroll
     for (int q = 0; q < TL_Q; ++q)
 #pragma unroll
       for (int k = 0; k < 4; ++k) smem[4u * (q * TL_T + tid) + k] = ps[q][k];
     __syncthreads();
-#pragma unroll
-    for (int q = 0; q < TL_Q; ++q) {
-      uint32_t mine = 0;
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int b = q * 4 + k;
-        const bool kind = ((live_mask >> b) & 1) && (((heavy_mask >> b) & 1) != 0) == OWN_HEAVY;
-        if (kind && key[q][k] >= lo && key[q][k] < hi) mine |= 1u << k;
-      }
-      if (!mine) continue;
-      const uint32_t base[4] = {0, 0, 0, 0};
-      uint32_t pos[4];
-      search4(smem, base, key[q], (uint32_t)TILE, pos);
-      if (OWN_HEAVY) {
-        // next heavy after each slot of the quad; the row's last heavy never retires
-        uint32_t nxt = nh_after[q];
-#pragma unroll
-        for (int k = 3; k >= 0; --k) {
-          if (((mine >> k) & 1) && nxt != NONE32) {
-            op[q][k] = residual_prob(L.one + key[q][k] + 1 - smem[pos[k]], L);
-            oa[q][k] = nxt - r.lead;
-          }
-          if ((heavy_mask >> (q * 4 + k)) & 1) nxt = T * TILE + 4u * (q * TL_T + tid) + k;
-        }
-      } else {
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if ((mine >> k) & 1) oa[q][k] = pt * TILE + pos[k] - r.lead;
-      }
-    }
+    resolve_in_tile<OWN_HEAVY>(r, L, smem, pt, lo, hi, heavy_mask, live_mask, nh_after, T, key, op, oa);
   }
 }
 
@@ -383,20 +416,19 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
                                                           const float* __restrict__ wgt,
                                                           const uint64_t* __restrict__ gBL,
                                                           const uint64_t* __restrict__ gBH,
-                                                          const uint32_t* __restrict__ nfh, float* __restrict__ prob,
+                                                          const uint32_t* __restrict__ nfh,
+                                                          const uint4* __restrict__ ranges, float* __restrict__ prob,
                                                           uint32_t* __restrict__ alias,
                                                           int8_t* __restrict__ valid) {
   constexpr int NW = TL_T / 64;
-  extern __shared__ uint64_t smem[];   // [TILE] per-slot prefix of the current partner tile, then BL, BH
-  uint64_t* s_BL = smem + TILE;        // [nt + 1]
+  __shared__ uint64_t smem[TILE];      // per-slot prefix of the current partner tile
   __shared__ uint64_t s_ex[2 * TL_Q * NW];
   __shared__ uint32_t s_fh[TL_Q][NW];
   const uint32_t tile = blockIdx.x;
   const uint32_t ri = tile2row[tile];
   const TiledRow r = rows[ri];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const uint32_t T = tile - r.tile0, nt = r.ntiles;
-  uint64_t* s_BH = s_BL + nt + 1;
+  const uint32_t T = tile - r.tile0;
 
   float w[TL_Q][4];
   load_tile(wgt, r, T, tid, w);
@@ -415,20 +447,19 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
     return;
   }
   const Ledger L = row_ledger(r);
-  const uint32_t b0 = r.tile0 + ri;
-  for (uint32_t i = tid; i <= nt; i += TL_T) {
-    s_BL[i] = gBL[b0 + i];
-    s_BH[i] = gBH[b0 + i];
-  }
+  const uint64_t* BL = gBL + r.tile0 + ri;  // tile prefixes of this row
+  const uint64_t* BH = gBH + r.tile0 + ri;
+  const uint64_t bl = BL[T], bl1 = BL[T + 1], bh = BH[T], bh1 = BH[T + 1];
+  const uint4 rg = ranges[tile];
 
-  // own tile: class and amount of every slot, prefix of the own kind -> search key
-  uint64_t key[TL_Q][4];
+  // own tile: class and amount of every slot, both prefixes, search key of the own kind
+  uint64_t key[TL_Q][4], sl[TL_Q][4], sh[TL_Q][4];
   float op[TL_Q][4];
   uint32_t oa[TL_Q][4];
   uint32_t heavy_mask = 0, live_mask = 0;
   uint64_t hb_mask[TL_Q];
   {
-    uint64_t dl[TL_Q][4], dh[TL_Q][4], sl[TL_Q][4], sh[TL_Q][4];
+    uint64_t dl[TL_Q][4], dh[TL_Q][4];
 #pragma unroll
     for (int q = 0; q < TL_Q; ++q) {
 #pragma unroll
@@ -454,13 +485,15 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
       if (lane == 0) s_fh[q][wave] = fh;
     }
     uint64_t tl, th;
-    block_scan2<TL_T, TL_Q>(dl, dh, s_ex, sl, sh, tl, th);  // its barrier also publishes s_BL / s_BH / s_fh
-    const uint64_t bl = s_BL[T], bh = s_BH[T];
+    block_scan2<TL_T, TL_Q>(dl, dh, s_ex, sl, sh, tl, th);  // its barrier also publishes s_fh
 #pragma unroll
     for (int q = 0; q < TL_Q; ++q)
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        key[q][k] = ((heavy_mask >> (q * 4 + k)) & 1) ? bh + sh[q][k] - 1 : bl + sl[q][k] - dl[q][k];
+      for (int k = 0; k < 4; ++k) {
+        sl[q][k] += bl;
+        sh[q][k] += bh;
+        key[q][k] = ((heavy_mask >> (q * 4 + k)) & 1) ? sh[q][k] - 1 : sl[q][k] - dl[q][k];
+      }
   }
   // next heavy after each quad (span index): later lanes, later waves, later sub-tiles, later tiles
   uint32_t nh_after[TL_Q];
@@ -492,16 +525,24 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
       const bool heavy = (heavy_mask >> (q * 4 + k)) & 1;
       oa[q][k] = (!heavy && r.total_h) ? r.last_heavy - r.lead : idx - r.lead;
     }
+  // the own tile is usually its own main partner, and its prefixes are already in registers
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) smem[4u * (q * TL_T + tid) + k] = sh[q][k];
+  __syncthreads();
+  resolve_in_tile<false>(r, L, smem, T, bh, bh1, heavy_mask, live_mask, nh_after, T, key, op, oa);
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < TL_Q; ++q)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) smem[4u * (q * TL_T + tid) + k] = sl[q][k];
+  __syncthreads();
+  resolve_in_tile<true>(r, L, smem, T, bl, bl1, heavy_mask, live_mask, nh_after, T, key, op, oa);
 
-  // lights: partner tiles are those whose surplus range meets [BL[T], BL[T+1]]
-  partner_pass<false>(r, L, wgt, s_BH, first_tile_above(s_BH, nt, s_BL[T]),
-                      min(first_tile_above(s_BH, nt, s_BL[T + 1]), nt - 1), smem, s_ex, heavy_mask, live_mask,
-                      nh_after, T, key, op, oa);
-  // heavies: y in (BH[T], BH[T+1]] retires in the tile whose deficit range (BL[t], BL[t+1]] holds y
-  if (s_BH[T + 1] != s_BH[T])
-    partner_pass<true>(r, L, wgt, s_BL, first_tile_above(s_BL, nt, s_BH[T]),
-                       min(first_tile_above(s_BL, nt, s_BH[T + 1] - 1), nt - 1), smem, s_ex, heavy_mask, live_mask,
-                       nh_after, T, key, op, oa);
+  // the other partner tiles (ranges precomputed per tile by tiled_scan_kernel)
+  partner_pass<false>(r, L, wgt, BH, rg.x, rg.y, smem, s_ex, heavy_mask, live_mask, nh_after, T, key, op, oa);
+  partner_pass<true>(r, L, wgt, BL, rg.z, rg.w, smem, s_ex, heavy_mask, live_mask, nh_after, T, key, op, oa);
 
 #pragma unroll
   for (int q = 0; q < TL_Q; ++q) {
@@ -532,6 +573,7 @@ struct TiledScratch {
   TileTotals* ttot = nullptr;
   uint64_t *BL = nullptr, *BH = nullptr;
   uint32_t* nfh = nullptr;
+  uint4* ranges = nullptr;
   uint32_t row_cap = 0, tile_cap = 0;
   bool lds_enabled = false;
 };
@@ -557,12 +599,6 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
     sc.row_cap = n;
   }
   if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, 12));
-  if (!sc.lds_enabled) {
-    SKY_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_emit_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)((TILE + 2 * (TILED_MAX_TILES + 1)) * 8)));
-    sc.lds_enabled = true;
-  }
   hipLaunchKernelGGL(tiled_rows_kernel, dim3(1), dim3(1024), 0, st, rows_list, n, g->xadj, g_tiled_max_tiles, sc.rows,
                      sc.totals);
   uint32_t totals[3] = {0, 0, 0};
@@ -572,16 +608,17 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
   *skipped = totals[1];
   if (ntiles == 0) return SKY_OK;
   if (sc.tile_cap < ntiles) {
-    void* olds[] = {sc.tile2row, sc.tsum, sc.ttot, sc.BL, sc.BH, sc.nfh};
+    void* olds[] = {sc.tile2row, sc.tsum, sc.ttot, sc.nfh, sc.ranges};
     for (void* p : olds)
       if (p) SKY_HIP(hipFree(p));
-    sc.tile2row = nullptr; sc.tsum = nullptr; sc.ttot = nullptr; sc.BL = nullptr; sc.BH = nullptr; sc.nfh = nullptr;
+    sc.tile2row = nullptr; sc.tsum = nullptr; sc.ttot = nullptr; sc.nfh = nullptr; sc.ranges = nullptr;
     sc.tile_cap = 0;
     const size_t cap = (size_t)ntiles + ntiles / 4 + 1024;
     SKY_HIP(hipMalloc((void**)&sc.tile2row, cap * 4));
     SKY_HIP(hipMalloc((void**)&sc.tsum, cap * sizeof(u128)));
     SKY_HIP(hipMalloc((void**)&sc.ttot, cap * sizeof(TileTotals)));
     SKY_HIP(hipMalloc((void**)&sc.nfh, cap * 4));
+    SKY_HIP(hipMalloc((void**)&sc.ranges, cap * sizeof(uint4)));
     sc.tile_cap = (uint32_t)cap;
   }
   // prefix arrays hold ntiles + one extra entry per row
@@ -600,10 +637,9 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
   hipLaunchKernelGGL(tiled_sum_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.tsum);
   hipLaunchKernelGGL(tiled_ledger_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.tsum);
   hipLaunchKernelGGL(tiled_totals_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.ttot);
-  hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh);
-  const size_t lds = (size_t)(TILE + 2 * (totals[2] + 1)) * 8;  // partner prefix + the longest row's tile prefixes
-  hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), lds, st, sc.tile2row, sc.rows, g->adjwgt, sc.BL,
-                     sc.BH, sc.nfh, g->prob, g->alias, g->valid);
+  hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh, sc.ranges);
+  hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.BL,
+                     sc.BH, sc.nfh, sc.ranges, g->prob, g->alias, g->valid);
   return SKY_OK;
 }
 

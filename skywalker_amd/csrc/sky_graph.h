@@ -40,12 +40,11 @@ enum BuildClass : int {
   CLS_LDS_H1 = 7,  // deg <= 125       one wavefront, LDS prefix arrays, 4 entries per lane (half the lanes idle)
   CLS_LDS_W1 = 8,  // deg <= 253       one wavefront, 4 entries per lane
   CLS_LDS_W2 = 9,  // deg <= 509       one wavefront, 8 entries per lane
-  CLS_LDS_W4 = 10, // deg <= 1021      one wavefront, 16 entries per lane
+  CLS_LDS_W4 = 10, // deg <= 1021      128 threads, 8 entries per thread
   CLS_LDS_B2 = 11, // deg <= 2045      256 threads, 8 entries per thread
-  CLS_LDS_B4 = 12, // deg <= 4093      256 threads, 16 entries per thread
-  CLS_LDS_X2 = 13, // deg <= 8189      1024 threads, 128 KB of LDS
-  CLS_HUGE = 14,   // above            built tile by tile by the whole GPU
-  CLS_COUNT = 15
+  CLS_LDS_B4 = 12, // deg <= 4093      512 threads, 8 entries per thread
+  CLS_HUGE = 13,   // above            built tile by tile by the whole GPU
+  CLS_COUNT = 14
 };
 
 // Sequence of HIP events on one stream; consecutive marks bracket one kernel (or group).
@@ -65,7 +64,8 @@ int ensure_table_storage(sky_graph* g);
 int prepare_build_scratch(uint32_t max_rows);
 int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm);
 int build_all_tables(sky_graph* g, double* seconds);
-// rows of more than 8189 entries: tile-parallel path, and how many tiles per row it accepts
+// rows of more than 4093 entries: tile-parallel path, and how many tiles per row it accepts
+constexpr uint32_t TILED_TILE = 1024;  // slots per tile of the tile-parallel path
 int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped);
 void set_tiled_max_tiles(uint32_t n);
 uint32_t tiled_max_tiles();

@@ -104,10 +104,10 @@ def test_bad_arguments_are_reported(orc):
 
 @pytest.mark.parametrize("dist", ["lognormal2", "nearequal", "sparse", "fewlights", "fewheavies"])
 def test_rows_built_tile_by_tile(orc, dist):
-    # rows beyond one workgroup's LDS: 3 to 80 tiles of 4096, starts of every alignment
+    # rows beyond one workgroup's LDS: 8 to 320 tiles, starts of every alignment
     from helpers import weights
     rng = np.random.default_rng(21)
-    degs = [8190, 1, 8193, 2, 12288, 3, 12289, 40000, 5, 100001, 330000]
+    degs = [4094, 4097, 7, 5121, 8190, 1, 8193, 2, 12288, 3, 12289, 40000, 5, 100001, 330000]
     xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=4096)
     if dist == "fewlights":      # almost every entry barely heavy, 1 % very light: a light tile spans many partners
         w = np.where(rng.random(len(w)) < 0.01, 0.01, 1.01).astype(np.float32)
@@ -121,9 +121,9 @@ def test_rows_built_tile_by_tile(orc, dist):
 def test_streaming_kernel_for_rows_with_too_many_tiles(orc):
     from skywalker_amd import capi
     rng = np.random.default_rng(22)
-    xadj, adjncy, w = graph_from_degrees([9000, 20000, 3, 70000], rng, "lognormal2", V=4096)
-    capi.set_option("tiled_max_tiles", 3)  # 9000 stays tile-parallel, the other two are streamed
+    xadj, adjncy, w = graph_from_degrees([4100, 9000, 20000, 3, 70000], rng, "lognormal2", V=4096)
+    capi.set_option("tiled_max_tiles", 10)  # up to 9000 (9 tiles) stays tile-parallel, the other two are streamed
     try:
         build_and_compare(orc, xadj, adjncy, w, "streaming")
     finally:
-        capi.set_option("tiled_max_tiles", 2047)
+        capi.set_option("tiled_max_tiles", 1 << 22)
