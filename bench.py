@@ -33,7 +33,7 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
 }
 
 
-def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=400_000_000, walk_sample=65536):
+def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sample=1_000_000):
     """Oracle timed on the host cores, on a bounded sample of the same workload."""
     import numpy as np
     V, E = g.V, g.E

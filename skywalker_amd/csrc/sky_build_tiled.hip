@@ -28,7 +28,7 @@ static_assert(TILE == (int)TILED_TILE, "tile size is part of the dispatch contra
 constexpr uint32_t TILED_MAX_TILES = 1u << 22;  // rows of more tiles (4G entries) cannot exist with 32-bit offsets
 
 struct TiledRow {
-  uint32_t v, off, d, base, lead, span, ntiles, tile0;  // tile0: first global tile id; prefix arrays start at tile0 + row
+  uint32_t v, off, d, base, lead, span, ntiles, tile0, bofs;  // tile0: first tile id; bofs: first slot of the row's BL/BH
   double scale, fs, inv_fs;
   uint64_t one, total_h;
   uint32_t ok, last_heavy;  // last_heavy: span index
@@ -66,70 +66,55 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ wgt, const T
 __device__ __forceinline__ bool in_row(const TiledRow& r, uint32_t idx) { return idx >= r.lead && idx < r.span; }
 
 // ---------------------------------------------------------------- row and tile bookkeeping
-// One block: geometry of every row and the exclusive prefix of the tile counts.  Rows with more
-// than TILED_MAX_TILES tiles get no tiles here (they are left to the streaming kernel).
-__global__ __launch_bounds__(1024) void tiled_rows_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
-                                                          const uint32_t* __restrict__ xadj, uint32_t max_tiles,
-                                                          TiledRow* __restrict__ rows,
-                                                          uint32_t* __restrict__ totals /* [0] tiles, [1] skipped rows, [2] most tiles in a row */) {
-  __shared__ uint32_t s_w[16];
+struct TiledCounters {
+  unsigned long long next;  // low 32 bits: tiles handed out; high 32 bits: rows handed out
+  uint32_t skipped;         // rows with more tiles than the path accepts (left to the streaming kernel)
+  uint32_t pad;
+};
+
+// Geometry of every row; each block reserves a run of tile ids (and of prefix-array slots) for its
+// rows with one atomic.  Tile numbering therefore depends on scheduling; no result does.
+__global__ __launch_bounds__(256) void tiled_rows_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+                                                         const uint32_t* __restrict__ xadj, uint32_t max_tiles,
+                                                         TiledRow* __restrict__ rows,
+                                                         TiledCounters* __restrict__ ctr) {
+  __shared__ uint32_t s_w[4];
+  __shared__ unsigned long long s_base;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  uint32_t carry = 0, skipped = 0, most = 0;
-  for (uint32_t chunk = 0; chunk < count; chunk += 1024) {
-    const uint32_t r = chunk + tid;
-    TiledRow row = {};
-    uint32_t nt = 0;
-    if (r < count) {
-      row.v = vlist[r];
-      row.off = xadj[row.v];
-      row.d = xadj[row.v + 1] - row.off;
-      row.base = row.off & ~3u;
-      row.lead = row.off - row.base;
-      row.span = row.lead + row.d;
-      nt = (row.span + TILE - 1) / TILE;
-      if (nt > max_tiles) {
-        nt = 0;
-        ++skipped;
-      }
-      row.ntiles = nt;
-      most = max(most, nt);
+  const uint32_t r = blockIdx.x * 256u + tid;
+  TiledRow row = {};
+  uint32_t nt = 0;
+  bool skip = false;
+  if (r < count) {
+    row.v = vlist[r];
+    row.off = xadj[row.v];
+    row.d = xadj[row.v + 1] - row.off;
+    row.base = row.off & ~3u;
+    row.lead = row.off - row.base;
+    row.span = row.lead + row.d;
+    nt = (row.span + TILE - 1) / TILE;
+    if (nt > max_tiles) {
+      nt = 0;
+      skip = true;
     }
-    const uint32_t inc = group_scan_u32<64>(nt);
-    __syncthreads();
-    if (lane == 63) s_w[wave] = inc;
-    __syncthreads();
-    uint32_t b = carry, t = 0;
-    for (int k = 0; k < 16; ++k) {
-      if (k == wave) b += t;
-      t += s_w[k];
-    }
-    if (r < count) {
-      row.tile0 = b + inc - nt;
-      rows[r] = row;
-    }
-    carry += t;
+    row.ntiles = nt;
   }
-  // skipped rows: sum over the block
-  for (int m = 32; m >= 1; m >>= 1) {
-    skipped += __shfl_xor((int)skipped, m, 64);
-    most = max(most, (uint32_t)__shfl_xor((int)most, m, 64));
-  }
-  __shared__ uint32_t s_most[16];
+  const uint32_t inc = group_scan_u32<64>(nt);
+  const uint32_t nskip = __popcll(__ballot(skip));
+  if (lane == 63) s_w[wave] = inc;
   __syncthreads();
-  if (lane == 0) {
-    s_w[wave] = skipped;
-    s_most[wave] = most;
+  uint32_t before = 0, total = 0;
+  for (int k = 0; k < 4; ++k) {
+    if (k == wave) before = total;
+    total += s_w[k];
   }
+  if (tid == 0) s_base = atomicAdd(&ctr->next, ((unsigned long long)256u << 32) | total);
+  if (lane == 0 && nskip) atomicAdd(&ctr->skipped, nskip);
   __syncthreads();
-  if (tid == 0) {
-    uint32_t s = 0, mm = 0;
-    for (int k = 0; k < 16; ++k) {
-      s += s_w[k];
-      mm = max(mm, s_most[k]);
-    }
-    totals[0] = carry;
-    totals[1] = s;
-    totals[2] = mm;
+  if (r < count) {
+    row.tile0 = (uint32_t)s_base + before + inc - nt;
+    row.bofs = row.tile0 + (uint32_t)(s_base >> 32) + tid;  // every row owns ntiles + 1 prefix slots
+    rows[r] = row;
   }
 }
 
@@ -263,7 +248,7 @@ __global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ r
   const uint32_t t0 = rows[r].tile0, nt = rows[r].ntiles;
   if (nt == 0 || !rows[r].ok) return;
   const int lane = threadIdx.x;
-  const uint32_t b0 = t0 + r;
+  const uint32_t b0 = rows[r].bofs;
   uint64_t cl = 0, ch = 0;
   uint32_t last = NONE32;
   for (uint32_t c = 0; c < nt; c += 64) {
@@ -447,8 +432,8 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
     return;
   }
   const Ledger L = row_ledger(r);
-  const uint64_t* BL = gBL + r.tile0 + ri;  // tile prefixes of this row
-  const uint64_t* BH = gBH + r.tile0 + ri;
+  const uint64_t* BL = gBL + r.bofs;  // tile prefixes of this row
+  const uint64_t* BH = gBH + r.bofs;
   const uint64_t bl = BL[T], bl1 = BL[T + 1], bh = BH[T], bh1 = BH[T + 1];
   const uint4 rg = ranges[tile];
 
@@ -567,7 +552,7 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
 namespace {
 struct TiledScratch {
   TiledRow* rows = nullptr;
-  uint32_t* totals = nullptr;  // [2]
+  TiledCounters* totals = nullptr;
   uint32_t* tile2row = nullptr;
   u128* tsum = nullptr;
   TileTotals* ttot = nullptr;
@@ -598,14 +583,16 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
     SKY_HIP(hipMalloc((void**)&sc.rows, (size_t)n * sizeof(TiledRow)));
     sc.row_cap = n;
   }
-  if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, 12));
-  hipLaunchKernelGGL(tiled_rows_kernel, dim3(1), dim3(1024), 0, st, rows_list, n, g->xadj, g_tiled_max_tiles, sc.rows,
-                     sc.totals);
-  uint32_t totals[3] = {0, 0, 0};
-  SKY_HIP(hipMemcpyAsync(totals, sc.totals, 12, hipMemcpyDeviceToHost, st));
+  if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, sizeof(TiledCounters)));
+  SKY_HIP(hipMemsetAsync(sc.totals, 0, sizeof(TiledCounters), st));
+  hipLaunchKernelGGL(tiled_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, st, rows_list, n, g->xadj,
+                     g_tiled_max_tiles, sc.rows, sc.totals);
+  TiledCounters totals = {};
+  SKY_HIP(hipMemcpyAsync(&totals, sc.totals, sizeof(totals), hipMemcpyDeviceToHost, st));
   SKY_HIP(hipStreamSynchronize(st));
-  const uint32_t ntiles = totals[0];
-  *skipped = totals[1];
+  const uint32_t ntiles = (uint32_t)totals.next;
+  const uint32_t nslots = (uint32_t)(totals.next >> 32);  // 256 per block of rows
+  *skipped = totals.skipped;
   if (ntiles == 0) return SKY_OK;
   if (sc.tile_cap < ntiles) {
     void* olds[] = {sc.tile2row, sc.tsum, sc.ttot, sc.nfh, sc.ranges};
@@ -623,7 +610,7 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
   }
   // prefix arrays hold ntiles + one extra entry per row
   static size_t b_cap = 0;
-  const size_t b_need = (size_t)ntiles + n;
+  const size_t b_need = (size_t)ntiles + nslots;
   if (b_cap < b_need) {
     if (sc.BL) SKY_HIP(hipFree(sc.BL));
     if (sc.BH) SKY_HIP(hipFree(sc.BH));
