@@ -23,13 +23,22 @@ CONFIGS = {
     "c2": dict(scale=20, ef=16, wkind="unit", wa=0.0, wb=0.0, seed=1, walkers=40000, length=80, ppr=False),
     "c5": dict(scale=26, ef=28, wkind="lognormal", wa=0.0, wb=2.0, seed=5, walkers=1000000, length=80, ppr=True),
 }
+# algorithmic bytes per edge of one launch: read w (4) and write prob + alias (8); the two tiled passes that only
+# read the weights count 4; xadj / valid are per vertex and small
+BYTES_PER_EDGE = {"tiled_sum": 4, "tiled_totals": 4, "bin": 12}
+# HBM bytes per edge measured with rocprofv3 --pmc FETCH_SIZE (x2.0, calibrated on copy_u32_kernel) and WRITE_SIZE
+# (x1.0); see profiles/c5_build_traffic.md
+TRAFFIC_PER_EDGE = {"tiled_emit": 20.8, "tiled_sum": 4.3, "tiled_totals": 4.4, "lds_b2": 12.2, "lds_w2": 12.9,
+                    "lds_w1": 14.7, "wave64": 17.1}
 KERNEL_OF = {  # build_profile entry -> kernel symbol
     "bin": "bin_count_kernel+bin_scatter_kernel", "sub4": "build_subwave_kernel<4>", "sub8": "build_subwave_kernel<8>",
     "sub16": "build_subwave_kernel<16>", "sub32": "build_subwave_kernel<32>", "wave64": "build_subwave_kernel<64>",
     "lds_h1": "build_lds_kernel<64,1> (deg<=125)", "lds_w1": "build_lds_kernel<64,1>",
     "lds_w2": "build_lds_kernel<64,2>", "lds_w4": "build_lds_kernel<128,2>", "lds_b2": "build_lds_kernel<256,2>",
     "lds_b4": "build_lds_kernel<512,2>",
-    "huge": "tiled_*_kernel (rows > 4093)",
+    "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
+    "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
+    "streamed": "huge_prefix_kernel+build_huge_kernel",
 }
 
 
@@ -67,6 +76,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--config", default="c5", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="first run one plain 1 GiB copy kernel (copy_u32_kernel): known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the multi-GPU path of the reference is out of scope); "
@@ -78,6 +89,13 @@ def main():
     import numpy as np
 
     cfg = CONFIGS[args.config]
+    if args.calibrate:
+        words = 1 << 28
+        a = capi.DeviceArray(words, np.uint32, fill=1)
+        b = capi.DeviceArray(words, np.uint32, fill=2)
+        capi.device_copy(b, a, words)
+        a.free()
+        b.free()
     wk = {"uniform": capi.W_UNIFORM, "unit": capi.W_UNIT, "lognormal": capi.W_LOGNORMAL}[cfg["wkind"]]
     name, cus = capi.device_name()
     t_gen = time.perf_counter()
@@ -129,7 +147,7 @@ def main():
             p[0] += ms / len(rec)
     dom = max(prof, key=lambda k: prof[k][0])
     dom_ms, dom_edges = prof[dom]
-    dom_bytes = 12 * dom_edges  # read w, write prob and alias of the class's rows; xadj/valid are per vertex and small
+    dom_bytes = BYTES_PER_EDGE.get(dom, 12) * dom_edges
     out = {
         "metric": "edges/sec over the hot path (alias-table build edges + sampled walk edges) on 1 MI355X",
         "value": work / (ms_per_step * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps,
@@ -143,13 +161,14 @@ def main():
         "build": {"edges_per_s": E / build_s, "ms": build_s * 1e3, "algorithmic_bytes": build_bytes,
                   "hbm_frac": build_bytes / build_s / HBM_PEAK,
                   "kernels": {KERNEL_OF.get(k, k): {"ms": round(v[0], 4), "edges": v[1],
-                                                    "GBps": round(12 * v[1] / (v[0] * 1e-3) / 1e9, 1) if v[0] > 0 else 0}
+                                                    "GBps": round(BYTES_PER_EDGE.get(k, 12) * v[1] / (v[0] * 1e-3) / 1e9, 1) if v[0] > 0 else 0}
                               for k, v in prof.items()}},
         "walk": {"seps": walk_edges / walk_s, "ms": walk_s * 1e3, "steps": walk_edges,
                  "algorithmic_bytes": 24 * walk_edges, "hbm_frac": 24 * walk_edges / walk_s / HBM_PEAK},
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF.get(dom, dom), "achieved": dom_bytes / (dom_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK,
-                     "traffic": None, "launch_ms": dom_ms, "algorithmic_bytes_per_launch": dom_bytes},
+                     "traffic": TRAFFIC_PER_EDGE[dom] * dom_edges if dom in TRAFFIC_PER_EDGE else None,
+                     "launch_ms": dom_ms, "algorithmic_bytes_per_launch": dom_bytes},
     }
     if cfg["ppr"]:
         ppr_s, ppr_edges = mean("ppr_s"), rec[-1]["ppr_edges"]

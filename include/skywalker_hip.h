@@ -56,6 +56,9 @@ int sky_device_free(void* p);
 int sky_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
 int sky_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
 int sky_device_fill_u32(void* dst_device, uint32_t value, size_t count);
+/* Plain device-to-device copy kernel of `count` 32-bit words: the known-size reference for calibrating
+ * HBM traffic counters. */
+int sky_device_copy_u32(void* dst_device, const void* src_device, size_t count);
 int sky_device_synchronize(void);
 int sky_device_name(char* buf, size_t buflen, int* compute_units);
 

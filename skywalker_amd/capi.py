@@ -19,7 +19,7 @@ W_UNIFORM, W_UNIT, W_LOGNORMAL = 0, 1, 2
 
 EXPORTS = [
     "sky_last_error", "sky_version", "sky_device_malloc", "sky_device_free", "sky_memcpy_h2d", "sky_memcpy_d2h",
-    "sky_device_fill_u32", "sky_device_synchronize", "sky_device_name", "sky_graph_upload",
+    "sky_device_fill_u32", "sky_device_copy_u32", "sky_device_synchronize", "sky_device_name", "sky_graph_upload",
     "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
     "sky_alias_build_all", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
     "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_philox_selftest",
@@ -106,6 +106,10 @@ class DeviceArray:
             self.free()
         except Exception:
             pass
+
+
+def device_copy(dst, src, count):
+    _ck(lib().sky_device_copy_u32(dst.ptr, src.ptr, C.c_size_t(count)))
 
 
 def sample_layout(fanout):

@@ -704,7 +704,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   if (counts[CLS_HUGE]) {
     const uint32_t cnt = counts[CLS_HUGE];
     uint32_t skipped = 0;
-    SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_HUGE], cnt, &skipped));
+    SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_HUGE], cnt, &skipped, tm, host.edges[CLS_HUGE]));
     if (skipped) {  // rows with more tiles than the tile-parallel path takes: one workgroup streams each
       const uint32_t max_tiles = tiled_max_tiles();
       if (sc.huge_cap < cnt) {
@@ -731,7 +731,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
                          g->prob, g->alias, g->valid);
     }
   }
-  if (tm) SKY_TRY(tm->mark("huge", host.edges[CLS_HUGE]));
+  if (tm) SKY_TRY(tm->mark("streamed", 0));
   return SKY_OK;
 }
 

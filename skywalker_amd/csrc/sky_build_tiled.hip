@@ -571,7 +571,8 @@ void set_tiled_max_tiles(uint32_t n) { g_tiled_max_tiles = std::min<uint32_t>(st
 
 // Builds the rows of `rows_list` (device, n entries) that have at most the configured number of
 // tiles; *skipped receives how many rows were left for the streaming kernel.
-int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped) {
+int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
+                     uint64_t edges) {
   hipStream_t st = g->stream;
   TiledScratch& sc = g_tiled;
   *skipped = 0;
@@ -621,12 +622,16 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
     b_cap = b_need + b_need / 4 + 1024;
   }
   hipLaunchKernelGGL(tiled_map_kernel, dim3(n), dim3(256), 0, st, sc.rows, n, sc.tile2row);
+  if (tm) SKY_TRY(tm->mark("tiled_rows", 0));
   hipLaunchKernelGGL(tiled_sum_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.tsum);
+  if (tm) SKY_TRY(tm->mark("tiled_sum", edges));
   hipLaunchKernelGGL(tiled_ledger_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.tsum);
   hipLaunchKernelGGL(tiled_totals_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.ttot);
+  if (tm) SKY_TRY(tm->mark("tiled_totals", edges));
   hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh, sc.ranges);
   hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.BL,
                      sc.BH, sc.nfh, sc.ranges, g->prob, g->alias, g->valid);
+  if (tm) SKY_TRY(tm->mark("tiled_emit", edges));
   return SKY_OK;
 }
 

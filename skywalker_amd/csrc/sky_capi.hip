@@ -69,6 +69,21 @@ int sky_device_fill_u32(void* dst, uint32_t value, size_t count) {
   }
   return SKY_OK;
 }
+__global__ void copy_u32_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+int sky_device_copy_u32(void* dst, const void* src, size_t count) {
+  if (count && (!dst || !src)) return fail(SKY_ERR_ARG, "sky_device_copy_u32: null pointer");
+  if (count) {
+    const unsigned grid = (unsigned)std::min<size_t>((count + 255) / 256, 65536);
+    hipLaunchKernelGGL(copy_u32_kernel, dim3(grid), dim3(256), 0, nullptr, (uint32_t*)dst, (const uint32_t*)src,
+                       count);
+    SKY_HIP(hipStreamSynchronize(nullptr));
+    SKY_HIP(hipGetLastError());
+  }
+  return SKY_OK;
+}
 int sky_device_synchronize(void) {
   SKY_HIP(hipDeviceSynchronize());
   return SKY_OK;

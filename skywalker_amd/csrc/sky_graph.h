@@ -66,7 +66,8 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm);
 int build_all_tables(sky_graph* g, double* seconds);
 // rows of more than 4093 entries: tile-parallel path, and how many tiles per row it accepts
 constexpr uint32_t TILED_TILE = 1024;  // slots per tile of the tile-parallel path
-int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped);
+int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
+                     uint64_t edges);
 void set_tiled_max_tiles(uint32_t n);
 uint32_t tiled_max_tiles();
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
