@@ -32,6 +32,14 @@ extern "C" {
 
 typedef struct sky_graph sky_graph;
 
+/* One slot of an alias table: draw col uniformly, keep it when u < prob, else take alias (a row-local index).
+ * The reference keeps two arrays (prob_array, alias_array; include/gpu_graph.cuh:41-43); here the pair is
+ * interleaved so that a draw touches one cache line instead of two. */
+typedef struct sky_alias_entry {
+  float prob;
+  uint32_t alias;
+} sky_alias_entry;
+
 enum sky_status {
   SKY_OK = 0,
   SKY_ERR_ARG = -1,     /* null pointer, zero size, inconsistent CSR */
@@ -75,17 +83,18 @@ int sky_graph_generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph
 int sky_graph_info(const sky_graph* g, uint32_t* V, uint32_t* E, uint32_t* max_degree);
 /* Copies to host; any destination may be NULL. */
 int sky_graph_download(const sky_graph* g, uint32_t* xadj, uint32_t* adjncy, float* adjwgt);
-/* Device addresses of the resident arrays (xadj, adjncy, adjwgt, prob, alias, valid); any output may be NULL. */
+/* Device addresses of the resident arrays (xadj, adjncy, adjwgt, table[E], valid); any output may be NULL. */
 int sky_graph_device_ptrs(const sky_graph* g, const uint32_t** xadj, const uint32_t** adjncy, const float** adjwgt,
-                          const float** prob, const uint32_t** alias, const int8_t** valid);
+                          const sky_alias_entry** table, const int8_t** valid);
 /* Replaces gpu_graph::Free + Sampler::Free (gpu_graph.cuh:164-177, sampler.cuh:65-81). */
 int sky_graph_free(sky_graph* g);
 
 /* ---- offline alias tables for every vertex: replaces ConstructTable(Sampler&, ngpu=1, index=0)
- *      (src/createTable.cu:119-179, kernel :48-108).  Allocates prob[E] f32, alias[E] u32 (row-local
+ *      (src/createTable.cu:119-179, kernel :48-108).  Allocates table[E] ({prob f32, alias u32}: row-local
  *      index, same slot as the CSR edge) and valid[V] i8 inside the graph.  Unlike the reference the
  *      edge weights are kept (createTable.cu:175-177 frees them). ---- */
 int sky_alias_build_all(sky_graph* g, double* seconds);
+/* Copies the table to host as two arrays (any destination may be NULL). */
 int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid);
 /* Installs caller-built tables (host arrays) instead of building: for tests and table persistence. */
 int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, const int8_t* valid);

@@ -82,8 +82,9 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
                                                           const float* __restrict__ wgt,
                                                           const uint32_t* __restrict__ src, uint32_t n,
                                                           uint32_t* __restrict__ cursors,
-                                                          uint32_t* __restrict__ vlist, float* __restrict__ prob,
-                                                          uint32_t* __restrict__ alias, int8_t* __restrict__ valid) {
+                                                          uint32_t* __restrict__ vlist,
+                                                          AliasEntry* __restrict__ table,
+                                                          int8_t* __restrict__ valid) {
   __shared__ uint32_t s_cnt[CLS_COUNT], s_base[CLS_COUNT];
   if (threadIdx.x < CLS_COUNT) s_cnt[threadIdx.x] = 0;
   __syncthreads();
@@ -107,24 +108,20 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
       if (d == 1) {
         const u128 q = weight_fixed(w0);
         const bool ok = (q.lo | q.hi) != 0;
-        prob[off] = ok ? 1.0f : 0.0f;
-        alias[off] = ok ? 0u : SKY_INVALID;
+        table[off] = AliasEntry{ok ? 1.0f : 0.0f, ok ? 0u : SKY_INVALID};
         valid[v] = ok;
       } else {
         const float w1 = clamp_weight(wgt[off + 1]);
         const u128 s = add128(weight_fixed(w0), weight_fixed(w1));
         if ((s.lo | s.hi) == 0) {
-          prob[off] = prob[off + 1] = 0.0f;
-          alias[off] = alias[off + 1] = SKY_INVALID;
+          table[off] = table[off + 1] = AliasEntry{0.0f, SKY_INVALID};
           valid[v] = 0;
         } else {
           const Ledger L = make_ledger(2, s);
           const Entry e0 = classify(w0, L), e1 = classify(w1, L);
           // a lone heavy is the last heavy: it keeps its bucket and tops up the light
-          prob[off] = e0.heavy ? 1.0f : (float)e0.p;
-          prob[off + 1] = e1.heavy ? 1.0f : (float)e1.p;
-          alias[off] = (!e0.heavy && e1.heavy) ? 1u : 0u;
-          alias[off + 1] = (!e1.heavy && e0.heavy) ? 0u : 1u;
+          table[off] = AliasEntry{e0.heavy ? 1.0f : (float)e0.p, (!e0.heavy && e1.heavy) ? 1u : 0u};
+          table[off + 1] = AliasEntry{e1.heavy ? 1.0f : (float)e1.p, (!e1.heavy && e0.heavy) ? 0u : 1u};
           valid[v] = 1;
         }
       }
@@ -148,8 +145,8 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
 template <int G>
 __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
                                                             const uint32_t* __restrict__ xadj,
-                                                            const float* __restrict__ wgt, float* __restrict__ prob,
-                                                            uint32_t* __restrict__ alias,
+                                                            const float* __restrict__ wgt,
+                                                            AliasEntry* __restrict__ table,
                                                             int8_t* __restrict__ valid) {
   __shared__ uint64_t s_sl[256], s_sh[256];
   const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
@@ -207,8 +204,7 @@ __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __re
   }
   if (!row_ok) { out_p = 0.0f; out_a = SKY_INVALID; }
   if (act) {
-    prob[off + gl] = out_p;
-    alias[off + gl] = out_a;
+    table[off + gl] = AliasEntry{out_p, out_a};
   }
   if (gl == 0 && grp < count) valid[v] = row_ok;
 }
@@ -222,8 +218,8 @@ __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __re
 template <int ROWT, int T>
 __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restrict__ vlist,
                                                          const uint32_t* __restrict__ xadj,
-                                                         const float* __restrict__ wgt, float* __restrict__ prob,
-                                                         uint32_t* __restrict__ alias, int8_t* __restrict__ valid) {
+                                                         const float* __restrict__ wgt,
+                                                         AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
   constexpr int CAP = ROWT * 4 * T;
   constexpr int NW = ROWT / 64;
   extern __shared__ uint64_t smem[];
@@ -278,8 +274,7 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
       for (int k = 0; k < 4; ++k)
         if ((live >> (t * 4 + k)) & 1) {
           const uint32_t idx = 4u * (t * ROWT + tid) + k;
-          prob[base + idx] = 0.0f;
-          alias[base + idx] = SKY_INVALID;
+          table[base + idx] = AliasEntry{0.0f, SKY_INVALID};
         }
     if (tid == 0) valid[v] = 0;
     return;
@@ -404,14 +399,12 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
       }
     }
     if (pos >= lead && pos + 4 <= span) {
-      *reinterpret_cast<float4*>(prob + base + pos) = make_float4(op[t][0], op[t][1], op[t][2], op[t][3]);
-      *reinterpret_cast<uint4*>(alias + base + pos) = make_uint4(oa[0], oa[1], oa[2], oa[3]);
+      store_entries4(table + base + pos, op[t], oa);
     } else {
 #pragma unroll
       for (int k = 0; k < 4; ++k)
         if ((live >> (t * 4 + k)) & 1) {
-          prob[base + pos + k] = op[t][k];
-          alias[base + pos + k] = oa[k];
+          table[base + pos + k] = AliasEntry{op[t][k], oa[k]};
         }
     }
   }
@@ -443,8 +436,8 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __re
                                                             const uint64_t* __restrict__ scratch_off,
                                                             const uint32_t* __restrict__ xadj,
                                                             const float* __restrict__ wgt,
-                                                            uint64_t* __restrict__ scratch, float* __restrict__ prob,
-                                                            uint32_t* __restrict__ alias,
+                                                            uint64_t* __restrict__ scratch,
+                                                            AliasEntry* __restrict__ table,
                                                             int8_t* __restrict__ valid) {
   constexpr int NW = HUGE_T / 64;
   __shared__ u128 s_tmp[NW];
@@ -463,8 +456,7 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __re
     sum = block_sum_u128(sum, s_tmp);
     if ((sum.lo | sum.hi) == 0) {
       for (uint32_t i = tid; i < d; i += HUGE_T) {
-        prob[off + i] = 0.0f;
-        alias[off + i] = SKY_INVALID;
+        table[off + i] = AliasEntry{0.0f, SKY_INVALID};
       }
       if (tid == 0) valid[v] = 0;
       continue;
@@ -523,8 +515,7 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __re
           oa = i;
         }
       }
-      prob[off + i] = op;
-      alias[off + i] = oa;
+      table[off + i] = AliasEntry{op, oa};
     }
     if (tid == 0) valid[v] = 1;
     __syncthreads();
@@ -616,8 +607,7 @@ EventTimer::~EventTimer() {
 }
 
 int ensure_table_storage(sky_graph* g) {
-  if (!g->prob) SKY_TRY(alloc_padded(&g->prob, (size_t)g->E));
-  if (!g->alias) SKY_TRY(alloc_padded(&g->alias, (size_t)g->E));
+  if (!g->table) SKY_TRY(alloc_padded(&g->table, (size_t)g->E));
   if (!g->valid) SKY_TRY(alloc_padded(&g->valid, (size_t)g->V));
   return SKY_OK;
 }
@@ -665,7 +655,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     SKY_HIP(hipMemcpyAsync(sc.counters + CLS_COUNT, starts, sizeof(starts), hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL(bin_scatter_kernel, dim3((n + 256 * BIN_ITEMS - 1) / (256 * BIN_ITEMS)), dim3(256), 0, st,
-                       g->xadj, g->adjwgt, src, n, sc.counters + CLS_COUNT, sc.vlist, g->prob, g->alias, g->valid);
+                       g->xadj, g->adjwgt, src, n, sc.counters + CLS_COUNT, sc.vlist, g->table, g->valid);
   }
   if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
   uint32_t* const vlist = sc.vlist;
@@ -675,7 +665,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     if (cnt) {
       const uint32_t per_block = 256 / G;
       hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, st, vlist + starts[cls],
-                         cnt, g->xadj, g->adjwgt, g->prob, g->alias, g->valid);
+                         cnt, g->xadj, g->adjwgt, g->table, g->valid);
     }
     return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
@@ -690,7 +680,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     if (cnt) {
       const size_t bytes = (size_t)rowt * 4 * t * 16;
       hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
-                         g->prob, g->alias, g->valid);
+                         g->table, g->valid);
     }
     return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
@@ -728,7 +718,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       }
       hipLaunchKernelGGL(build_huge_kernel, dim3(std::min<uint32_t>(cnt, 512)), dim3(HUGE_T), 0, st,
                          vlist + starts[CLS_HUGE], cnt, max_tiles, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch,
-                         g->prob, g->alias, g->valid);
+                         g->table, g->valid);
     }
   }
   if (tm) SKY_TRY(tm->mark("streamed", 0));

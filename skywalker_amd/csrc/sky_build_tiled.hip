@@ -402,8 +402,8 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
                                                           const uint64_t* __restrict__ gBL,
                                                           const uint64_t* __restrict__ gBH,
                                                           const uint32_t* __restrict__ nfh,
-                                                          const uint4* __restrict__ ranges, float* __restrict__ prob,
-                                                          uint32_t* __restrict__ alias,
+                                                          const uint4* __restrict__ ranges,
+                                                          AliasEntry* __restrict__ table,
                                                           int8_t* __restrict__ valid) {
   constexpr int NW = TL_T / 64;
   __shared__ uint64_t smem[TILE];      // per-slot prefix of the current partner tile
@@ -424,8 +424,7 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
       for (int k = 0; k < 4; ++k) {
         const uint32_t idx = T * TILE + 4u * (q * TL_T + tid) + k;
         if (in_row(r, idx)) {
-          prob[r.base + idx] = 0.0f;
-          alias[r.base + idx] = SKY_INVALID;
+          table[r.base + idx] = AliasEntry{0.0f, SKY_INVALID};
         }
       }
     if (T == 0 && tid == 0) valid[r.v] = 0;
@@ -534,14 +533,12 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
     const uint32_t pos = T * TILE + 4u * (q * TL_T + tid);
     if (pos >= r.span) continue;
     if (pos >= r.lead && pos + 4 <= r.span) {
-      *reinterpret_cast<float4*>(prob + r.base + pos) = make_float4(op[q][0], op[q][1], op[q][2], op[q][3]);
-      *reinterpret_cast<uint4*>(alias + r.base + pos) = make_uint4(oa[q][0], oa[q][1], oa[q][2], oa[q][3]);
+      store_entries4(table + r.base + pos, op[q], oa[q]);
     } else {
 #pragma unroll
       for (int k = 0; k < 4; ++k)
         if (in_row(r, pos + k)) {
-          prob[r.base + pos + k] = op[q][k];
-          alias[r.base + pos + k] = oa[q][k];
+          table[r.base + pos + k] = AliasEntry{op[q][k], oa[q][k]};
         }
     }
   }
@@ -630,7 +627,7 @@ int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32
   if (tm) SKY_TRY(tm->mark("tiled_totals", edges));
   hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh, sc.ranges);
   hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.BL,
-                     sc.BH, sc.nfh, sc.ranges, g->prob, g->alias, g->valid);
+                     sc.BH, sc.nfh, sc.ranges, g->table, g->valid);
   if (tm) SKY_TRY(tm->mark("tiled_emit", edges));
   return SKY_OK;
 }

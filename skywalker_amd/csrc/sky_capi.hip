@@ -170,20 +170,19 @@ int sky_graph_download(const sky_graph* g, uint32_t* xadj, uint32_t* adjncy, flo
 }
 
 int sky_graph_device_ptrs(const sky_graph* g, const uint32_t** xadj, const uint32_t** adjncy, const float** adjwgt,
-                          const float** prob, const uint32_t** alias, const int8_t** valid) {
+                          const sky_alias_entry** table, const int8_t** valid) {
   if (!g) return fail(SKY_ERR_ARG, "sky_graph_device_ptrs: null graph");
   if (xadj) *xadj = g->xadj;
   if (adjncy) *adjncy = g->adjncy;
   if (adjwgt) *adjwgt = g->adjwgt;
-  if (prob) *prob = g->prob;
-  if (alias) *alias = g->alias;
+  if (table) *table = reinterpret_cast<const sky_alias_entry*>(g->table);
   if (valid) *valid = g->valid;
   return SKY_OK;
 }
 
 int sky_graph_free(sky_graph* g) {
   if (!g) return SKY_OK;
-  void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->prob, g->alias, g->valid};
+  void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->table, g->valid};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   delete g;
@@ -199,19 +198,27 @@ int sky_alias_build_all(sky_graph* g, double* seconds) {
 int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid) {
   if (!g) return fail(SKY_ERR_ARG, "sky_alias_download: null graph");
   if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_alias_download: tables have not been built");
-  if (prob && g->E) SKY_HIP(hipMemcpy(prob, g->prob, (size_t)g->E * 4, hipMemcpyDeviceToHost));
-  if (alias && g->E) SKY_HIP(hipMemcpy(alias, g->alias, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  if ((prob || alias) && g->E) {
+    std::vector<AliasEntry> host(g->E);
+    SKY_HIP(hipMemcpy(host.data(), g->table, (size_t)g->E * sizeof(AliasEntry), hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < g->E; ++i) {
+      if (prob) prob[i] = host[i].prob;
+      if (alias) alias[i] = host[i].alias;
+    }
+  }
   if (valid && g->V) SKY_HIP(hipMemcpy(valid, g->valid, (size_t)g->V, hipMemcpyDeviceToHost));
   return SKY_OK;
 }
 
 int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, const int8_t* valid) {
   if (!g || !prob || !alias || !valid) return fail(SKY_ERR_ARG, "sky_alias_upload: null pointer");
-  if (!g->prob) SKY_TRY(alloc_padded(&g->prob, (size_t)g->E));
-  if (!g->alias) SKY_TRY(alloc_padded(&g->alias, (size_t)g->E));
+  if (!g->table) SKY_TRY(alloc_padded(&g->table, (size_t)g->E));
   if (!g->valid) SKY_TRY(alloc_padded(&g->valid, (size_t)g->V));
-  if (g->E) SKY_HIP(hipMemcpy(g->prob, prob, (size_t)g->E * 4, hipMemcpyHostToDevice));
-  if (g->E) SKY_HIP(hipMemcpy(g->alias, alias, (size_t)g->E * 4, hipMemcpyHostToDevice));
+  if (g->E) {
+    std::vector<AliasEntry> host(g->E);
+    for (size_t i = 0; i < g->E; ++i) host[i] = AliasEntry{prob[i], alias[i]};
+    SKY_HIP(hipMemcpy(g->table, host.data(), (size_t)g->E * sizeof(AliasEntry), hipMemcpyHostToDevice));
+  }
   if (g->V) SKY_HIP(hipMemcpy(g->valid, valid, (size_t)g->V, hipMemcpyHostToDevice));
   g->has_tables = true;
   return SKY_OK;

@@ -155,6 +155,20 @@ __device__ __forceinline__ uint32_t first_greater(const uint64_t* a, uint32_t lo
   return lo;
 }
 
+// ---------------------------------------------------------------- alias table entries
+// The table keeps {prob, alias} of a slot side by side: a draw reads one 8-byte entry, not two
+// arrays (one cache line less per walk step).  Same definition as sky_alias_entry of the C header.
+struct AliasEntry {
+  float prob;
+  uint32_t alias;
+};
+// Four consecutive entries starting at a 32-byte aligned slot, as two 16-byte stores.
+__device__ __forceinline__ void store_entries4(AliasEntry* t, const float (&p)[4], const uint32_t (&a)[4]) {
+  uint4* o = reinterpret_cast<uint4*>(t);
+  o[0] = make_uint4(__float_as_uint(p[0]), a[0], __float_as_uint(p[1]), a[1]);
+  o[1] = make_uint4(__float_as_uint(p[2]), a[2], __float_as_uint(p[3]), a[3]);
+}
+
 // ---------------------------------------------------------------- wave64 primitives
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 

@@ -11,9 +11,8 @@ struct sky_graph {
   uint32_t* xadj = nullptr;    // [V+1]
   uint32_t* adjncy = nullptr;  // [E]
   float* adjwgt = nullptr;     // [E]
-  // alias tables: slot i of the table is CSR slot i; alias holds a row-local index
-  float* prob = nullptr;      // [E]
-  uint32_t* alias = nullptr;  // [E]
+  // alias table: entry i belongs to CSR slot i; alias holds a row-local index
+  sky::AliasEntry* table = nullptr;  // [E] {prob, alias}
   int8_t* valid = nullptr;    // [V]
   bool has_tables = false;
   hipStream_t stream = nullptr;  // null stream, like the reference ("0 stream everywhere")

@@ -44,8 +44,7 @@ __global__ __launch_bounds__(256) void walk_collect_kernel(const uint32_t* __res
 
 __global__ __launch_bounds__(256) void walk_step_kernel(const uint32_t* __restrict__ xadj,
                                                         const uint32_t* __restrict__ adjncy,
-                                                        const float* __restrict__ prob,
-                                                        const uint32_t* __restrict__ alias, uint32_t N, uint32_t len,
+                                                        const AliasEntry* __restrict__ table, uint32_t N, uint32_t len,
                                                         uint32_t s, uint64_t seed, uint32_t* __restrict__ paths,
                                                         uint32_t* __restrict__ lengths) {
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -55,7 +54,8 @@ __global__ __launch_bounds__(256) void walk_step_kernel(const uint32_t* __restri
   const uint32_t v = path[s];
   const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
   const uint32_t col = __umulhi(r.x, deg);
-  const uint32_t cand = u24(r.y) < prob[off + col] ? col : alias[off + col];
+  const AliasEntry e = table[off + col];
+  const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
   if (cand == SKY_INVALID) {
     lengths[i] = s;
     return;
@@ -114,7 +114,7 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
         SKY_HIP(hipStreamSynchronize(st));
         if (cnt[1] == 0) break;  // every walker has stopped
         SKY_TRY(build_rows(g, list, cnt[0], nullptr));
-        hipLaunchKernelGGL(walk_step_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjncy, g->prob, g->alias, N,
+        hipLaunchKernelGGL(walk_step_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjncy, g->table, N,
                            len, s, seed, paths, lengths);
       }
       hipLaunchKernelGGL(sum_lengths_kernel, dim3(std::min<uint32_t>(blocks, 1024)), dim3(256), 0, st, lengths, N,

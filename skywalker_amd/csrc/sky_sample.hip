@@ -30,8 +30,7 @@ __device__ __forceinline__ bool slot_filled(const HopGeom& g, const uint32_t* sl
 
 __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restrict__ xadj,
                                                          const uint32_t* __restrict__ adjncy,
-                                                         const float* __restrict__ prob,
-                                                         const uint32_t* __restrict__ alias, uint64_t total,
+                                                         const AliasEntry* __restrict__ table, uint64_t total,
                                                          HopGeom g, uint64_t seed, uint32_t* __restrict__ data,
                                                          uint32_t* __restrict__ sl,
                                                          unsigned long long* __restrict__ sampled) {
@@ -45,7 +44,7 @@ __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restr
     if (slot_filled(g, sl, si, s)) {
       const uint32_t v = data[si * g.lps + g.off + s];
       const uint32_t o = xadj[v], deg = xadj[v + 1] - o;
-      if (deg != 0 && alias[o] != SKY_INVALID) {
+      if (deg != 0 && table[o].alias != SKY_INVALID) {
         uint32_t* out = data + si * g.lps + g.off_next + s * g.k;
         uint32_t cnt;
         if (g.k >= deg) {
@@ -55,7 +54,8 @@ __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restr
           cnt = g.k;
           const u32x4 r = philox(seed, (uint32_t)si, (uint32_t)(s * g.k + i), g.h, DOM_SAMPLE);
           const uint32_t col = __umulhi(r.x, deg);
-          const uint32_t cand = u24(r.y) < prob[o + col] ? col : alias[o + col];
+          const AliasEntry e = table[o + col];
+          const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
           out[i] = adjncy[o + cand];
         }
         if (i == 0) {
@@ -159,7 +159,7 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
       const uint64_t total = (uint64_t)N * hg.width * hg.k;
       if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");
       hipLaunchKernelGGL(sample_hop_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, g->xadj,
-                         g->adjncy, g->prob, g->alias, total, hg, seed, data, sample_lengths, d_sampled);
+                         g->adjncy, g->table, total, hg, seed, data, sample_lengths, d_sampled);
     }
     SKY_TRY(tm.mark("sample", 0));
     SKY_TRY(tm.finish(nullptr, seconds));

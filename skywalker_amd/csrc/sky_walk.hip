@@ -14,8 +14,8 @@ namespace sky {
 constexpr int WALK_BLOCK = 256;
 
 __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
-    const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy, const float* __restrict__ prob,
-    const uint32_t* __restrict__ alias, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t len,
+    const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
+    const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t len,
     float stop_prob, uint64_t seed, uint32_t* __restrict__ paths, uint32_t* __restrict__ lengths,
     unsigned long long* __restrict__ sampled) {
   const uint32_t i = blockIdx.x * WALK_BLOCK + threadIdx.x;
@@ -30,9 +30,8 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
       const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
       if (deg == 0) break;
       const uint32_t col = __umulhi(r.x, deg);
-      const float pr = prob[off + col];
-      const uint32_t al = alias[off + col];
-      const uint32_t cand = u24(r.y) < pr ? col : al;
+      const AliasEntry e = table[off + col];
+      const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
       if (cand == SKY_INVALID) break;
       v = adjncy[off + cand];
       path[s + 1] = v;
@@ -58,7 +57,7 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   SKY_HIP(hipEventRecord(e0, st));
   if (N)
     hipLaunchKernelGGL(walk_offline_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st, g->xadj,
-                       g->adjncy, g->prob, g->alias, seeds, N, len, stop_prob, seed, paths, lengths, d_sampled);
+                       g->adjncy, g->table, seeds, N, len, stop_prob, seed, paths, lengths, d_sampled);
   SKY_HIP(hipEventRecord(e1, st));
   SKY_HIP(hipStreamSynchronize(st));
   SKY_HIP(hipGetLastError());

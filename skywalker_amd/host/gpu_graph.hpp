@@ -24,8 +24,7 @@ class gpu_graph {
   const vtx_t* adjncy = nullptr;
   const weight_t* adjwgt = nullptr;
   const edge_t* xadj = nullptr;
-  const float* prob_array = nullptr;
-  const uint* alias_array = nullptr;
+  const sky_alias_entry* alias_table = nullptr;  // {prob, alias} per CSR slot (the reference's prob_array / alias_array)
   const int8_t* valid = nullptr;
   edge_t vtx_num = 0, edge_num = 0, avg_degree = 0;
   uint MaxDegree = 0, device_id = 0;
@@ -45,7 +44,7 @@ class gpu_graph {
   }
   // Re-reads the device addresses after the library allocated tables.
   void Refresh() {
-    SKY_RT_CALL(sky_graph_device_ptrs(handle, &xadj, &adjncy, &adjwgt, &prob_array, &alias_array, &valid));
+    SKY_RT_CALL(sky_graph_device_ptrs(handle, &xadj, &adjncy, &adjwgt, &alias_table, &valid));
   }
   void Free() {
     if (handle) SKY_RT_CALL(sky_graph_free(handle));

@@ -139,8 +139,7 @@ class Sampler {
   uint num_seed = 0;
   std::vector<uint> seeds, hops;
   uint hop_num = 0;
-  const float* prob_array = nullptr;
-  const uint* alias_array = nullptr;
+  const sky_alias_entry* alias_table = nullptr;
   const int8_t* valid = nullptr;
   uint device_id = 0;
   size_t sampled_edges = 0;
@@ -206,8 +205,7 @@ inline float ConstructTable(Sampler& sampler, uint ngpu = 1, uint index = 0) {
   double sec = 0;
   SKY_RT_CALL(sky_alias_build_all(sampler.ggraph.handle, &sec));
   sampler.ggraph.Refresh();
-  sampler.prob_array = sampler.ggraph.prob_array;
-  sampler.alias_array = sampler.ggraph.alias_array;
+  sampler.alias_table = sampler.ggraph.alias_table;
   sampler.valid = sampler.ggraph.valid;
   LOG("Construct table time:\t%.6f\n", sec);
   return (float)sec;
