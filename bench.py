@@ -28,8 +28,9 @@ CONFIGS = {
 BYTES_PER_EDGE = {"tiled_sum": 4, "tiled_totals": 4, "bin": 12}
 # HBM bytes per edge measured with rocprofv3 --pmc FETCH_SIZE (x2.0, calibrated on copy_u32_kernel) and WRITE_SIZE
 # (x1.0); see profiles/c5_build_traffic.md
-TRAFFIC_PER_EDGE = {"tiled_emit": 20.8, "tiled_sum": 4.3, "tiled_totals": 4.4, "lds_b2": 12.2, "lds_w2": 12.9,
-                    "lds_w1": 14.7, "wave64": 17.1}
+TRAFFIC_PER_EDGE = {"tiled_emit": 20.8, "tiled_sum": 4.3, "tiled_totals": 4.4, "lds_b2": 12.2, "lds_w2": 12.8,
+                    "lds_w1": 14.5, "wave64": 16.6}
+WALK_TRAFFIC_PER_STEP = 398.6  # walk_offline_kernel, same source
 KERNEL_OF = {  # build_profile entry -> kernel symbol
     "bin": "bin_count_kernel+bin_scatter_kernel", "sub4": "build_subwave_kernel<4>", "sub8": "build_subwave_kernel<8>",
     "sub16": "build_subwave_kernel<16>", "sub32": "build_subwave_kernel<32>", "wave64": "build_subwave_kernel<64>",
@@ -164,7 +165,10 @@ def main():
                                                     "GBps": round(BYTES_PER_EDGE.get(k, 12) * v[1] / (v[0] * 1e-3) / 1e9, 1) if v[0] > 0 else 0}
                               for k, v in prof.items()}},
         "walk": {"seps": walk_edges / walk_s, "ms": walk_s * 1e3, "steps": walk_edges,
-                 "algorithmic_bytes": 24 * walk_edges, "hbm_frac": 24 * walk_edges / walk_s / HBM_PEAK},
+                 "algorithmic_bytes": 24 * walk_edges, "hbm_frac": 24 * walk_edges / walk_s / HBM_PEAK,
+                 # every step gathers three 128-byte lines (xadj, table entry, adjncy): measured 399 B/step
+                 "measured_traffic_bytes_per_step": WALK_TRAFFIC_PER_STEP,
+                 "hbm_frac_measured_traffic": WALK_TRAFFIC_PER_STEP * walk_edges / walk_s / HBM_PEAK},
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF.get(dom, dom), "achieved": dom_bytes / (dom_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK,
                      "traffic": TRAFFIC_PER_EDGE[dom] * dom_edges if dom in TRAFFIC_PER_EDGE else None,
