@@ -21,6 +21,11 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X published
 CONFIGS = {
     "c1": dict(scale=16, ef=16, wkind="uniform", wa=1.0, wb=100.0, seed=42, walkers=4096, length=80, ppr=False),
     "c2": dict(scale=20, ef=16, wkind="unit", wa=0.0, wb=0.0, seed=1, walkers=40000, length=80, ppr=False),
+    # online configurations: tables are built on the fly, nothing is built beforehand
+    "c3": dict(scale=22, ef=32, wkind="lognormal", wa=0.0, wb=1.0, seed=3, walkers=40000, length=0, ppr=False,
+               mode="sage", fanout=[1, 25, 10]),
+    "c4": dict(scale=24, ef=16, wkind="uniform", wa=1.0, wb=100.0, seed=4, walkers=40000, length=80, ppr=False,
+               mode="node2vec", p=2.0, q=0.5),
     "c5": dict(scale=26, ef=28, wkind="lognormal", wa=0.0, wb=2.0, seed=5, walkers=1000000, length=80, ppr=True),
 }
 # algorithmic bytes per edge of one launch: read w (4) and write prob + alias (8); the two tiled passes that only
@@ -70,6 +75,51 @@ def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sa
     }
 
 
+def online_bench(args, cfg, capi, g, seeds, name, cus, t_gen, torch):
+    """Configs 3 and 4: online 2-hop sampling / online node2vec.  A step = one whole batch."""
+    import numpy as np
+    N = cfg["walkers"]
+    if cfg["mode"] == "sage":
+        lps, slen = capi.sample_layout(cfg["fanout"])
+        out = (capi.DeviceArray(N * lps, np.uint32, fill=capi.FILL), capi.DeviceArray(N * slen, np.uint32, fill=0))
+        run = lambda: g.sample_online(seeds, cfg["fanout"], cfg["seed"], out=out)
+        what = "online biased %d-hop sampling, fanout %s, with replacement" % (len(cfg["fanout"]) - 1, cfg["fanout"][1:])
+    else:
+        L = cfg["length"]
+        out = (capi.DeviceArray(N * (L + 1), np.uint32, fill=capi.FILL), capi.DeviceArray(N, np.uint32, fill=0))
+        if args.n2v_table:
+            run = lambda: g.walk_online(capi.BIAS_NODE2VEC, cfg["p"], cfg["q"], seeds, L, 0.0, cfg["seed"], out=out)
+            how = "second-order table built per (walker, step)"
+        else:
+            # every step pays for the first-order tables of the whole graph again, then walks by rejection
+            def run():
+                bsec = g.build_tables()
+                r = g.walk_online(capi.BIAS_NODE2VEC_REJECT, cfg["p"], cfg["q"], seeds, L, 0.0, cfg["seed"], out=out)
+                return r[0], r[1], r[2], r[3] + bsec
+            how = "first-order tables of all rows rebuilt in every step + rejection on them"
+        what = "online node2vec p=%g q=%g, walk length %d (%s)" % (cfg["p"], cfg["q"], L, how)
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    capi.synchronize()
+    t0 = time.perf_counter()
+    rec = [run() for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    capi.synchronize()
+    wall = (time.perf_counter() - t0) / args.steps
+    sampled, ksec = rec[-1][2], sum(r[3] for r in rec) / len(rec)
+    print(json.dumps({
+        "metric": "sampled edges/sec (SEPS) on 1 MI355X", "value": sampled / wall, "unit": "edges/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 tables, u64 fixed-point ledger, u32 indices",
+        "data": "synthetic",
+        "config": {"workload": "%s: R-MAT scale %d ef %d (%d V, %d E), %s weights; %s, %d start vertices" %
+                               (args.config, cfg["scale"], cfg["ef"], g.V, g.E, cfg["wkind"], what, N),
+                   "device": name, "compute_units": cus, "graph_generation_s": t_gen},
+        "sampled_edges": sampled, "kernel_region_ms": ksec * 1e3, "seps_kernel_region": sampled / ksec,
+        "roofline": None, "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -77,6 +127,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--config", default="c5", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--n2v-table", action="store_true",
+                    help="config c4: build the second-order table of every (walker, step) instead of rejection sampling")
     ap.add_argument("--calibrate", action="store_true",
                     help="first run one plain 1 GiB copy kernel (copy_u32_kernel): known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -104,6 +156,8 @@ def main():
     t_gen = time.perf_counter() - t_gen
     V, E, N, L = g.V, g.E, cfg["walkers"], cfg["length"]
     seeds = g.gen_seeds(cfg["seed"], N)
+    if cfg.get("mode") in ("sage", "node2vec"):
+        return online_bench(args, cfg, capi, g, seeds, name, cus, t_gen, torch)
     paths = capi.DeviceArray(N * (L + 1), np.uint32, fill=capi.FILL)
     lengths = capi.DeviceArray(N, np.uint32, fill=0)
     if cfg["ppr"]:

@@ -49,7 +49,10 @@ enum sky_status {
   SKY_ERR_LIMIT = -5    /* size beyond what the entry point supports */
 };
 
-enum sky_bias { SKY_BIAS_STATIC = 0, SKY_BIAS_NODE2VEC = 1 };
+/* SKY_BIAS_NODE2VEC builds the second-order table of every (walker, step) and draws from it, as the reference
+ * does; SKY_BIAS_NODE2VEC_REJECT samples the same law by rejection on the first-order tables (built by the call
+ * when the graph has none): one membership search per trial instead of one per neighbour. */
+enum sky_bias { SKY_BIAS_STATIC = 0, SKY_BIAS_NODE2VEC = 1, SKY_BIAS_NODE2VEC_REJECT = 2 };
 enum sky_weight_kind { SKY_W_UNIFORM = 0, SKY_W_UNIT = 1, SKY_W_LOGNORMAL = 2 };
 
 #define SKY_INVALID 0xFFFFFFFFu /* alias value of rows whose total weight is zero */
@@ -112,7 +115,8 @@ int sky_walk_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uin
 
 /* ---- walk that rebuilds the table of the current vertex at every step: replaces OnlineWalkShMem(Walker&) /
  *      OnlineWalkGMem(Walker&) (src/online_walk.cu:245-327, online_walk_gmem.cu); bias SKY_BIAS_NODE2VEC applies
- *      the second-order factors of src/api/bias_node2vec.cu:15-27 with (p, q). ---- */
+ *      the second-order factors of src/api/bias_node2vec.cu:15-27 with (p, q); SKY_BIAS_NODE2VEC_REJECT reaches
+ *      the same distribution by rejection, the way src/unbiased_walk.cu:14-60 does for unit weights. ---- */
 int sky_walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds_device, uint32_t N,
                     uint32_t len, float stop_prob, uint64_t philox_seed, uint32_t* paths_device,
                     uint32_t* lengths_device, uint64_t* sampled, double* seconds);

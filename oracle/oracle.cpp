@@ -489,6 +489,60 @@ int orc_walk_online(const uint32_t* xadj, const uint32_t* adjncy, const float* w
   return 0;
 }
 
+// node2vec by rejection on the first-order tables (the "second-order rejection" of KnightKing-style
+// walkers; the reference's own unbiased node2vec, src/unbiased_walk.cu:14-60, uses the same idea).
+// Step s of walker i with a previous vertex: trial t draws a candidate from the first-order table of
+// the current vertex with r_t = Philox(seed; i, s, t, DOM_WALK) (t = 0 shares the step's counter with the
+// stop test), cand = u24(r_t[1]) < prob[col] ? col : alias[col], col = mulhi(r_t[0], deg), and accepts
+// it when u24(r_t[3]) * fmax < f(nbr), f = 1/p if nbr is the previous vertex, 1 if adjacent to it, 1/q
+// otherwise, fmax = max(1/p, 1, 1/q).  After 65536 rejections the last candidate is taken.  The law of
+// the accepted neighbour is w * f / sum(w * f), the same as a draw from the second-order table.
+int orc_walk_node2vec_reject(const uint32_t* xadj, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
+                             float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob,
+                             uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled) {
+  const float fp = 1.0f / p, fq = 1.0f / q;
+  const float fmax = std::max(1.0f, std::max(fp, fq));
+  uint64_t total = 0;
+#pragma omp parallel for schedule(dynamic, 64) reduction(+ : total)
+  for (int64_t i = 0; i < (int64_t)N; ++i) {
+    uint32_t* path = paths + (size_t)i * (len + 1);
+    uint32_t v = seeds[i], prev = 0;
+    bool has_prev = false;
+    path[0] = v;
+    uint32_t s = 0;
+    for (; s < len; ++s) {
+      uint32_t r[4];
+      philox(seed, (uint32_t)i, s, 0, DOM_WALK, r);
+      if (stop_prob > 0.0f && u24(r[2]) < stop_prob) break;
+      const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
+      if (deg == 0) break;
+      uint32_t next = 0;
+      bool dead = false;
+      for (uint32_t t = 0;; ++t) {
+        if (t) philox(seed, (uint32_t)i, s, t, DOM_WALK, r);
+        const uint32_t col = mulhi32(r[0], deg);
+        const uint32_t cand = u24(r[1]) < prob[off + col] ? col : alias[off + col];
+        if (cand == ORC_INVALID) { dead = true; break; }
+        next = adjncy[off + cand];
+        if (!has_prev || t >= 65536) break;
+        float f;
+        if (next == prev) f = fp;
+        else if (std::binary_search(adjncy + xadj[prev], adjncy + xadj[prev + 1], next)) f = 1.0f;
+        else f = fq;
+        if (u24(r[3]) * fmax < f) break;
+      }
+      if (dead) break;
+      prev = v; has_prev = true;
+      v = next;
+      path[s + 1] = v;
+    }
+    lengths[i] = s;
+    total += s;
+  }
+  if (sampled) *sampled = total;
+  return 0;
+}
+
 // ---------------------------------------------------------------- k-hop neighbour sampling
 // Layout (sampler_result.cuh:226-260,421-426): per seed, data holds
 // length_per_sample = sum_h prod_{g<=h} fanout[g] vertex ids (fanout[0] = 1 is the seed

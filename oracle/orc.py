@@ -48,6 +48,8 @@ def lib():
                                    _u32p, _u32p, C.POINTER(C.c_uint64)]
     L.orc_walk_online.argtypes = [_u32p, _u32p, _f32p, C.c_int, C.c_float, C.c_float, _u32p, C.c_uint32, C.c_uint32,
                                   C.c_float, C.c_uint64, _u32p, _u32p, C.POINTER(C.c_uint64)]
+    L.orc_walk_node2vec_reject.argtypes = [_u32p, _u32p, _f32p, _u32p, C.c_float, C.c_float, _u32p, C.c_uint32, C.c_uint32,
+                                           C.c_float, C.c_uint64, _u32p, _u32p, C.POINTER(C.c_uint64)]
     L.orc_sample_offline.argtypes = [_u32p, _u32p, _f32p, _u32p, _u32p, C.c_uint32, _u32p, C.c_uint32, C.c_uint64,
                                      _u32p, _u32p, C.POINTER(C.c_uint64)]
     L.orc_sample_online.argtypes = [_u32p, _u32p, _f32p, _u32p, C.c_uint32, _u32p, C.c_uint32, C.c_uint64, _u32p,
@@ -149,6 +151,16 @@ def walk_online(xadj, adjncy, w, bias_kind, p, q, seeds, length, stop_prob, seed
     lib().orc_walk_online(xadj, adjncy, np.ascontiguousarray(w, np.float32), bias_kind, p, q,
                           np.ascontiguousarray(seeds, np.uint32), N, length, stop_prob, seed, paths, lengths,
                           C.byref(sampled))
+    return paths, lengths, sampled.value
+
+
+def walk_node2vec_reject(xadj, adjncy, prob, alias, p, q, seeds, length, stop_prob, seed):
+    N = len(seeds)
+    paths = np.full((N, length + 1), FILL, np.uint32)
+    lengths = np.zeros(N, np.uint32)
+    sampled = C.c_uint64(0)
+    lib().orc_walk_node2vec_reject(xadj, adjncy, prob, alias, p, q, np.ascontiguousarray(seeds, np.uint32), N, length,
+                                   stop_prob, seed, paths, lengths, C.byref(sampled))
     return paths, lengths, sampled.value
 
 

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(HERE, "libskywalker_hip.so")
 
 INVALID = 0xFFFFFFFF
 FILL = 0xFFFFFFFF
-BIAS_STATIC, BIAS_NODE2VEC = 0, 1
+BIAS_STATIC, BIAS_NODE2VEC, BIAS_NODE2VEC_REJECT = 0, 1, 2
 W_UNIFORM, W_UNIT, W_LOGNORMAL = 0, 1, 2
 
 EXPORTS = [

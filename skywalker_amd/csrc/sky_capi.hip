@@ -252,9 +252,9 @@ int sky_walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_
                     uint32_t len, float stop_prob, uint64_t philox_seed, uint32_t* paths_device,
                     uint32_t* lengths_device, uint64_t* sampled, double* seconds) {
   SKY_TRY(check_walk_args("sky_walk_online", g, seeds_device, N, len, stop_prob, paths_device, lengths_device));
-  if (bias_kind != SKY_BIAS_STATIC && bias_kind != SKY_BIAS_NODE2VEC)
+  if (bias_kind != SKY_BIAS_STATIC && bias_kind != SKY_BIAS_NODE2VEC && bias_kind != SKY_BIAS_NODE2VEC_REJECT)
     return fail(SKY_ERR_ARG, "sky_walk_online: unknown bias kind");
-  if (bias_kind == SKY_BIAS_NODE2VEC && !(p > 0.0f && q > 0.0f))
+  if (bias_kind != SKY_BIAS_STATIC && !(p > 0.0f && q > 0.0f))
     return fail(SKY_ERR_ARG, "sky_walk_online: node2vec needs p > 0 and q > 0");
   return walk_online(g, bias_kind, p, q, seeds_device, N, len, stop_prob, philox_seed, paths_device, lengths_device,
                      sampled, seconds);

@@ -74,6 +74,9 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
 int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
                 float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
                 double* seconds);
+int walk_node2vec_reject(sky_graph* g, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
+                         float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
+                         double* seconds);
 int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
                 uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds);
 int generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int weight_kind, float wa, float wb,

@@ -79,6 +79,8 @@ int walk_online_node2vec(sky_graph* g, float p, float q, const uint32_t* seeds, 
 int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
                 float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
                 double* seconds) {
+  if (bias_kind == SKY_BIAS_NODE2VEC_REJECT)
+    return walk_node2vec_reject(g, p, q, seeds, N, len, stop_prob, seed, paths, lengths, sampled, seconds);
   if (bias_kind == SKY_BIAS_NODE2VEC)
     return walk_online_node2vec(g, p, q, seeds, N, len, stop_prob, seed, paths, lengths, sampled, seconds);
   hipStream_t st = g->stream;

@@ -73,4 +73,103 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   return SKY_OK;
 }
 
+// ---------------------------------------------------------------- node2vec by rejection
+// The second-order law of a step, w(v,x) * f(x) with f = 1/p for the previous vertex, 1 for its
+// neighbours and 1/q for the rest (src/api/bias_node2vec.cu:15-27), is sampled without building the
+// step's table: trial t draws a candidate from the first-order table of the current vertex with
+// r_t = Philox(seed; i, s, t, DOM_WALK) (trial 0 shares the counter of the stop test) and keeps it when
+// u24(r_t.w) * fmax < f(candidate), fmax = max(1/p, 1, 1/q); the 65537th candidate is kept whatever
+// it is.  One membership search in the previous vertex's sorted row per trial, instead of one
+// per neighbour of the current vertex.  The reference's unbiased node2vec walker rejects the same way
+// (src/unbiased_walk.cu:14-60).  One walker per lane.
+__device__ __forceinline__ bool row_has(const uint32_t* __restrict__ row, uint32_t n, uint32_t key) {
+  uint32_t lo = 0;
+  while (n > 1) {  // invariant: if key is in the row it is in [lo, lo + n)
+    const uint32_t half = n >> 1;
+    lo = row[lo + half] <= key ? lo + half : lo;
+    n -= half;
+  }
+  return n == 1 && row[lo] == key;
+}
+
+__global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_kernel(
+    const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
+    const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t len, float fp,
+    float fq, float fmax, float stop_prob, uint64_t seed, uint32_t* __restrict__ paths,
+    uint32_t* __restrict__ lengths, unsigned long long* __restrict__ sampled) {
+  const uint32_t i = blockIdx.x * WALK_BLOCK + threadIdx.x;
+  uint32_t s = 0;
+  if (i < N) {
+    uint32_t* path = paths + (size_t)i * (len + 1);
+    uint32_t v = seeds[i], prev = 0, prev_off = 0, prev_deg = 0;
+    path[0] = v;
+    for (; s < len; ++s) {
+      u32x4 r = philox(seed, i, s, 0, DOM_WALK);
+      if (stop_prob > 0.0f && u24(r.z) < stop_prob) break;
+      const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
+      if (deg == 0) break;
+      uint32_t next = 0;
+      bool dead = false;
+      for (uint32_t t = 0;; ++t) {
+        if (t) r = philox(seed, i, s, t, DOM_WALK);
+        const uint32_t col = __umulhi(r.x, deg);
+        const AliasEntry e = table[off + col];
+        const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
+        if (cand == SKY_INVALID) {
+          dead = true;
+          break;
+        }
+        next = adjncy[off + cand];
+        if (s == 0 || t >= 65536u) break;
+        const float f = next == prev ? fp : (row_has(adjncy + prev_off, prev_deg, next) ? 1.0f : fq);
+        if (u24(r.w) * fmax < f) break;
+      }
+      if (dead) break;
+      prev = v;
+      prev_off = off;
+      prev_deg = deg;
+      v = next;
+      path[s + 1] = v;
+    }
+    lengths[i] = s;
+  }
+  unsigned long long t = s;
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) t += shfl_xor_u64(t, m);
+  if ((threadIdx.x & 63) == 0 && t) atomicAdd(sampled, t);
+}
+
+int walk_node2vec_reject(sky_graph* g, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
+                         float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
+                         double* seconds) {
+  hipStream_t st = g->stream;
+  double build_sec = 0;
+  if (!g->has_tables) SKY_TRY(build_all_tables(g, &build_sec));  // first-order tables, built on demand
+  const float fp = 1.0f / p, fq = 1.0f / q;
+  const float fmax = fmaxf(1.0f, fmaxf(fp, fq));
+  unsigned long long* d_sampled = nullptr;
+  auto body = [&]() -> int {
+    SKY_HIP(hipMalloc((void**)&d_sampled, 8));
+    SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
+    EventTimer tm(st);
+    SKY_TRY(tm.mark("start", 0));
+    if (N)
+      hipLaunchKernelGGL(walk_n2v_reject_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st,
+                         g->xadj, g->adjncy, g->table, seeds, N, len, fp, fq, fmax, stop_prob, seed, paths, lengths,
+                         d_sampled);
+    SKY_TRY(tm.mark("walk", 0));
+    double sec = 0;
+    SKY_TRY(tm.finish(nullptr, &sec));
+    SKY_HIP(hipGetLastError());
+    unsigned long long h = 0;
+    SKY_HIP(hipMemcpy(&h, d_sampled, 8, hipMemcpyDeviceToHost));
+    if (sampled) *sampled = h;
+    if (seconds) *seconds = sec + build_sec;
+    return SKY_OK;
+  };
+  const int rc = body();
+  if (d_sampled) (void)hipFree(d_sampled);
+  return rc;
+}
+
 }  // namespace sky

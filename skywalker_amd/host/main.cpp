@@ -22,6 +22,7 @@ DEFINE_int32(weightrange, 2, "generate random weight with range from 0 to ");
 DEFINE_bool(sage, false, "GraphSage");
 DEFINE_bool(deepwalk, false, "deepwalk");
 DEFINE_bool(node2vec, false, "node2vec");
+DEFINE_bool(n2v_table, false, "node2vec: build the second-order table of every step instead of rejection sampling");
 DEFINE_bool(ppr, false, "ppr");
 DEFINE_double(p, 2.0, "hyper-parameter p for node2vec");
 DEFINE_double(q, 0.5, "hyper-parameter q for node2vec");
@@ -91,7 +92,7 @@ int main(int argc, char* argv[]) {
     FLAGS_randomweight = false;
   }
   if (FLAGS_node2vec && !FLAGS_ol) {
-    LOG("node2vec needs a table per step: switching to --ol=1\n");
+    LOG("node2vec is second-order: switching to --ol=1\n");
     FLAGS_ol = true;
   }
   int sample_size = FLAGS_n;

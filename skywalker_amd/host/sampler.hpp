@@ -15,6 +15,7 @@ DECLARE_bool(itl);
 DECLARE_bool(replica);
 DECLARE_bool(printresult);
 DECLARE_bool(node2vec);
+DECLARE_bool(n2v_table);
 DECLARE_double(p);
 DECLARE_double(q);
 DECLARE_double(tp);
@@ -218,7 +219,9 @@ inline float walk_common(Walker& walker, bool online, const char* who) {
   const uint len = walker.result.hop_num - 1;
   const uint* seeds = (const uint*)walker.result.seed_buf.ptr;
   if (online) {
-    SKY_RT_CALL(sky_walk_online(walker.ggraph.handle, FLAGS_node2vec ? SKY_BIAS_NODE2VEC : SKY_BIAS_STATIC,
+    SKY_RT_CALL(sky_walk_online(walker.ggraph.handle, !FLAGS_node2vec  ? SKY_BIAS_STATIC
+                                : FLAGS_n2v_table ? SKY_BIAS_NODE2VEC
+                                                  : SKY_BIAS_NODE2VEC_REJECT,
                                 (float)FLAGS_p, (float)FLAGS_q, seeds, walker.num_seed, len, (float)FLAGS_tp,
                                 (uint64_t)FLAGS_seed, walker.result.data, walker.result.length, &sampled, &sec));
   } else {

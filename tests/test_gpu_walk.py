@@ -145,3 +145,50 @@ def test_node2vec_hub_rows_beyond_the_weight_cache(orc):
     g.free()
     opaths, olengths, osampled = orc.walk_online(xadj, adjncy, w, 1, 2.0, 0.5, seeds, 12, 0.0, 4)
     assert np.array_equal(got[0], opaths) and np.array_equal(got[1], olengths) and sampled == osampled
+
+
+@pytest.mark.parametrize("scale,ef,stop,p,q", [(11, 8, 0.0, 2.0, 0.5), (13, 16, 0.05, 0.25, 4.0), (12, 8, 0.0, 1.0, 1.0)])
+def test_node2vec_rejection_bit_exact(orc, scale, ef, stop, p, q):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(scale, ef, 33)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 33, len(adjncy), 0.0, 1.0)
+    seeds = orc.gen_seeds(3, 1 << scale, 5000)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    # no tables yet: the call builds the first-order tables itself
+    paths, lengths, sampled, _ = g.walk_online(capi.BIAS_NODE2VEC_REJECT, p, q, seeds, 40, stop, 17)
+    got = (paths.to_host((5000, 41)), lengths.to_host())
+    prob, alias, valid = g.tables()
+    g.free()
+    oprob, oalias, ovalid = orc.alias_build(xadj, w)
+    assert np.array_equal(prob.view(np.uint32), oprob.view(np.uint32)) and np.array_equal(alias, oalias)
+    opaths, olengths, osampled = orc.walk_node2vec_reject(xadj, adjncy, oprob, oalias, p, q, seeds, 40, stop, 17)
+    assert np.array_equal(got[1], olengths)
+    assert np.array_equal(got[0], opaths)
+    assert sampled == osampled
+
+
+def test_node2vec_rejection_second_step_law(orc):
+    # exact second-order law on a small graph, sampled on the device
+    from skywalker_amd import capi
+    edges = [(0, 1), (0, 2), (1, 2), (2, 3), (2, 4)]
+    wts = [1.0, 2.0, 3.0, 4.0, 5.0]
+    src = [a for a, b in edges] + [b for a, b in edges]
+    dst = [b for a, b in edges] + [a for a, b in edges]
+    ww = wts + wts
+    order = np.lexsort((dst, src))
+    adjncy = np.array(dst, np.uint32)[order]
+    w = np.array(ww, np.float32)[order]
+    xadj = np.zeros(6, np.uint32)
+    np.add.at(xadj, np.array(src)[order] + 1, 1)
+    xadj = np.cumsum(xadj).astype(np.uint32)
+    p, q, N = 2.0, 0.5, 400000
+    g = capi.Graph.upload(xadj, adjncy, w)
+    paths, lengths, sampled, _ = g.walk_online(capi.BIAS_NODE2VEC_REJECT, p, q, np.zeros(N, np.uint32), 2, 0.0, 9)
+    paths = paths.to_host((N, 3))
+    g.free()
+    sel = paths[:, 1] == 2
+    second = np.bincount(paths[sel, 2], minlength=5)
+    law = np.array([2.0 / p, 3.0, 0.0, 4.0 / q, 5.0 / q])
+    law /= law.sum()
+    assert second[2] == 0 and sampled == 2 * N
+    assert chi_square_p(second[[0, 1, 3, 4]], law[[0, 1, 3, 4]]) > 0.01

@@ -126,6 +126,83 @@ def test_node2vec_p_q_one_is_first_order(orc):
     assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
 
 
+def test_node2vec_rejection_brute_force_law(orc):
+    # same graph and laws as the table-per-step test above, sampled by rejection on the first-order tables
+    edges = [(0, 1), (0, 2), (1, 2), (2, 3), (2, 4)]
+    wts = [1.0, 2.0, 3.0, 4.0, 5.0]
+    xadj, adjncy, w = undirected(edges, 5, wts)
+    prob, alias, valid = orc.alias_build(xadj, w)
+    for p, q in [(2.0, 0.5), (0.25, 4.0)]:
+        N = 400000
+        paths, lengths, sampled = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, p, q, np.zeros(N, np.uint32), 2,
+                                                           0.0, 78)
+        assert np.all(lengths == 2) and sampled == 2 * N
+        first = np.bincount(paths[:, 1], minlength=5)
+        assert chi_square_p(first[[1, 2]], np.array([1.0, 2.0]) / 3.0) > 0.01
+        sel = paths[:, 1] == 2
+        second = np.bincount(paths[sel, 2], minlength=5)
+        law = np.array([2.0 / p, 3.0, 0.0, 4.0 / q, 5.0 / q])
+        law /= law.sum()
+        assert second[2] == 0
+        assert chi_square_p(second[[0, 1, 3, 4]], law[[0, 1, 3, 4]]) > 0.01
+        sel = paths[:, 1] == 1
+        second = np.bincount(paths[sel, 2], minlength=5)
+        law = np.array([1.0 / p, 0, 3.0, 0, 0])
+        law /= law.sum()
+        assert chi_square_p(second[[0, 2]], law[[0, 2]]) > 0.01
+
+
+def test_node2vec_rejection_p_q_one_is_first_order(orc):
+    # f == fmax == 1 for every candidate: trial 0 is always kept, so the walk is the offline walk
+    xadj, adjncy = orc.rmat_csr(9, 8, 2)
+    w = orc.gen_weights(orc.W_UNIFORM, 2, len(adjncy), 1.0, 100.0)
+    prob, alias, valid = orc.alias_build(xadj, w)
+    seeds = orc.gen_seeds(5, 1 << 9, 300)
+    a = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, 1.0, 1.0, seeds, 20, 0.1, 3)
+    b = orc.walk_offline(xadj, adjncy, prob, alias, seeds, 20, 0.1, 3)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]) and a[2] == b[2]
+
+
+def test_node2vec_rejection_and_table_agree_in_law(orc):
+    # third vertex of walks from one seed on a random graph: both node2vec samplers, one chi-square each
+    # against the exact two-step law computed from the weights
+    rng = np.random.default_rng(21)
+    V = 40
+    xadj, adjncy, w = graph_from_degrees(rng.integers(3, 9, V), rng, "lognormal", V=V)
+    # node2vec needs rows sorted by neighbour id and an undirected membership relation is not required
+    for v in range(V):
+        o = np.argsort(adjncy[xadj[v]:xadj[v + 1]], kind="stable")
+        adjncy[xadj[v]:xadj[v + 1]] = adjncy[xadj[v]:xadj[v + 1]][o]
+        w[xadj[v]:xadj[v + 1]] = w[xadj[v]:xadj[v + 1]][o]
+    p, q = 2.0, 0.5
+    law = np.zeros(V)
+    row0 = slice(xadj[0], xadj[1])
+    w0 = np.zeros(V)
+    np.add.at(w0, adjncy[row0], w[row0].astype(np.float64))
+    w0 /= w0.sum()
+    nb0 = set(adjncy[row0].tolist())
+    for v in range(V):
+        if w0[v] == 0:
+            continue
+        sec = np.zeros(V)
+        for e in range(xadj[v], xadj[v + 1]):
+            x = int(adjncy[e])
+            f = 1 / p if x == 0 else (1.0 if x in nb0 else 1 / q)
+            sec[x] += float(w[e]) * f
+        law += w0[v] * sec / sec.sum()
+    N = 300000
+    prob, alias, valid = orc.alias_build(xadj, w)
+    seeds = np.zeros(N, np.uint32)
+    a, la, _ = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, p, q, seeds, 2, 0.0, 5)
+    b, lb, _ = orc.walk_online(xadj, adjncy, w, 1, p, q, seeds, 2, 0.0, 5)
+    assert np.all(la == 2) and np.all(lb == 2)
+    keep = law > 0
+    for paths in (a, b):
+        cnt = np.bincount(paths[:, 2], minlength=V)
+        assert cnt[~keep].sum() == 0
+        assert chi_square_p(cnt[keep], law[keep]) > 0.01
+
+
 def test_sample_layout_and_counts(orc):
     assert orc.sample_layout([1, 25, 10])[:2] == (276, 26)
     assert orc.sample_layout([1, 25, 10])[2] == [0, 1, 26]
