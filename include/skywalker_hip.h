@@ -140,7 +140,9 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
 
 /* ---- tuning knobs (no counterpart in the reference).  "tiled_max_tiles": rows of more than 4093 entries are
  *      built tile by tile (1024 entries per tile) up to this many tiles (default: no limit); longer rows
- *      are streamed by one workgroup each.  Tests lower it to exercise the streaming kernel. ---- */
+ *      are streamed by one workgroup each.  Tests lower it to exercise the streaming kernel.
+ *      "row_merge" (default 1): rows of 62..4093 entries pair lights and heavies by a merge of their prefix
+ *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table. ---- */
 int sky_set_option(const char* name, long value);
 
 /* ---- per-kernel timing of the last sky_alias_build_all on this graph, for roofline reporting:

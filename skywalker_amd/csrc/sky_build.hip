@@ -411,6 +411,195 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   if (tid == 0) valid[v] = 1;
 }
 
+// ---------------------------------------------------------------- one row per workgroup, pairing by merge
+// Same table as build_lds_kernel, reached without a binary search per entry.  Lights and heavies
+// are compacted by rank into one LDS array (inclusive SL of the lights from the front, inclusive
+// SH of the heavies from the back, a sentinel after each).  In the order of the merged sequence,
+// ties heavy first,
+//   the alias of light r is the heavy rank reached when light r - 1 is taken (rank 0 for r = 0),
+//   the light that finishes heavy h is the light rank reached when heavy h is taken,
+// so each thread finds where its share of PER merged elements starts (one diagonal search) and
+// walks it.  The heavy count rides in bits 52..63 of the SH scan: a row of at most 4093 entries
+// keeps its sums below 2^52.
+constexpr uint64_t MERGE_CNT = 1ull << 52;
+constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
+
+template <int ROWT, int T>
+__global__ __launch_bounds__(ROWT) void build_merge_kernel(const uint32_t* __restrict__ vlist,
+                                                           const uint32_t* __restrict__ xadj,
+                                                           const float* __restrict__ wgt,
+                                                           AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
+  constexpr int PER = 4 * T;  // consecutive slots per thread, counted from the row's 16-byte aligned start
+  constexpr int CAP = ROWT * PER;
+  constexpr int NW = ROWT / 64;
+  constexpr uint32_t TOP = CAP + 1;  // heavy h lives at index TOP - h of the value array and of the result array
+  static_assert(CAP <= 4096, "the heavy count shares a 64-bit word with sums below 2^52");
+  extern __shared__ uint64_t smem[];
+  uint64_t* s_v = smem;                                             // [CAP + 2]
+  uint32_t* s_res = reinterpret_cast<uint32_t*>(smem + CAP + 2);  // [CAP + 2]
+  uint32_t* s_hs = s_res + CAP + 2;                                 // [CAP + 2] row-local slot of heavy h
+  __shared__ WSum3 s_wsum[NW];
+  __shared__ uint64_t s_ex[2 * NW];
+
+  const uint32_t v = vlist[blockIdx.x];
+  const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+  const uint32_t base = off & ~3u, lead = off - base, span = lead + d;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t pos0 = (uint32_t)PER * (uint32_t)tid;
+  const bool wave_on = (uint32_t)(PER * 64 * wave) < span;
+
+  double wd[PER];
+  uint32_t live = 0;  // bit j: slot pos0 + j belongs to the row
+  WSum3 sum{0.0, 0.0, 0.0};
+  if (wave_on) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const uint32_t pos = pos0 + 4u * t;
+      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (pos < span) x = *reinterpret_cast<const float4*>(wgt + base + pos);
+      const float xs[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t idx = pos + k;
+        const bool in = idx >= lead && idx < span;
+        if (in) live |= 1u << (t * 4 + k);
+        wd[t * 4 + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
+        wsum3_add(sum, wd[t * 4 + k]);
+      }
+    }
+    sum = group_sum_wsum3<64>(sum);
+  } else {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) wd[j] = 0.0;
+  }
+  if (NW > 1) {
+    if (lane == 0) s_wsum[wave] = sum;
+    __syncthreads();
+    sum = s_wsum[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) {
+      sum.top += s_wsum[i].top;
+      sum.mid += s_wsum[i].mid;
+      sum.low += s_wsum[i].low;
+    }
+  }
+  if (sum.top + sum.mid + sum.low == 0.0) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if ((live >> j) & 1) table[base + pos0 + j] = AliasEntry{0.0f, SKY_INVALID};
+    if (tid == 0) valid[v] = 0;
+    return;
+  }
+  const Ledger L = make_ledger_small(d, wsum3_to_double(sum));
+
+  float op[PER];
+  uint32_t hcnt[PER];  // heavies up to and including this slot
+  uint32_t heavy = 0;
+  uint32_t nh, nl;
+  {
+    uint64_t dl[PER], dh[PER], sl[PER], sh[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const Entry e = classify_small(wd[j], (live >> j) & 1, L);
+      dl[j] = e.heavy ? 0 : e.amount;
+      dh[j] = e.heavy ? (e.amount | MERGE_CNT) : 0;
+      op[j] = (float)e.p;
+      if (e.heavy) heavy |= 1u << j;
+    }
+    uint64_t total_l, total_h;
+    block_scan2_flat<ROWT, PER>(dl, dh, s_ex, sl, sh, total_l, total_h, wave_on);
+    nh = (uint32_t)(total_h >> 52);
+    nl = d - nh;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const uint32_t hc = (uint32_t)(sh[j] >> 52);
+      hcnt[j] = hc;
+      if (!((live >> j) & 1)) continue;
+      const uint32_t li = pos0 + j - lead;
+      const bool hv = (heavy >> j) & 1;
+      s_v[hv ? TOP + 1 - hc : li - hc] = hv ? (sh[j] & (MERGE_CNT - 1)) : sl[j];
+      if (hv) {
+        s_hs[hc - 1] = li;
+        if (hc == 1) s_res[0] = li;  // the first light starts in the first heavy
+      }
+    }
+  }
+  if (tid == 0) {
+    s_v[nl] = ~0ull;
+    s_v[TOP - nh] = ~0ull;
+  }
+  __syncthreads();
+
+  if (nh) {
+    // merged positions [k0, k0 + PER) belong to this thread; a lights and k0 - a heavies come before them
+    const uint32_t k0 = pos0;
+    if (k0 < d) {
+      uint32_t lo = k0 > nh ? k0 - nh : 0u, hi = min(k0, nl);
+      while (lo < hi) {
+        const uint32_t mid = (lo + hi + 1) >> 1;
+        if (s_v[mid - 1] < s_v[TOP - (k0 - mid)]) lo = mid; else hi = mid - 1;
+      }
+      uint32_t a = lo, b = k0 - lo;
+      const uint32_t steps = min((uint32_t)PER, d - k0);
+#pragma unroll
+      for (int s = 0; s < PER; ++s) {
+        if ((uint32_t)s < steps) {
+          const uint64_t va = s_v[a], vb = s_v[TOP - b];
+          if (vb <= va) {
+            s_res[TOP - b] = a;
+            ++b;
+          } else {
+            ++a;
+            if (a < nl) s_res[a] = s_hs[min(b, nh - 1)];
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // heavies, densely by rank: residual probability from the light that finishes them
+    for (uint32_t h = tid; h < nh; h += ROWT) {
+      const uint32_t r = s_res[TOP - h];
+      uint32_t out = MERGE_SELF;
+      if (h + 1 < nh && r < nl) out = __float_as_uint(residual_prob(L.one + s_v[TOP - h] - s_v[r], L));
+      s_res[TOP - h] = out;
+    }
+    __syncthreads();
+  }
+
+  if (pos0 < span) {
+    uint32_t oa[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const uint32_t li = pos0 + j - lead;
+      const uint32_t hc = hcnt[j];
+      oa[j] = li;
+      if (nh && ((live >> j) & 1)) {
+        if ((heavy >> j) & 1) {
+          const uint32_t x = s_res[TOP - (hc - 1)];
+          op[j] = x == MERGE_SELF ? 1.0f : __uint_as_float(x);
+          if (x != MERGE_SELF) oa[j] = s_hs[hc];
+        } else {
+          oa[j] = s_res[li - hc];
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const uint32_t pos = pos0 + 4u * t;
+      if (pos >= lead && pos + 4 <= span) {
+        const float p4[4] = {op[4 * t], op[4 * t + 1], op[4 * t + 2], op[4 * t + 3]};
+        const uint32_t a4[4] = {oa[4 * t], oa[4 * t + 1], oa[4 * t + 2], oa[4 * t + 3]};
+        store_entries4(table + base + pos, p4, a4);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if ((live >> (t * 4 + k)) & 1) table[base + pos + k] = AliasEntry{op[4 * t + k], oa[4 * t + k]};
+      }
+    }
+  }
+  if (tid == 0) valid[v] = 1;
+}
+
 // ---------------------------------------------------------------- rows beyond LDS: global scratch
 // 1024 threads stream one row three times: exact sum; prefix sums written to a scratch
 // region private to the row (16 bytes per slot); searches over that scratch.
@@ -569,6 +758,7 @@ struct BuildScratch {
   bool lds_enabled = false;
 };
 BuildScratch g_scratch;  // reused across builds; one build at a time per process
+bool g_row_merge = true;   // rows of 62..4093 entries: pairing by merge (else one binary search per entry)
 
 template <class K>
 int enable_big_lds(K kernel, size_t bytes) {
@@ -578,6 +768,7 @@ int enable_big_lds(K kernel, size_t bytes) {
 }
 
 }  // namespace
+void set_row_merge(bool on) { g_row_merge = on; }
 
 int EventTimer::mark(const char* name, uint64_t e) {
   hipEvent_t x;
@@ -624,6 +815,7 @@ int prepare_build_scratch(uint32_t max_rows) {
   if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, COUNTER_BYTES));
   if (!sc.lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
+    SKY_TRY(enable_big_lds(build_merge_kernel<512, 2>, 512 * 4 * 2 * 16 + 32));
     sc.lds_enabled = true;
   }
   return SKY_OK;
@@ -684,12 +876,30 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
-  SKY_TRY(lds(CLS_LDS_H1, build_lds_kernel<64, 1>, 64, 1, "lds_h1"));
-  SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
-  SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
-  SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<128, 2>, 128, 2, "lds_w4"));
-  SKY_TRY(lds(CLS_LDS_B2, build_lds_kernel<256, 2>, 256, 2, "lds_b2"));
-  SKY_TRY(lds(CLS_LDS_B4, build_lds_kernel<512, 2>, 512, 2, "lds_b4"));
+  auto mrg = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
+    const uint32_t cnt = counts[cls];
+    if (cnt) {
+      const size_t bytes = (size_t)rowt * 4 * t * 16 + 32;
+      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
+                         g->table, g->valid);
+    }
+    return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
+  };
+  if (g_row_merge) {
+    SKY_TRY(mrg(CLS_LDS_H1, build_merge_kernel<64, 1>, 64, 1, "lds_h1"));
+    SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 1>, 64, 1, "lds_w1"));
+    SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 2>, 64, 2, "lds_w2"));
+    SKY_TRY(mrg(CLS_LDS_W4, build_merge_kernel<128, 2>, 128, 2, "lds_w4"));
+    SKY_TRY(mrg(CLS_LDS_B2, build_merge_kernel<256, 2>, 256, 2, "lds_b2"));
+    SKY_TRY(mrg(CLS_LDS_B4, build_merge_kernel<512, 2>, 512, 2, "lds_b4"));
+  } else {
+    SKY_TRY(lds(CLS_LDS_H1, build_lds_kernel<64, 1>, 64, 1, "lds_h1"));
+    SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
+    SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
+    SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<128, 2>, 128, 2, "lds_w4"));
+    SKY_TRY(lds(CLS_LDS_B2, build_lds_kernel<256, 2>, 256, 2, "lds_b2"));
+    SKY_TRY(lds(CLS_LDS_B4, build_lds_kernel<512, 2>, 512, 2, "lds_b4"));
+  }
 
   if (counts[CLS_HUGE]) {
     const uint32_t cnt = counts[CLS_HUGE];

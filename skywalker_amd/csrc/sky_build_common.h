@@ -68,6 +68,65 @@ __device__ __forceinline__ void block_scan2(const uint64_t (&a)[Q][4], const uin
   tot_b = run_b;
 }
 
+// Inclusive prefixes of two quantities over PER consecutive slots per thread (thread tid owns slots
+// PER * tid ..).  One barrier.  Waves whose `wave_on` is false hold zeros only and skip their scan.
+template <int ROWT, int PER>
+__device__ __forceinline__ void block_scan2_flat(const uint64_t (&a)[PER], const uint64_t (&b)[PER],
+                                                 uint64_t* __restrict__ s_ex /* [2 * ROWT/64] */,
+                                                 uint64_t (&oa)[PER], uint64_t (&ob)[PER], uint64_t& tot_a,
+                                                 uint64_t& tot_b, bool wave_on) {
+  constexpr int NW = ROWT / 64;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  uint64_t ia = 0, ib = 0;
+  if (wave_on) {
+    uint64_t ra = 0, rb = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      ra += a[k];
+      rb += b[k];
+      oa[k] = ra;
+      ob[k] = rb;
+    }
+    ia = group_scan_u64<64>(ra);
+    ib = group_scan_u64<64>(rb);
+    if (NW > 1 && lane == 63) {
+      s_ex[wave * 2] = ia;
+      s_ex[wave * 2 + 1] = ib;
+    }
+    if (NW == 1) {
+      tot_a = shfl_u64(ia, 63);
+      tot_b = shfl_u64(ib, 63);
+    }
+    ia -= ra;
+    ib -= rb;
+  } else {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) oa[k] = ob[k] = 0;
+    if (NW > 1 && lane == 63) s_ex[wave * 2] = s_ex[wave * 2 + 1] = 0;
+    if (NW == 1) tot_a = tot_b = 0;
+  }
+  if (NW > 1) {
+    __syncthreads();
+    uint64_t run_a = 0, run_b = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      if (w == wave) {
+        ia += run_a;
+        ib += run_b;
+      }
+      run_a += s_ex[w * 2];
+      run_b += s_ex[w * 2 + 1];
+    }
+    tot_a = run_a;
+    tot_b = run_b;
+  }
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    oa[k] += ia;
+    ob[k] += ib;
+  }
+}
+
 // For four keys at once: number of entries of the sorted array that starts `base_k` bytes into the LDS
 // block `s` and has n >= 1 entries that are <= key_k.  The first probe narrows the answer to a window
 // of hb = 2^floor(log2 n) entries that ends inside the array, so no later probe needs a bound check.

@@ -315,6 +315,10 @@ int sky_set_option(const char* name, long value) {
     set_tiled_max_tiles((uint32_t)value);
     return SKY_OK;
   }
+  if (!strcmp(name, "row_merge")) {
+    set_row_merge(value != 0);
+    return SKY_OK;
+  }
   return fail(SKY_ERR_ARG, std::string("sky_set_option: unknown option ") + name);
 }
 

@@ -98,6 +98,33 @@ __device__ __forceinline__ double fixed_to_double(u128 s) {
   return hi + lo;
 }
 
+// The same exact sum without 128-bit integer work per entry: floor(w * 2^64) of a clamped weight is
+// top * 2^64 + mid * 2^32 + low with three integers of at most 2^32, here kept as doubles.  Sums of up
+// to 2^20 such terms stay below 2^53, so fp64 additions of them are exact in any order.
+struct WSum3 {
+  double top, mid, low;
+};
+__device__ __forceinline__ void wsum3_add(WSum3& s, double wd /* (double) clamped weight */) {
+  const double top = trunc(wd);
+  const double m = (wd - top) * 4294967296.0;  // exact: wd carries 24 significant bits
+  const double mid = trunc(m);
+  s.top += top;
+  s.mid += mid;
+  s.low += floor((m - mid) * 4294967296.0);
+}
+// double(S) exactly as fixed_to_double gives it for the u128 S = top * 2^64 + mid * 2^32 + low
+// (needs top + carries < 2^53: rows of fewer than 2^20 entries).  Returns 0 for the zero sum.
+__device__ __forceinline__ double wsum3_to_double(const WSum3& s) {
+  const double c0 = floor(s.low * (1.0 / 4294967296.0));
+  const double l0 = s.low - c0 * 4294967296.0;
+  const double m = s.mid + c0;
+  const double c1 = floor(m * (1.0 / 4294967296.0));
+  const double l1 = m - c1 * 4294967296.0;
+  const double hi = s.top + c1;  // = l3 * 2^32 + l2, exact
+  const double lo = l1 * (1.0 / 4294967296.0) + l0 * (1.0 / 18446744073709551616.0);
+  return hi + lo;
+}
+
 // The integer ledger of a row keeps F fraction bits: 40, fewer only for rows of 2^22 entries
 // and more so that the row's prefix sums stay below 2^63.
 struct Ledger {
@@ -134,6 +161,26 @@ __device__ __forceinline__ Entry classify(float w, const Ledger& L) {
   e.heavy = t >= 0.5;
   e.amount = round_to_u64(fmax(e.heavy ? t : -t, 0.0));  // a light with 0 < t < 0.5 has deficit 0
   if (e.heavy && e.amount == 0) e.amount = 1;  // t = 0.5 exactly rounds to even 0: a heavy always has surplus >= 1
+  return e;
+}
+__device__ __forceinline__ Ledger make_ledger_small(uint32_t deg, double sum /* double(S), deg < 2^22 */) {
+  Ledger L;
+  L.scale = (double)deg / sum;
+  L.one = 1ull << 40;
+  L.fs = 1099511627776.0;
+  L.inv_fs = 1.0 / 1099511627776.0;
+  return L;
+}
+// classify for rows of fewer than 2^12 entries (|t| < 2^52, F = 40): same values as classify, fewer
+// instructions.  `in` false gives a light of deficit 0.  fma(p, fs, -fs) == (p - 1) * fs because fs is a
+// power of two; max(t, 1) before rounding == max(rint(t), 1) for a heavy.
+__device__ __forceinline__ Entry classify_small(double wd, bool in, const Ledger& L) {
+  Entry e;
+  e.p = in ? wd * L.scale : 1.0;
+  const double t = fma(e.p, L.fs, -L.fs);
+  e.heavy = t >= 0.5;
+  const double a = fmax(e.heavy ? t : -t, e.heavy ? 1.0 : 0.0);
+  e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) - 0x4330000000000000ull;
   return e;
 }
 __device__ __forceinline__ float residual_prob(uint64_t r_units, const Ledger& L) {
@@ -267,6 +314,29 @@ __device__ __forceinline__ u128 group_sum_u128(u128 v) {
   if (G >= 32) mix([](uint64_t x) { return shfl_xor_u64(x, 16); });
   if (G >= 64) mix([](uint64_t x) { return shfl_xor_u64(x, 32); });
   return v;
+}
+
+// Sum of a double over aligned groups of G lanes; every lane receives the total.
+template <int G>
+__device__ __forceinline__ double group_sum_f64(double v) {
+  auto get = [](double x, auto f) {
+    const uint64_t b = (uint64_t)__double_as_longlong(x);
+    return __longlong_as_double((long long)f(b));
+  };
+  v += get(v, [](uint64_t b) { return dpp0_u64<DPP_QUAD_XOR1, 0xF>(b); });
+  v += get(v, [](uint64_t b) { return dpp0_u64<DPP_QUAD_XOR2, 0xF>(b); });
+  if (G >= 8) v += get(v, [](uint64_t b) { return dpp0_u64<DPP_ROW_HALF_MIRROR, 0xF>(b); });
+  if (G >= 16) v += get(v, [](uint64_t b) { return dpp0_u64<DPP_ROW_MIRROR, 0xF>(b); });
+  if (G >= 32) v += get(v, [](uint64_t b) { return shfl_xor_u64(b, 16); });
+  if (G >= 64) v += get(v, [](uint64_t b) { return shfl_xor_u64(b, 32); });
+  return v;
+}
+template <int G>
+__device__ __forceinline__ WSum3 group_sum_wsum3(WSum3 s) {
+  s.top = group_sum_f64<G>(s.top);
+  s.mid = group_sum_f64<G>(s.mid);
+  s.low = group_sum_f64<G>(s.low);
+  return s;
 }
 
 }  // namespace sky

@@ -68,6 +68,7 @@ constexpr uint32_t TILED_TILE = 1024;  // slots per tile of the tile-parallel pa
 int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
                      uint64_t edges);
 void set_tiled_max_tiles(uint32_t n);
+void set_row_merge(bool on);
 uint32_t tiled_max_tiles();
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
                  uint32_t* paths, uint32_t* lengths, uint64_t* sampled, double* seconds);
