@@ -162,13 +162,14 @@ __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __re
     d = xadj[v + 1] - off;
   }
   const bool act = (uint32_t)gl < d;
-  const float w = act ? clamp_weight(wgt[off + gl]) : 0.0f;
-  const u128 S = group_sum_u128<G>(weight_fixed(w));
-  const bool row_ok = (S.lo | S.hi) != 0;
-  Ledger L = make_ledger(d, S);
+  const double wd = (double)(act ? clamp_weight(wgt[off + gl]) : 0.0f);
+  WSum3 S{0.0, 0.0, 0.0};
+  wsum3_add(S, wd);
+  S = group_sum_wsum3<G>(S);
+  const bool row_ok = S.top + S.mid + S.low != 0.0;
+  Ledger L = make_ledger_small(d, wsum3_to_double(S));
   if (!row_ok) L.scale = 0.0;
-  Entry e = classify(w, L);
-  if (!act) { e.heavy = false; e.amount = 0; }
+  const Entry e = classify_small(wd, act, L);
   const uint64_t SL = group_scan_u64<G>(e.heavy ? 0 : e.amount);
   const uint64_t SH = group_scan_u64<G>(e.heavy ? e.amount : 0);
   s_sl[threadIdx.x] = SL;

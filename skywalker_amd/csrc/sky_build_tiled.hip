@@ -130,24 +130,28 @@ __global__ __launch_bounds__(256) void tiled_map_kernel(const TiledRow* __restri
 __global__ __launch_bounds__(TL_T) void tiled_sum_kernel(const uint32_t* __restrict__ tile2row,
                                                          const TiledRow* __restrict__ rows,
                                                          const float* __restrict__ wgt, u128* __restrict__ tsum) {
-  __shared__ u128 s_w[TL_T / 64];
+  __shared__ WSum3 s_w[TL_T / 64];
   const uint32_t tile = blockIdx.x;
   const TiledRow r = rows[tile2row[tile]];
   const int tid = threadIdx.x;
   float w[TL_Q][4];
   load_tile(wgt, r, tile - r.tile0, tid, w);
-  u128 sum{0, 0};
+  WSum3 sum{0.0, 0.0, 0.0};  // exact: a tile adds at most 1024 limbs below 2^32 + 1
 #pragma unroll
   for (int q = 0; q < TL_Q; ++q)
 #pragma unroll
-    for (int k = 0; k < 4; ++k) sum = add128(sum, weight_fixed(w[q][k]));
-  sum = group_sum_u128<64>(sum);
+    for (int k = 0; k < 4; ++k) wsum3_add(sum, (double)w[q][k]);
+  sum = group_sum_wsum3<64>(sum);
   if ((tid & 63) == 0) s_w[tid >> 6] = sum;
   __syncthreads();
   if (tid == 0) {
-    u128 s = s_w[0];
-    for (int i = 1; i < TL_T / 64; ++i) s = add128(s, s_w[i]);
-    tsum[tile] = s;
+    WSum3 s = s_w[0];
+    for (int i = 1; i < TL_T / 64; ++i) {
+      s.top += s_w[i].top;
+      s.mid += s_w[i].mid;
+      s.low += s_w[i].low;
+    }
+    tsum[tile] = wsum3_to_u128(s);
   }
 }
 
@@ -196,7 +200,7 @@ __global__ __launch_bounds__(TL_T) void tiled_totals_kernel(const uint32_t* __re
     for (int k = 0; k < 4; ++k) {
       const uint32_t idx = t * TILE + 4u * (q * TL_T + tid) + k;
       if (!in_row(r, idx)) continue;
-      const Entry e = classify(w[q][k], L);
+      const Entry e = classify_fast((double)w[q][k], true, L);
       if (e.heavy) {
         su += e.amount;
         fh = min(fh, idx);
@@ -382,8 +386,8 @@ __device__ __forceinline__ void partner_pass(const TiledRow& r, const Ledger& L,
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const uint32_t idx = pt * TILE + 4u * (q * TL_T + tid) + k;
-        const Entry e = classify(pw[q][k], L);
-        pv[q][k] = (in_row(r, idx) && e.heavy != OWN_HEAVY) ? e.amount : 0;
+        const Entry e = classify_fast((double)pw[q][k], in_row(r, idx), L);
+        pv[q][k] = e.heavy != OWN_HEAVY ? e.amount : 0;
       }
     __syncthreads();  // searches of the previous partner are done: s_ex and the prefix may be overwritten
     block_scan1<TL_T, TL_Q>(pv, s_ex, lo, ps);
@@ -449,13 +453,13 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const uint32_t idx = T * TILE + 4u * (q * TL_T + tid) + k;
-        const Entry e = classify(w[q][k], L);
         const bool in = in_row(r, idx);
-        dl[q][k] = (in && !e.heavy) ? e.amount : 0;
-        dh[q][k] = (in && e.heavy) ? e.amount : 0;
+        const Entry e = classify_fast((double)w[q][k], in, L);
+        dl[q][k] = e.heavy ? 0 : e.amount;
+        dh[q][k] = e.heavy ? e.amount : 0;
         op[q][k] = e.heavy ? 1.0f : (float)e.p;
         if (in) live_mask |= 1u << (q * 4 + k);
-        if (in && e.heavy) heavy_mask |= 1u << (q * 4 + k);
+        if (e.heavy) heavy_mask |= 1u << (q * 4 + k);
       }
       const uint32_t m = (heavy_mask >> (q * 4)) & 15u;
       const uint64_t bal = __ballot(m != 0);
