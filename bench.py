@@ -39,13 +39,13 @@ WALK_TRAFFIC_PER_STEP = 398.6  # walk_offline_kernel, same source
 KERNEL_OF = {  # build_profile entry -> kernel symbol
     "bin": "bin_count_kernel+bin_scatter_kernel", "sub4": "build_subwave_kernel<4>", "sub8": "build_subwave_kernel<8>",
     "sub16": "build_subwave_kernel<16>", "sub32": "build_subwave_kernel<32>", "wave64": "build_subwave_kernel<64>",
-    "lds_h1": "build_lds_kernel<64,1> (deg<=125)", "lds_w1": "build_lds_kernel<64,1>",
-    "lds_w2": "build_lds_kernel<64,2>", "lds_w4": "build_lds_kernel<128,2>", "lds_b2": "build_lds_kernel<256,2>",
-    "lds_b4": "build_lds_kernel<512,2>",
+    "lds_h1": "build_merge_kernel<64,1> (deg<=125)", "lds_w1": "build_merge_kernel<64,1>",
+    "lds_w2": "build_merge_kernel<64,2>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
     "streamed": "huge_prefix_kernel+build_huge_kernel",
 }
+KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,2>" % (64 * nw) for nw in range(2, 17)})
 
 
 def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sample=1_000_000):

@@ -160,10 +160,10 @@ class Graph:
         return sec.value
 
     def build_profile(self):
-        names = (C.c_char_p * 32)()
-        ms = (C.c_float * 32)()
-        edges = (C.c_uint64 * 32)()
-        n = lib().sky_last_build_profile(self.h, names, ms, edges, 32)
+        names = (C.c_char_p * 64)()
+        ms = (C.c_float * 64)()
+        edges = (C.c_uint64 * 64)()
+        n = lib().sky_last_build_profile(self.h, names, ms, edges, 64)
         return [(names[i].decode(), float(ms[i]), int(edges[i])) for i in range(n)]
 
     def tables(self):

@@ -41,10 +41,8 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 125) return CLS_LDS_H1;
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
-  if (d <= 1021) return CLS_LDS_W4;
-  if (d <= 2045) return CLS_LDS_B2;
-  if (d <= 4093) return CLS_LDS_B4;
-  return CLS_HUGE;
+  const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
+  return nw <= 16 ? CLS_MW2 + (int)nw - 2 : CLS_HUGE;
 }
 
 // ---------------------------------------------------------------- binning
@@ -434,13 +432,14 @@ __global__ __launch_bounds__(ROWT) void build_merge_kernel(const uint32_t* __res
   constexpr int CAP = ROWT * PER;
   constexpr int NW = ROWT / 64;
   constexpr uint32_t TOP = CAP + 1;  // heavy h lives at index TOP - h of the value array and of the result array
-  static_assert(CAP <= 4096, "the heavy count shares a 64-bit word with sums below 2^52");
+  constexpr bool PACKED = CAP <= 4096;  // the heavy count rides in the SH scan; larger rows scan it separately
+  static_assert(CAP <= 8192, "sums and shifts below assume rows of fewer than 2^13 entries");
   extern __shared__ uint64_t smem[];
   uint64_t* s_v = smem;                                             // [CAP + 2]
   uint32_t* s_res = reinterpret_cast<uint32_t*>(smem + CAP + 2);  // [CAP + 2]
-  uint32_t* s_hs = s_res + CAP + 2;                                 // [CAP + 2] row-local slot of heavy h
+  uint16_t* s_hs = reinterpret_cast<uint16_t*>(s_res + CAP + 2);   // [CAP + 2] row-local slot of heavy h
   __shared__ WSum3 s_wsum[NW];
-  __shared__ uint64_t s_ex[2 * NW];
+  __shared__ uint64_t s_ex[3 * NW];
 
   const uint32_t v = vlist[blockIdx.x];
   const uint32_t off = xadj[v], d = xadj[v + 1] - off;
@@ -501,26 +500,31 @@ __global__ __launch_bounds__(ROWT) void build_merge_kernel(const uint32_t* __res
     uint64_t dl[PER], dh[PER], sl[PER], sh[PER];
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const Entry e = classify_small(wd[j], (live >> j) & 1, L);
+      const Entry e = PACKED ? classify_small(wd[j], (live >> j) & 1, L) : classify_fast(wd[j], (live >> j) & 1, L);
       dl[j] = e.heavy ? 0 : e.amount;
-      dh[j] = e.heavy ? (e.amount | MERGE_CNT) : 0;
+      dh[j] = e.heavy ? (PACKED ? (e.amount | MERGE_CNT) : e.amount) : 0;
       op[j] = (float)e.p;
       if (e.heavy) heavy |= 1u << j;
     }
     uint64_t total_l, total_h;
-    block_scan2_flat<ROWT, PER>(dl, dh, s_ex, sl, sh, total_l, total_h, wave_on);
-    nh = (uint32_t)(total_h >> 52);
+    uint32_t ex_c = 0;
+    if constexpr (PACKED) {
+      block_scan2_flat<ROWT, PER>(dl, dh, s_ex, sl, sh, total_l, total_h, wave_on);
+      nh = (uint32_t)(total_h >> 52);
+    } else {
+      block_scan2c_flat<ROWT, PER>(dl, dh, (uint32_t)__popc(heavy), s_ex, sl, sh, ex_c, total_l, total_h, nh, wave_on);
+    }
     nl = d - nh;
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const uint32_t hc = (uint32_t)(sh[j] >> 52);
+      const uint32_t hc = PACKED ? (uint32_t)(sh[j] >> 52) : ex_c + (uint32_t)__popc(heavy & ((2u << j) - 1));
       hcnt[j] = hc;
       if (!((live >> j) & 1)) continue;
       const uint32_t li = pos0 + j - lead;
       const bool hv = (heavy >> j) & 1;
-      s_v[hv ? TOP + 1 - hc : li - hc] = hv ? (sh[j] & (MERGE_CNT - 1)) : sl[j];
+      s_v[hv ? TOP + 1 - hc : li - hc] = hv ? (PACKED ? (sh[j] & (MERGE_CNT - 1)) : sh[j]) : sl[j];
       if (hv) {
-        s_hs[hc - 1] = li;
+        s_hs[hc - 1] = (uint16_t)li;
         if (hc == 1) s_res[0] = li;  // the first light starts in the first heavy
       }
     }
@@ -816,7 +820,9 @@ int prepare_build_scratch(uint32_t max_rows) {
   if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, COUNTER_BYTES));
   if (!sc.lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
-    SKY_TRY(enable_big_lds(build_merge_kernel<512, 2>, 512 * 4 * 2 * 16 + 32));
+#define SKY_BIG(NW) SKY_TRY(enable_big_lds(build_merge_kernel<64 * NW, 2>, (64 * NW * 8 + 2) * 14))
+    SKY_BIG(10); SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
+#undef SKY_BIG
     sc.lds_enabled = true;
   }
   return SKY_OK;
@@ -880,26 +886,40 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   auto mrg = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
     const uint32_t cnt = counts[cls];
     if (cnt) {
-      const size_t bytes = (size_t)rowt * 4 * t * 16 + 32;
+      const size_t bytes = ((size_t)rowt * 4 * t + 2) * 14;
       hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
                          g->table, g->valid);
     }
     return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
+  static const char* const mw_name[15] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9",
+                                          "mw10", "mw11", "mw12", "mw13", "mw14", "mw15", "mw16"};
   if (g_row_merge) {
     SKY_TRY(mrg(CLS_LDS_H1, build_merge_kernel<64, 1>, 64, 1, "lds_h1"));
     SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 1>, 64, 1, "lds_w1"));
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 2>, 64, 2, "lds_w2"));
-    SKY_TRY(mrg(CLS_LDS_W4, build_merge_kernel<128, 2>, 128, 2, "lds_w4"));
-    SKY_TRY(mrg(CLS_LDS_B2, build_merge_kernel<256, 2>, 256, 2, "lds_b2"));
-    SKY_TRY(mrg(CLS_LDS_B4, build_merge_kernel<512, 2>, 512, 2, "lds_b4"));
+#define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 2>, 64 * NW, 2, mw_name[NW - 2]))
+    SKY_MW(2); SKY_MW(3); SKY_MW(4); SKY_MW(5); SKY_MW(6); SKY_MW(7); SKY_MW(8); SKY_MW(9);
+    SKY_MW(10); SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
+#undef SKY_MW
   } else {
     SKY_TRY(lds(CLS_LDS_H1, build_lds_kernel<64, 1>, 64, 1, "lds_h1"));
     SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
     SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
-    SKY_TRY(lds(CLS_LDS_W4, build_lds_kernel<128, 2>, 128, 2, "lds_w4"));
-    SKY_TRY(lds(CLS_LDS_B2, build_lds_kernel<256, 2>, 256, 2, "lds_b2"));
-    SKY_TRY(lds(CLS_LDS_B4, build_lds_kernel<512, 2>, 512, 2, "lds_b4"));
+    for (int nw = 2; nw <= 16; ++nw) {
+      const int cls = CLS_MW2 + nw - 2;
+      if (nw <= 2) SKY_TRY(lds(cls, build_lds_kernel<128, 2>, 128, 2, mw_name[nw - 2]));
+      else if (nw <= 4) SKY_TRY(lds(cls, build_lds_kernel<256, 2>, 256, 2, mw_name[nw - 2]));
+      else if (nw <= 8) SKY_TRY(lds(cls, build_lds_kernel<512, 2>, 512, 2, mw_name[nw - 2]));
+      else {  // this variant has no kernel for rows of 4094..8189 entries: tile-parallel path
+        if (counts[cls]) {
+          uint32_t skipped = 0;
+          SKY_TRY(build_rows_tiled(g, vlist + starts[cls], counts[cls], &skipped, nullptr, 0));
+          if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles below 9 needs row_merge");
+        }
+        if (tm) SKY_TRY(tm->mark(mw_name[nw - 2], host.edges[cls]));
+      }
+    }
   }
 
   if (counts[CLS_HUGE]) {

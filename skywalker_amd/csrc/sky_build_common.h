@@ -127,6 +127,67 @@ __device__ __forceinline__ void block_scan2_flat(const uint64_t (&a)[PER], const
   }
 }
 
+// block_scan2_flat plus an exclusive prefix (and total) of one 32-bit count per thread, same barrier.
+template <int ROWT, int PER>
+__device__ __forceinline__ void block_scan2c_flat(const uint64_t (&a)[PER], const uint64_t (&b)[PER], uint32_t c,
+                                                  uint64_t* __restrict__ s_ex /* [3 * ROWT/64] */,
+                                                  uint64_t (&oa)[PER], uint64_t (&ob)[PER], uint32_t& ex_c,
+                                                  uint64_t& tot_a, uint64_t& tot_b, uint32_t& tot_c, bool wave_on) {
+  constexpr int NW = ROWT / 64;
+  static_assert(NW > 1, "multi-wave rows only");
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  uint64_t ia = 0, ib = 0;
+  uint32_t ic = 0;
+  if (wave_on) {
+    uint64_t ra = 0, rb = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      ra += a[k];
+      rb += b[k];
+      oa[k] = ra;
+      ob[k] = rb;
+    }
+    ia = group_scan_u64<64>(ra);
+    ib = group_scan_u64<64>(rb);
+    ic = group_scan_u32<64>(c);
+    if (lane == 63) {
+      s_ex[wave * 3] = ia;
+      s_ex[wave * 3 + 1] = ib;
+      s_ex[wave * 3 + 2] = ic;
+    }
+    ia -= ra;
+    ib -= rb;
+    ic -= c;
+  } else {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) oa[k] = ob[k] = 0;
+    if (lane == 63) s_ex[wave * 3] = s_ex[wave * 3 + 1] = s_ex[wave * 3 + 2] = 0;
+  }
+  __syncthreads();
+  uint64_t run_a = 0, run_b = 0;
+  uint32_t run_c = 0;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) {
+    if (w == wave) {
+      ia += run_a;
+      ib += run_b;
+      ic += run_c;
+    }
+    run_a += s_ex[w * 3];
+    run_b += s_ex[w * 3 + 1];
+    run_c += (uint32_t)s_ex[w * 3 + 2];
+  }
+  tot_a = run_a;
+  tot_b = run_b;
+  tot_c = run_c;
+  ex_c = ic;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    oa[k] += ia;
+    ob[k] += ib;
+  }
+}
+
 // For four keys at once: number of entries of the sorted array that starts `base_k` bytes into the LDS
 // block `s` and has n >= 1 entries that are <= key_k.  The first probe narrows the answer to a window
 // of hb = 2^floor(log2 n) entries that ends inside the array, so no later probe needs a bound check.

@@ -39,11 +39,10 @@ enum BuildClass : int {
   CLS_LDS_H1 = 7,  // deg <= 125       one wavefront, LDS prefix arrays, 4 entries per lane (half the lanes idle)
   CLS_LDS_W1 = 8,  // deg <= 253       one wavefront, 4 entries per lane
   CLS_LDS_W2 = 9,  // deg <= 509       one wavefront, 8 entries per lane
-  CLS_LDS_W4 = 10, // deg <= 1021      128 threads, 8 entries per thread
-  CLS_LDS_B2 = 11, // deg <= 2045      256 threads, 8 entries per thread
-  CLS_LDS_B4 = 12, // deg <= 4093      512 threads, 8 entries per thread
-  CLS_HUGE = 13,   // above            built tile by tile by the whole GPU
-  CLS_COUNT = 14
+  CLS_MW2 = 10,    // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
+  CLS_MW16 = 24,   //                  class CLS_MW2 + nw - 2
+  CLS_HUGE = 25,   // deg > 8189       built tile by tile by the whole GPU
+  CLS_COUNT = 26
 };
 
 // Sequence of HIP events on one stream; consecutive marks bracket one kernel (or group).

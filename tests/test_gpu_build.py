@@ -127,3 +127,18 @@ def test_streaming_kernel_for_rows_with_too_many_tiles(orc):
         build_and_compare(orc, xadj, adjncy, w, "streaming")
     finally:
         capi.set_option("tiled_max_tiles", 1 << 22)
+
+
+def test_search_variant_of_the_row_kernels_gives_the_same_table(orc):
+    # "row_merge" = 0 selects the kernels that do one binary search per entry (rows of 62..4093 entries) and
+    # sends rows of 4094..8189 entries down the tile-parallel path
+    from skywalker_amd import capi
+    rng = np.random.default_rng(23)
+    degs = [70, 126, 254, 300, 509, 510, 1021, 1500, 2046, 3000, 4093, 4094, 5000, 8189, 8190, 3, 0, 1]
+    xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=8192)
+    capi.set_option("row_merge", 0)
+    try:
+        build_and_compare(orc, xadj, adjncy, w, "row_merge=0")
+    finally:
+        capi.set_option("row_merge", 1)
+    build_and_compare(orc, xadj, adjncy, w, "row_merge=1")
