@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
                                                           const float* __restrict__ wgt,
                                                           const uint32_t* __restrict__ src, uint32_t n,
                                                           uint32_t* __restrict__ cursors,
-                                                          uint32_t* __restrict__ vlist,
+                                                          RowRef* __restrict__ vlist,
                                                           AliasEntry* __restrict__ table,
                                                           int8_t* __restrict__ valid) {
   __shared__ uint32_t s_cnt[CLS_COUNT], s_base[CLS_COUNT];
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
   __syncthreads();
   const uint32_t chunk = blockIdx.x * (256u * BIN_ITEMS);
   int cls[BIN_ITEMS];
-  uint32_t rank[BIN_ITEMS], vtx[BIN_ITEMS];
+  uint32_t rank[BIN_ITEMS], vtx[BIN_ITEMS], offs[BIN_ITEMS], degs[BIN_ITEMS];
 #pragma unroll
   for (int i = 0; i < BIN_ITEMS; ++i) {
     const uint32_t item = chunk + i * 256u + threadIdx.x;
@@ -97,6 +97,8 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
     const uint32_t v = src ? src[item] : item;
     vtx[i] = v;
     const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+    offs[i] = off;
+    degs[i] = d;
     const int c = degree_class(d);
     cls[i] = c;
     if (c == CLS_EMPTY) {
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < BIN_ITEMS; ++i) {
-    if (cls[i] >= CLS_SUB4) vlist[s_base[cls[i]] + rank[i]] = vtx[i];
+    if (cls[i] >= CLS_SUB4) vlist[s_base[cls[i]] + rank[i]] = RowRef{vtx[i], offs[i], degs[i], 0};
   }
 }
 
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
 // One table entry per lane.  Prefix sums run over the group with shuffles; the two
 // searches read the group's strip of a per-wave LDS array.
 template <int G>
-__global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+__global__ __launch_bounds__(256) void build_subwave_kernel(const RowRef* __restrict__ vlist, uint32_t count,
                                                             const uint32_t* __restrict__ xadj,
                                                             const float* __restrict__ wgt,
                                                             AliasEntry* __restrict__ table,
@@ -155,9 +157,10 @@ __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __re
   const int gb = threadIdx.x - gl;         // first LDS slot of the group
   uint32_t v = 0, off = 0, d = 0;
   if (grp < count) {
-    v = vlist[grp];
-    off = xadj[v];
-    d = xadj[v + 1] - off;
+    const RowRef rr = vlist[grp];
+    v = rr.v;
+    off = rr.off;
+    d = rr.d;
   }
   const bool act = (uint32_t)gl < d;
   const double wd = (double)(act ? clamp_weight(wgt[off + gl]) : 0.0f);
@@ -215,7 +218,7 @@ __global__ __launch_bounds__(256) void build_subwave_kernel(const uint32_t* __re
 // does exactly one binary search, lights in SH and heavies in SL, four searches interleaved; the
 // next heavy after each heavy and the last heavy of the row come from a suffix scan, not a search.
 template <int ROWT, int T>
-__global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restrict__ vlist,
+__global__ __launch_bounds__(ROWT) void build_lds_kernel(const RowRef* __restrict__ vlist,
                                                          const uint32_t* __restrict__ xadj,
                                                          const float* __restrict__ wgt,
                                                          AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
@@ -228,8 +231,8 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const uint32_t* __restr
   __shared__ uint64_t s_ex[2 * T * NW];
   __shared__ uint32_t s_fh[T][NW], s_lh[T][NW];
 
-  const uint32_t v = vlist[blockIdx.x];
-  const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+  const RowRef rr = vlist[blockIdx.x];
+  const uint32_t v = rr.v, off = rr.off, d = rr.d;
   const uint32_t base = off & ~3u, lead = off - base, span = lead + d;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 
@@ -424,7 +427,7 @@ constexpr uint64_t MERGE_CNT = 1ull << 52;
 constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
 
 template <int ROWT, int T>
-__global__ __launch_bounds__(ROWT) void build_merge_kernel(const uint32_t* __restrict__ vlist,
+__global__ __launch_bounds__(ROWT) void build_merge_kernel(const RowRef* __restrict__ vlist,
                                                            const uint32_t* __restrict__ xadj,
                                                            const float* __restrict__ wgt,
                                                            AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
@@ -441,8 +444,8 @@ __global__ __launch_bounds__(ROWT) void build_merge_kernel(const uint32_t* __res
   __shared__ WSum3 s_wsum[NW];
   __shared__ uint64_t s_ex[3 * NW];
 
-  const uint32_t v = vlist[blockIdx.x];
-  const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+  const RowRef rr = vlist[blockIdx.x];
+  const uint32_t v = rr.v, off = rr.off, d = rr.d;
   const uint32_t base = off & ~3u, lead = off - base, span = lead + d;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t pos0 = (uint32_t)PER * (uint32_t)tid;
@@ -625,7 +628,7 @@ __device__ __forceinline__ bool streaming_row(uint32_t off, uint32_t d, uint32_t
   return ((off & 3u) + d + TILED_TILE - 1) / TILED_TILE > max_tiles;  // rows the tile-parallel path leaves alone
 }
 
-__global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+__global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const RowRef* __restrict__ vlist, uint32_t count,
                                                             uint32_t max_tiles,
                                                             const uint64_t* __restrict__ scratch_off,
                                                             const uint32_t* __restrict__ xadj,
@@ -638,7 +641,7 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __re
   __shared__ uint64_t s_wl[NW], s_wh[NW];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   for (uint32_t r = blockIdx.x; r < count; r += gridDim.x) {
-    const uint32_t v = vlist[r];
+    const uint32_t v = vlist[r].v;
     const uint32_t off = xadj[v], d = xadj[v + 1] - off;
     if (!streaming_row(off, d, max_tiles)) continue;
     const float* wr = wgt + off;
@@ -718,7 +721,7 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const uint32_t* __re
 
 // Exclusive prefix sum of the degrees of the huge rows (a few thousand at most per launch of
 // 1024 threads; longer lists are walked in chunks by the same block).
-__global__ __launch_bounds__(1024) void huge_prefix_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+__global__ __launch_bounds__(1024) void huge_prefix_kernel(const RowRef* __restrict__ vlist, uint32_t count,
                                                            uint32_t max_tiles, const uint32_t* __restrict__ xadj,
                                                            uint64_t* __restrict__ scratch_off,
                                                            uint64_t* __restrict__ total) {
@@ -729,7 +732,7 @@ __global__ __launch_bounds__(1024) void huge_prefix_kernel(const uint32_t* __res
     const uint32_t r = chunk + tid;
     uint64_t d = 0;
     if (r < count) {
-      const uint32_t v = vlist[r];
+      const uint32_t v = vlist[r].v;
       d = xadj[v + 1] - xadj[v];
       if (!streaming_row(xadj[v], (uint32_t)d, max_tiles)) d = 0;
     }
@@ -754,7 +757,7 @@ namespace {
 constexpr size_t COUNTER_BYTES = 2 * CLS_COUNT * 4 + CLS_COUNT * 8;
 
 struct BuildScratch {
-  uint32_t* vlist = nullptr;     // [vcap]
+  RowRef* vlist = nullptr;       // [vcap]
   uint32_t* counters = nullptr;  // [2*CLS_COUNT] counts then cursors, then CLS_COUNT 64-bit edge totals
   uint64_t* huge_off = nullptr;  // [huge_cap + 1], last = total
   uint64_t* huge_scratch = nullptr;
@@ -814,7 +817,7 @@ int prepare_build_scratch(uint32_t max_rows) {
     if (sc.vlist) SKY_HIP(hipFree(sc.vlist));
     sc.vlist = nullptr;
     sc.vcap = 0;
-    SKY_HIP(hipMalloc((void**)&sc.vlist, (size_t)max_rows * 4 + 16));
+    SKY_HIP(hipMalloc((void**)&sc.vlist, (size_t)max_rows * sizeof(RowRef) + 16));
     sc.vcap = max_rows;
   }
   if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, COUNTER_BYTES));
@@ -857,7 +860,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
                        g->xadj, g->adjwgt, src, n, sc.counters + CLS_COUNT, sc.vlist, g->table, g->valid);
   }
   if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
-  uint32_t* const vlist = sc.vlist;
+  RowRef* const vlist = sc.vlist;
 
   auto sub = [&](int cls, auto kernel, int G, const char* name) -> int {
     const uint32_t cnt = counts[cls];

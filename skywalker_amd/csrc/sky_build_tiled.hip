@@ -74,7 +74,7 @@ struct TiledCounters {
 
 // Geometry of every row; each block reserves a run of tile ids (and of prefix-array slots) for its
 // rows with one atomic.  Tile numbering therefore depends on scheduling; no result does.
-__global__ __launch_bounds__(256) void tiled_rows_kernel(const uint32_t* __restrict__ vlist, uint32_t count,
+__global__ __launch_bounds__(256) void tiled_rows_kernel(const RowRef* __restrict__ vlist, uint32_t count,
                                                          const uint32_t* __restrict__ xadj, uint32_t max_tiles,
                                                          TiledRow* __restrict__ rows,
                                                          TiledCounters* __restrict__ ctr) {
@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void tiled_rows_kernel(const uint32_t* __restr
   uint32_t nt = 0;
   bool skip = false;
   if (r < count) {
-    row.v = vlist[r];
+    row.v = vlist[r].v;
     row.off = xadj[row.v];
     row.d = xadj[row.v + 1] - row.off;
     row.base = row.off & ~3u;
@@ -572,7 +572,7 @@ void set_tiled_max_tiles(uint32_t n) { g_tiled_max_tiles = std::min<uint32_t>(st
 
 // Builds the rows of `rows_list` (device, n entries) that have at most the configured number of
 // tiles; *skipped receives how many rows were left for the streaming kernel.
-int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
+int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
                      uint64_t edges) {
   hipStream_t st = g->stream;
   TiledScratch& sc = g_tiled;

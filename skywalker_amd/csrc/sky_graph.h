@@ -45,6 +45,12 @@ enum BuildClass : int {
   CLS_COUNT = 26
 };
 
+// One listed row of a degree class: the build kernels read where the row lies from the list itself
+// instead of chasing xadj[v] after the list entry (one dependent global load less at every row start).
+struct RowRef {
+  uint32_t v, off, d, pad;
+};
+
 // Sequence of HIP events on one stream; consecutive marks bracket one kernel (or group).
 struct EventTimer {
   hipStream_t stream;
@@ -64,7 +70,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm);
 int build_all_tables(sky_graph* g, double* seconds);
 // rows of more than 4093 entries: tile-parallel path, and how many tiles per row it accepts
 constexpr uint32_t TILED_TILE = 1024;  // slots per tile of the tile-parallel path
-int build_rows_tiled(sky_graph* g, const uint32_t* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
+int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
                      uint64_t edges);
 void set_tiled_max_tiles(uint32_t n);
 void set_row_merge(bool on);
