@@ -427,7 +427,7 @@ constexpr uint64_t MERGE_CNT = 1ull << 52;
 constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
 
 template <int ROWT, int T>
-__global__ __launch_bounds__(ROWT) void build_merge_kernel(const RowRef* __restrict__ vlist,
+__global__ __launch_bounds__(ROWT, (ROWT >= 576 && ROWT <= 640 ? 6 : 4)) void build_merge_kernel(const RowRef* __restrict__ vlist,
                                                            const uint32_t* __restrict__ xadj,
                                                            const float* __restrict__ wgt,
                                                            AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
