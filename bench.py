@@ -37,9 +37,8 @@ TRAFFIC_PER_EDGE = {"tiled_emit": 20.8, "tiled_sum": 4.3, "tiled_totals": 4.4, "
                     "lds_w1": 14.5, "wave64": 16.6}
 WALK_TRAFFIC_PER_STEP = 398.6  # walk_offline_kernel, same source
 KERNEL_OF = {  # build_profile entry -> kernel symbol
-    "bin": "bin_count_kernel+bin_scatter_kernel", "sub4": "build_subwave_kernel<4>", "sub8": "build_subwave_kernel<8>",
-    "sub16": "build_subwave_kernel<16>", "sub32": "build_subwave_kernel<32>", "wave64": "build_subwave_kernel<64>",
-    "lds_h1": "build_merge_kernel<64,1> (deg<=125)", "lds_w1": "build_merge_kernel<64,1>",
+    "bin": "bin_count_kernel+bin_scatter_kernel", "g2": "build_group_kernel<2>", "g4": "build_group_kernel<4>",
+    "g8": "build_group_kernel<8>", "g16": "build_group_kernel<16>", "g32": "build_group_kernel<32>", "lds_w1": "build_merge_kernel<64,1>",
     "lds_w2": "build_merge_kernel<64,2>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",

@@ -33,12 +33,11 @@ namespace sky {
 __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d == 0) return CLS_EMPTY;
   if (d <= 2) return CLS_TINY;
-  if (d <= 4) return CLS_SUB4;
-  if (d <= 8) return CLS_SUB8;
-  if (d <= 16) return CLS_SUB16;
-  if (d <= 32) return CLS_SUB32;
-  if (d <= 64) return CLS_WAVE;
-  if (d <= 125) return CLS_LDS_H1;
+  if (d <= 5) return CLS_G2;
+  if (d <= 13) return CLS_G4;
+  if (d <= 29) return CLS_G8;
+  if (d <= 61) return CLS_G16;
+  if (d <= 125) return CLS_G32;
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
@@ -62,7 +61,7 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
     const uint32_t v = src ? src[i] : i;
     const uint32_t d = xadj[v + 1] - xadj[v];
     const int c = degree_class(d);
-    if (c >= CLS_SUB4) atomicAdd(&s_cnt[c], 1u);
+    if (c >= CLS_G2) atomicAdd(&s_cnt[c], 1u);
     if (c >= CLS_TINY) atomicAdd(&s_edges[c], (unsigned long long)d);
   }
   __syncthreads();
@@ -74,7 +73,7 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
 
 constexpr int BIN_ITEMS = 4;  // vertices per thread in the scatter pass
 
-// Writes each vertex of class >= CLS_SUB4 into its class segment of vlist, and finishes
+// Writes each vertex of class >= CLS_G2 into its class segment of vlist, and finishes
 // the classes that need no cooperation: deg 0 (valid = 0) and deg 1..2 (closed form).
 __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __restrict__ xadj,
                                                           const float* __restrict__ wgt,
@@ -135,80 +134,137 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < BIN_ITEMS; ++i) {
-    if (cls[i] >= CLS_SUB4) vlist[s_base[cls[i]] + rank[i]] = RowRef{vtx[i], offs[i], degs[i], 0};
+    if (cls[i] >= CLS_G2) vlist[s_base[cls[i]] + rank[i]] = RowRef{vtx[i], offs[i], degs[i], 0};
   }
 }
 
-// ---------------------------------------------------------------- 4..64 lanes per vertex
-// One table entry per lane.  Prefix sums run over the group with shuffles; the two
-// searches read the group's strip of a per-wave LDS array.
+// ---------------------------------------------------------------- 2..32 lanes per row
+// G lanes share one row of at most 4 * G slots (counted from the row's 16-byte aligned start); every
+// lane holds one aligned quad of weights, so a wavefront carries 64 / G rows and the per-row steps
+// that do not depend on the row length (exact sum, ledger, scans) are paid once per 64 / G rows.
+// Prefix sums run over the group by DPP; SL and SH of every slot go to a per-group LDS strip
+// padded to 4 * G slots (slots outside the row add nothing), which each entry then searches
+// once with a fixed number of probes; the heavies' slots, compacted by rank, give "next heavy"
+// and "last heavy".  The rank rides in bits 52..63 of the SH scan.
+constexpr uint64_t GROUP_CNT = 1ull << 52;
+
 template <int G>
-__global__ __launch_bounds__(256) void build_subwave_kernel(const RowRef* __restrict__ vlist, uint32_t count,
-                                                            const uint32_t* __restrict__ xadj,
-                                                            const float* __restrict__ wgt,
-                                                            AliasEntry* __restrict__ table,
-                                                            int8_t* __restrict__ valid) {
-  __shared__ uint64_t s_sl[256], s_sh[256];
-  const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
-  const uint32_t grp = tid / G;
+__global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restrict__ vlist, uint32_t count,
+                                                          const float* __restrict__ wgt,
+                                                          AliasEntry* __restrict__ table,
+                                                          int8_t* __restrict__ valid) {
+  constexpr uint32_t SLOTS = 4 * G;
+  __shared__ uint64_t s_pre[2048];  // [0, 1024): SL of every slot of the block; [1024, 2048): SH
+  __shared__ uint8_t s_hs[1024];    // per group: row-local slot of its h-th heavy
+  const uint32_t grp = (blockIdx.x * 256u + threadIdx.x) / G;
   const int gl = threadIdx.x & (G - 1);
   const int lane = lane_id();
-  const int gb_lane = lane - gl;           // first lane of the group inside the wave
-  const int gb = threadIdx.x - gl;         // first LDS slot of the group
-  uint32_t v = 0, off = 0, d = 0;
-  if (grp < count) {
-    const RowRef rr = vlist[grp];
-    v = rr.v;
-    off = rr.off;
-    d = rr.d;
-  }
-  const bool act = (uint32_t)gl < d;
-  const double wd = (double)(act ? clamp_weight(wgt[off + gl]) : 0.0f);
+  const uint32_t gbase = 4u * (threadIdx.x - gl);  // first LDS slot of the group
+  RowRef rr{0, 0, 0, 0};
+  if (grp < count) rr = vlist[grp];
+  const uint32_t off = rr.off, d = rr.d;
+  const uint32_t base = off & ~3u, lead = off - base, span = d ? lead + d : 0;
+  const uint32_t pos = 4u * gl;
+
+  float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (pos < span) x = *reinterpret_cast<const float4*>(wgt + base + pos);
+  const float xs[4] = {x.x, x.y, x.z, x.w};
+  double wd[4];
+  uint32_t live = 0;
   WSum3 S{0.0, 0.0, 0.0};
-  wsum3_add(S, wd);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t idx = pos + k;
+    const bool in = idx >= lead && idx < span;
+    if (in) live |= 1u << k;
+    wd[k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
+    wsum3_add(S, wd[k]);
+  }
   S = group_sum_wsum3<G>(S);
   const bool row_ok = S.top + S.mid + S.low != 0.0;
   Ledger L = make_ledger_small(d, wsum3_to_double(S));
   if (!row_ok) L.scale = 0.0;
-  const Entry e = classify_small(wd, act, L);
-  const uint64_t SL = group_scan_u64<G>(e.heavy ? 0 : e.amount);
-  const uint64_t SH = group_scan_u64<G>(e.heavy ? e.amount : 0);
-  s_sl[threadIdx.x] = SL;
-  s_sh[threadIdx.x] = SH;
-  const uint64_t hm = __ballot(e.heavy);
-  const uint64_t gm = G == 64 ? ~0ull : (((1ull << (G & 63)) - 1) << gb_lane);
-  const uint64_t hmg = hm & gm;
+
+  uint64_t dl[4], sl[4], sh[4];
+  float op[4];
+  uint32_t heavy = 0;
+  uint64_t ra = 0, rb = 0;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const Entry e = classify_small(wd[k], (live >> k) & 1, L);
+    dl[k] = e.heavy ? 0 : e.amount;
+    ra += dl[k];
+    rb += e.heavy ? (e.amount | GROUP_CNT) : 0;
+    sl[k] = ra;
+    sh[k] = rb;
+    op[k] = (float)e.p;
+    if (e.heavy) heavy |= 1u << k;
+  }
+  const uint64_t ia = group_scan_u64<G>(ra), ib = group_scan_u64<G>(rb);
+  const uint32_t nh = (uint32_t)(shfl_u64(ib, (lane - gl) + G - 1) >> 52);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    sl[k] += ia - ra;
+    sh[k] += ib - rb;
+    s_pre[gbase + pos + k] = sl[k];
+    s_pre[1024 + gbase + pos + k] = sh[k] & (GROUP_CNT - 1);
+    if ((heavy >> k) & 1) s_hs[gbase + (uint32_t)(sh[k] >> 52) - 1] = (uint8_t)(pos + k - lead);
+  }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
   // light: first slot with SH > SL - D.  heavy: first slot with SL >= SH, i.e. SL > SH - 1.
-  const uint64_t* arr = (e.heavy ? s_sl : s_sh) + gb;
-  const uint64_t key = e.heavy ? SH - 1 : SL - e.amount;
-  int pos = 0;
+  uint32_t arr[4], at[4];
+  uint64_t key[4];
 #pragma unroll
-  for (int step = G / 2; step >= 1; step >>= 1)
-    if (arr[pos + step - 1] <= key) pos += step;
-  const uint64_t at = arr[pos];
-  const bool found = at > key;
-  float out_p;
-  uint32_t out_a;
-  if (!e.heavy) {
-    out_p = (float)e.p;
-    out_a = found ? (uint32_t)pos : (hmg ? (uint32_t)(63 - __clzll(hmg) - gb_lane) : (uint32_t)gl);
-  } else {
-    const uint64_t above = hmg & ~((2ull << lane) - 1);
-    if (above == 0 || !found) {
-      out_p = 1.0f;
-      out_a = gl;
+  for (int k = 0; k < 4; ++k) {
+    const bool hv = (heavy >> k) & 1;
+    arr[k] = gbase + (hv ? 0u : 1024u);
+    key[k] = hv ? (sh[k] & (GROUP_CNT - 1)) - 1 : sl[k] - dl[k];
+    at[k] = 0;
+  }
+#pragma unroll
+  for (uint32_t step = SLOTS / 2; step >= 1; step >>= 1) {
+    uint64_t v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = s_pre[arr[k] + at[k] + step - 1];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) at[k] += v[k] <= key[k] ? step : 0u;
+  }
+  uint32_t oa[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint64_t v = s_pre[arr[k] + at[k]];
+    const bool found = v > key[k];
+    const uint32_t self = pos + k - lead;
+    if (!((heavy >> k) & 1)) {
+      oa[k] = found ? at[k] - lead : (nh ? (uint32_t)s_hs[gbase + nh - 1] : self);
     } else {
-      out_p = residual_prob(L.one + SH - at, L);
-      out_a = (uint32_t)(__ffsll((unsigned long long)above) - 1 - gb_lane);
+      const uint32_t hc = (uint32_t)(sh[k] >> 52);
+      if (hc < nh && found) {
+        op[k] = residual_prob(L.one + key[k] + 1 - v, L);
+        oa[k] = s_hs[gbase + hc];
+      } else {
+        op[k] = 1.0f;
+        oa[k] = self;
+      }
+    }
+    if (!row_ok) {
+      op[k] = 0.0f;
+      oa[k] = SKY_INVALID;
     }
   }
-  if (!row_ok) { out_p = 0.0f; out_a = SKY_INVALID; }
-  if (act) {
-    table[off + gl] = AliasEntry{out_p, out_a};
+  if (pos < span) {
+    if (pos >= lead && pos + 4 <= span) {
+      store_entries4(table + base + pos, op, oa);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if ((live >> k) & 1) table[base + pos + k] = AliasEntry{op[k], oa[k]};
+    }
   }
-  if (gl == 0 && grp < count) valid[v] = row_ok;
+  if (gl == 0 && d) valid[rr.v] = row_ok;
 }
 
 // ---------------------------------------------------------------- one row per workgroup, prefix arrays in LDS
@@ -862,20 +918,20 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
   RowRef* const vlist = sc.vlist;
 
-  auto sub = [&](int cls, auto kernel, int G, const char* name) -> int {
+  auto grp = [&](int cls, auto kernel, int G, const char* name) -> int {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const uint32_t per_block = 256 / G;
       hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, st, vlist + starts[cls],
-                         cnt, g->xadj, g->adjwgt, g->table, g->valid);
+                         cnt, g->adjwgt, g->table, g->valid);
     }
     return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
-  SKY_TRY(sub(CLS_SUB4, build_subwave_kernel<4>, 4, "sub4"));
-  SKY_TRY(sub(CLS_SUB8, build_subwave_kernel<8>, 8, "sub8"));
-  SKY_TRY(sub(CLS_SUB16, build_subwave_kernel<16>, 16, "sub16"));
-  SKY_TRY(sub(CLS_SUB32, build_subwave_kernel<32>, 32, "sub32"));
-  SKY_TRY(sub(CLS_WAVE, build_subwave_kernel<64>, 64, "wave64"));
+  SKY_TRY(grp(CLS_G2, build_group_kernel<2>, 2, "g2"));
+  SKY_TRY(grp(CLS_G4, build_group_kernel<4>, 4, "g4"));
+  SKY_TRY(grp(CLS_G8, build_group_kernel<8>, 8, "g8"));
+  SKY_TRY(grp(CLS_G16, build_group_kernel<16>, 16, "g16"));
+  SKY_TRY(grp(CLS_G32, build_group_kernel<32>, 32, "g32"));
 
   auto lds = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
     const uint32_t cnt = counts[cls];
@@ -898,7 +954,6 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   static const char* const mw_name[15] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9",
                                           "mw10", "mw11", "mw12", "mw13", "mw14", "mw15", "mw16"};
   if (g_row_merge) {
-    SKY_TRY(mrg(CLS_LDS_H1, build_merge_kernel<64, 1>, 64, 1, "lds_h1"));
     SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 1>, 64, 1, "lds_w1"));
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 2>, 64, 2, "lds_w2"));
 #define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 2>, 64 * NW, 2, mw_name[NW - 2]))
@@ -906,7 +961,6 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     SKY_MW(10); SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
 #undef SKY_MW
   } else {
-    SKY_TRY(lds(CLS_LDS_H1, build_lds_kernel<64, 1>, 64, 1, "lds_h1"));
     SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
     SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
     for (int nw = 2; nw <= 16; ++nw) {

@@ -287,8 +287,10 @@ __device__ __forceinline__ uint64_t group_scan_u64(uint64_t v) {
   } else {
     uint64_t o = dpp0_u64<DPP_ROW_SHR1, 0xF>(v);
     v += gl >= 1 ? o : 0;
-    o = dpp0_u64<DPP_ROW_SHR2, 0xF>(v);
-    v += gl >= 2 ? o : 0;
+    if (G >= 4) {
+      o = dpp0_u64<DPP_ROW_SHR2, 0xF>(v);
+      v += gl >= 2 ? o : 0;
+    }
     if (G >= 8) {
       o = dpp0_u64<DPP_ROW_SHR4, 0xF>(v);
       v += gl >= 4 ? o : 0;
@@ -345,7 +347,7 @@ __device__ __forceinline__ double group_sum_f64(double v) {
     return __longlong_as_double((long long)f(b));
   };
   v += get(v, [](uint64_t b) { return dpp0_u64<DPP_QUAD_XOR1, 0xF>(b); });
-  v += get(v, [](uint64_t b) { return dpp0_u64<DPP_QUAD_XOR2, 0xF>(b); });
+  if (G >= 4) v += get(v, [](uint64_t b) { return dpp0_u64<DPP_QUAD_XOR2, 0xF>(b); });
   if (G >= 8) v += get(v, [](uint64_t b) { return dpp0_u64<DPP_ROW_HALF_MIRROR, 0xF>(b); });
   if (G >= 16) v += get(v, [](uint64_t b) { return dpp0_u64<DPP_ROW_MIRROR, 0xF>(b); });
   if (G >= 32) v += get(v, [](uint64_t b) { return shfl_xor_u64(b, 16); });

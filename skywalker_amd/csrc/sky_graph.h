@@ -31,18 +31,17 @@ namespace sky {
 enum BuildClass : int {
   CLS_EMPTY = 0,   // deg 0            handled while binning
   CLS_TINY = 1,    // deg 1..2         one lane per vertex, handled while binning
-  CLS_SUB4 = 2,    // deg 3..4         4 lanes per vertex
-  CLS_SUB8 = 3,    // deg 5..8
-  CLS_SUB16 = 4,   // deg 9..16
-  CLS_SUB32 = 5,   // deg 17..32
-  CLS_WAVE = 6,    // deg 33..64       one wavefront, one entry per lane
-  CLS_LDS_H1 = 7,  // deg <= 125       one wavefront, LDS prefix arrays, 4 entries per lane (half the lanes idle)
-  CLS_LDS_W1 = 8,  // deg <= 253       one wavefront, 4 entries per lane
-  CLS_LDS_W2 = 9,  // deg <= 509       one wavefront, 8 entries per lane
-  CLS_MW2 = 10,    // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
-  CLS_MW16 = 24,   //                  class CLS_MW2 + nw - 2
-  CLS_HUGE = 25,   // deg > 8189       built tile by tile by the whole GPU
-  CLS_COUNT = 26
+  CLS_G2 = 2,      // deg 3..5         2 lanes per row, one quad of slots per lane
+  CLS_G4 = 3,      // deg <= 13        4 lanes per row
+  CLS_G8 = 4,      // deg <= 29
+  CLS_G16 = 5,     // deg <= 61
+  CLS_G32 = 6,     // deg <= 125
+  CLS_LDS_W1 = 7,  // deg <= 253       one wavefront, LDS prefix arrays, 4 entries per lane
+  CLS_LDS_W2 = 8,  // deg <= 509       one wavefront, 8 entries per lane
+  CLS_MW2 = 9,     // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
+  CLS_MW16 = 23,   //                  class CLS_MW2 + nw - 2
+  CLS_HUGE = 24,   // deg > 8189       built tile by tile by the whole GPU
+  CLS_COUNT = 25
 };
 
 // One listed row of a degree class: the build kernels read where the row lies from the list itself
