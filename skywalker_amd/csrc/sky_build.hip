@@ -45,10 +45,17 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
 }
 
 // ---------------------------------------------------------------- binning
-// `src` lists the vertices to bin (n of them); a null src means vertices 0..n-1.
+// `src` lists the vertices to bin (n of them); a null src means vertices 0..n-1.  Block b of the
+// count and scatter kernels owns the items [b * per_block, (b + 1) * per_block): the count kernel
+// leaves one row of class counts per block, bin_offsets_kernel turns the rows into each block's
+// first position inside every class segment, and the scatter kernel hands out positions from
+// cursors it keeps in LDS, so no global atomic is involved and the lists come out grouped by block.
+constexpr int BIN_BLOCKS = 2048;  // most blocks a binning pass uses
+constexpr int BIN_ITEMS = 4;      // vertices per thread and step of the scatter pass
+
 __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restrict__ xadj,
                                                         const uint32_t* __restrict__ src, uint32_t n,
-                                                        uint32_t* __restrict__ counts,
+                                                        uint32_t per_block, uint32_t* __restrict__ blk_cnt,
                                                         unsigned long long* __restrict__ class_edges) {
   __shared__ uint32_t s_cnt[CLS_COUNT];
   __shared__ unsigned long long s_edges[CLS_COUNT];
@@ -57,7 +64,8 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
     s_edges[threadIdx.x] = 0;
   }
   __syncthreads();
-  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += gridDim.x * 256u) {
+  const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
+  for (uint32_t i = lo + threadIdx.x; i < hi; i += 256u) {
     const uint32_t v = src ? src[i] : i;
     const uint32_t d = xadj[v + 1] - xadj[v];
     const int c = degree_class(d);
@@ -66,75 +74,78 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
   }
   __syncthreads();
   if (threadIdx.x < CLS_COUNT) {
-    if (s_cnt[threadIdx.x]) atomicAdd(&counts[threadIdx.x], s_cnt[threadIdx.x]);
+    blk_cnt[blockIdx.x * CLS_COUNT + threadIdx.x] = s_cnt[threadIdx.x];
     if (s_edges[threadIdx.x]) atomicAdd(&class_edges[threadIdx.x], s_edges[threadIdx.x]);
   }
 }
 
-constexpr int BIN_ITEMS = 4;  // vertices per thread in the scatter pass
+// One wavefront per class: exclusive prefix of the class's per-block counts (in place), total to counts[c].
+__global__ __launch_bounds__(64) void bin_offsets_kernel(uint32_t* __restrict__ blk_cnt, uint32_t blocks,
+                                                         uint32_t* __restrict__ counts) {
+  const uint32_t c = blockIdx.x, lane = threadIdx.x;
+  uint32_t run = 0;
+  for (uint32_t b0 = 0; b0 < blocks; b0 += 64) {
+    const uint32_t b = b0 + lane;
+    const uint32_t x = b < blocks ? blk_cnt[b * CLS_COUNT + c] : 0u;
+    const uint32_t inc = group_scan_u32<64>(x);
+    if (b < blocks) blk_cnt[b * CLS_COUNT + c] = run + inc - x;
+    run += (uint32_t)__shfl((int)inc, 63, 64);
+  }
+  if (lane == 0) counts[c] = run;
+}
 
-// Writes each vertex of class >= CLS_G2 into its class segment of vlist, and finishes
+// Writes each row of class >= CLS_G2 into its class segment of vlist, and finishes
 // the classes that need no cooperation: deg 0 (valid = 0) and deg 1..2 (closed form).
 __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __restrict__ xadj,
                                                           const float* __restrict__ wgt,
                                                           const uint32_t* __restrict__ src, uint32_t n,
-                                                          uint32_t* __restrict__ cursors,
+                                                          uint32_t per_block,
+                                                          const uint32_t* __restrict__ class_start,
+                                                          const uint32_t* __restrict__ blk_off,
                                                           RowRef* __restrict__ vlist,
                                                           AliasEntry* __restrict__ table,
                                                           int8_t* __restrict__ valid) {
-  __shared__ uint32_t s_cnt[CLS_COUNT], s_base[CLS_COUNT];
-  if (threadIdx.x < CLS_COUNT) s_cnt[threadIdx.x] = 0;
+  __shared__ uint32_t s_cur[CLS_COUNT];
+  if (threadIdx.x < CLS_COUNT)
+    s_cur[threadIdx.x] = class_start[threadIdx.x] + blk_off[blockIdx.x * CLS_COUNT + threadIdx.x];
   __syncthreads();
-  const uint32_t chunk = blockIdx.x * (256u * BIN_ITEMS);
-  int cls[BIN_ITEMS];
-  uint32_t rank[BIN_ITEMS], vtx[BIN_ITEMS], offs[BIN_ITEMS], degs[BIN_ITEMS];
+  const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
+  for (uint32_t chunk = lo; chunk < hi; chunk += 256u * BIN_ITEMS) {
 #pragma unroll
-  for (int i = 0; i < BIN_ITEMS; ++i) {
-    const uint32_t item = chunk + i * 256u + threadIdx.x;
-    cls[i] = -1;
-    if (item >= n) continue;
-    const uint32_t v = src ? src[item] : item;
-    vtx[i] = v;
-    const uint32_t off = xadj[v], d = xadj[v + 1] - off;
-    offs[i] = off;
-    degs[i] = d;
-    const int c = degree_class(d);
-    cls[i] = c;
-    if (c == CLS_EMPTY) {
-      valid[v] = 0;
-    } else if (c == CLS_TINY) {
-      const float w0 = clamp_weight(wgt[off]);
-      if (d == 1) {
-        const u128 q = weight_fixed(w0);
-        const bool ok = (q.lo | q.hi) != 0;
-        table[off] = AliasEntry{ok ? 1.0f : 0.0f, ok ? 0u : SKY_INVALID};
-        valid[v] = ok;
-      } else {
-        const float w1 = clamp_weight(wgt[off + 1]);
-        const u128 s = add128(weight_fixed(w0), weight_fixed(w1));
-        if ((s.lo | s.hi) == 0) {
-          table[off] = table[off + 1] = AliasEntry{0.0f, SKY_INVALID};
-          valid[v] = 0;
+    for (int i = 0; i < BIN_ITEMS; ++i) {
+      const uint32_t item = chunk + i * 256u + threadIdx.x;
+      if (item >= hi) continue;
+      const uint32_t v = src ? src[item] : item;
+      const uint32_t off = xadj[v], d = xadj[v + 1] - off;
+      const int c = degree_class(d);
+      if (c == CLS_EMPTY) {
+        valid[v] = 0;
+      } else if (c == CLS_TINY) {
+        const float w0 = clamp_weight(wgt[off]);
+        if (d == 1) {
+          const u128 q = weight_fixed(w0);
+          const bool ok = (q.lo | q.hi) != 0;
+          table[off] = AliasEntry{ok ? 1.0f : 0.0f, ok ? 0u : SKY_INVALID};
+          valid[v] = ok;
         } else {
-          const Ledger L = make_ledger(2, s);
-          const Entry e0 = classify(w0, L), e1 = classify(w1, L);
-          // a lone heavy is the last heavy: it keeps its bucket and tops up the light
-          table[off] = AliasEntry{e0.heavy ? 1.0f : (float)e0.p, (!e0.heavy && e1.heavy) ? 1u : 0u};
-          table[off + 1] = AliasEntry{e1.heavy ? 1.0f : (float)e1.p, (!e1.heavy && e0.heavy) ? 0u : 1u};
-          valid[v] = 1;
+          const float w1 = clamp_weight(wgt[off + 1]);
+          const u128 s = add128(weight_fixed(w0), weight_fixed(w1));
+          if ((s.lo | s.hi) == 0) {
+            table[off] = table[off + 1] = AliasEntry{0.0f, SKY_INVALID};
+            valid[v] = 0;
+          } else {
+            const Ledger L = make_ledger(2, s);
+            const Entry e0 = classify(w0, L), e1 = classify(w1, L);
+            // a lone heavy is the last heavy: it keeps its bucket and tops up the light
+            table[off] = AliasEntry{e0.heavy ? 1.0f : (float)e0.p, (!e0.heavy && e1.heavy) ? 1u : 0u};
+            table[off + 1] = AliasEntry{e1.heavy ? 1.0f : (float)e1.p, (!e1.heavy && e0.heavy) ? 0u : 1u};
+            valid[v] = 1;
+          }
         }
+      } else {
+        vlist[atomicAdd(&s_cur[c], 1u)] = RowRef{v, off, d, 0};
       }
-    } else {
-      rank[i] = atomicAdd(&s_cnt[c], 1u);
     }
-  }
-  __syncthreads();
-  if (threadIdx.x < CLS_COUNT && s_cnt[threadIdx.x])
-    s_base[threadIdx.x] = atomicAdd(&cursors[threadIdx.x], s_cnt[threadIdx.x]);
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < BIN_ITEMS; ++i) {
-    if (cls[i] >= CLS_G2) vlist[s_base[cls[i]] + rank[i]] = RowRef{vtx[i], offs[i], degs[i], 0};
   }
 }
 
@@ -814,7 +825,8 @@ constexpr size_t COUNTER_BYTES = 2 * CLS_COUNT * 4 + CLS_COUNT * 8;
 
 struct BuildScratch {
   RowRef* vlist = nullptr;       // [vcap]
-  uint32_t* counters = nullptr;  // [2*CLS_COUNT] counts then cursors, then CLS_COUNT 64-bit edge totals
+  uint32_t* counters = nullptr;  // [2*CLS_COUNT] counts then class starts, then CLS_COUNT 64-bit edge totals
+  uint32_t* blk_cnt = nullptr;   // [BIN_BLOCKS * CLS_COUNT] class counts of every binning block, then their prefixes
   uint64_t* huge_off = nullptr;  // [huge_cap + 1], last = total
   uint64_t* huge_scratch = nullptr;
   uint32_t vcap = 0, huge_cap = 0;
@@ -877,6 +889,7 @@ int prepare_build_scratch(uint32_t max_rows) {
     sc.vcap = max_rows;
   }
   if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, COUNTER_BYTES));
+  if (!sc.blk_cnt) SKY_HIP(hipMalloc((void**)&sc.blk_cnt, (size_t)BIN_BLOCKS * CLS_COUNT * 4));
   if (!sc.lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
 #define SKY_BIG(NW) SKY_TRY(enable_big_lds(build_merge_kernel<64 * NW, 2>, (64 * NW * 8 + 2) * 14))
@@ -900,9 +913,13 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   static_assert(sizeof(host) == COUNTER_BYTES, "counter block layout");
   if (n > 0) {
     SKY_HIP(hipMemsetAsync(sc.counters, 0, COUNTER_BYTES, st));
-    const uint32_t grid = std::min<uint32_t>((n + 255) / 256, 256 * 8);
-    hipLaunchKernelGGL(bin_count_kernel, dim3(grid), dim3(256), 0, st, g->xadj, src, n, sc.counters,
+    // at most BIN_BLOCKS blocks, each a multiple of one scatter step
+    const uint32_t step = 256u * BIN_ITEMS;
+    const uint32_t per_block = ((n + BIN_BLOCKS - 1) / BIN_BLOCKS + step - 1) / step * step;
+    const uint32_t blocks = (n + per_block - 1) / per_block;
+    hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n, per_block, sc.blk_cnt,
                        reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
+    hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(64), 0, st, sc.blk_cnt, blocks, sc.counters);
     SKY_HIP(hipMemcpyAsync(&host, sc.counters, COUNTER_BYTES, hipMemcpyDeviceToHost, st));
     SKY_HIP(hipStreamSynchronize(st));
     for (int c = 0; c < CLS_COUNT; ++c) counts[c] = host.counts[c];
@@ -912,8 +929,8 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       acc += counts[c];
     }
     SKY_HIP(hipMemcpyAsync(sc.counters + CLS_COUNT, starts, sizeof(starts), hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL(bin_scatter_kernel, dim3((n + 256 * BIN_ITEMS - 1) / (256 * BIN_ITEMS)), dim3(256), 0, st,
-                       g->xadj, g->adjwgt, src, n, sc.counters + CLS_COUNT, sc.vlist, g->table, g->valid);
+    hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n, per_block,
+                       sc.counters + CLS_COUNT, sc.blk_cnt, sc.vlist, g->table, g->valid);
   }
   if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
   RowRef* const vlist = sc.vlist;
