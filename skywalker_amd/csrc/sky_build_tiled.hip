@@ -38,6 +38,20 @@ struct TileTotals {
   uint32_t first_heavy, last_heavy;  // span indices, NONE32 when the tile has no heavy
 };
 
+// Where a tile lies, one aligned record per tile: a tile's weights can be requested after one
+// dependent load instead of two (tile -> row -> geometry).
+struct __attribute__((aligned(32))) TileGeom {
+  uint32_t row, T, base, lead, span, pad[3];  // row: index into the row array; T: tile number inside the row
+};
+__device__ __forceinline__ TiledRow geom_row(const TileGeom& tg, uint32_t tile) {
+  TiledRow r = {};
+  r.base = tg.base;
+  r.lead = tg.lead;
+  r.span = tg.span;
+  r.tile0 = tile - tg.T;
+  return r;
+}
+
 __device__ __forceinline__ Ledger row_ledger(const TiledRow& r) {
   Ledger L;
   L.scale = r.scale;
@@ -119,23 +133,24 @@ __global__ __launch_bounds__(256) void tiled_rows_kernel(const RowRef* __restric
 }
 
 __global__ __launch_bounds__(256) void tiled_map_kernel(const TiledRow* __restrict__ rows, uint32_t count,
-                                                        uint32_t* __restrict__ tile2row) {
+                                                        TileGeom* __restrict__ geom) {
   const uint32_t r = blockIdx.x;
   if (r >= count) return;
-  const uint32_t t0 = rows[r].tile0, nt = rows[r].ntiles;
-  for (uint32_t t = threadIdx.x; t < nt; t += 256) tile2row[t0 + t] = r;
+  const TiledRow row = rows[r];
+  for (uint32_t t = threadIdx.x; t < row.ntiles; t += 256)
+    geom[row.tile0 + t] = TileGeom{r, t, row.base, row.lead, row.span, {0, 0, 0}};
 }
 
 // ---------------------------------------------------------------- pass 1: exact sums
-__global__ __launch_bounds__(TL_T) void tiled_sum_kernel(const uint32_t* __restrict__ tile2row,
-                                                         const TiledRow* __restrict__ rows,
+__global__ __launch_bounds__(TL_T) void tiled_sum_kernel(const TileGeom* __restrict__ geom,
                                                          const float* __restrict__ wgt, u128* __restrict__ tsum) {
   __shared__ WSum3 s_w[TL_T / 64];
   const uint32_t tile = blockIdx.x;
-  const TiledRow r = rows[tile2row[tile]];
+  const TileGeom tg = geom[tile];
+  const TiledRow r = geom_row(tg, tile);
   const int tid = threadIdx.x;
   float w[TL_Q][4];
-  load_tile(wgt, r, tile - r.tile0, tid, w);
+  load_tile(wgt, r, tg.T, tid, w);
   WSum3 sum{0.0, 0.0, 0.0};  // exact: a tile adds at most 1024 limbs below 2^32 + 1
 #pragma unroll
   for (int q = 0; q < TL_Q; ++q)
@@ -178,20 +193,21 @@ __global__ __launch_bounds__(64) void tiled_ledger_kernel(TiledRow* __restrict__
 }
 
 // ---------------------------------------------------------------- pass 2: tile totals
-__global__ __launch_bounds__(TL_T) void tiled_totals_kernel(const uint32_t* __restrict__ tile2row,
+__global__ __launch_bounds__(TL_T) void tiled_totals_kernel(const TileGeom* __restrict__ geom,
                                                             const TiledRow* __restrict__ rows,
                                                             const float* __restrict__ wgt,
                                                             TileTotals* __restrict__ ttot) {
   __shared__ uint64_t s_d[TL_T / 64], s_u[TL_T / 64];
   __shared__ uint32_t s_f[TL_T / 64], s_l[TL_T / 64];
   const uint32_t tile = blockIdx.x;
-  const TiledRow r = rows[tile2row[tile]];
+  const TileGeom tg = geom[tile];
   const int tid = threadIdx.x;
+  const uint32_t t = tg.T;
+  float w[TL_Q][4];
+  load_tile(wgt, geom_row(tg, tile), t, tid, w);  // requested before the row's ledger arrives
+  const TiledRow r = rows[tg.row];
   if (!r.ok) return;
   const Ledger L = row_ledger(r);
-  const uint32_t t = tile - r.tile0;
-  float w[TL_Q][4];
-  load_tile(wgt, r, t, tid, w);
   uint64_t sd = 0, su = 0;
   uint32_t fh = NONE32, lh = 0;  // lh holds idx + 1 so that 0 means none
 #pragma unroll
@@ -400,7 +416,7 @@ __device__ __forceinline__ void partner_pass(const TiledRow& r, const Ledger& L,
   }
 }
 
-__global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __restrict__ tile2row,
+__global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const TileGeom* __restrict__ geom,
                                                           const TiledRow* __restrict__ rows,
                                                           const float* __restrict__ wgt,
                                                           const uint64_t* __restrict__ gBL,
@@ -414,13 +430,13 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const uint32_t* __rest
   __shared__ uint64_t s_ex[2 * TL_Q * NW];
   __shared__ uint32_t s_fh[TL_Q][NW];
   const uint32_t tile = blockIdx.x;
-  const uint32_t ri = tile2row[tile];
-  const TiledRow r = rows[ri];
+  const TileGeom tg = geom[tile];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const uint32_t T = tile - r.tile0;
+  const uint32_t T = tg.T;
 
   float w[TL_Q][4];
-  load_tile(wgt, r, T, tid, w);
+  load_tile(wgt, geom_row(tg, tile), T, tid, w);  // requested before the row record arrives
+  const TiledRow r = rows[tg.row];
   if (!r.ok) {
 #pragma unroll
     for (int q = 0; q < TL_Q; ++q)
@@ -554,7 +570,7 @@ namespace {
 struct TiledScratch {
   TiledRow* rows = nullptr;
   TiledCounters* totals = nullptr;
-  uint32_t* tile2row = nullptr;
+  TileGeom* geom = nullptr;
   u128* tsum = nullptr;
   TileTotals* ttot = nullptr;
   uint64_t *BL = nullptr, *BH = nullptr;
@@ -597,13 +613,13 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
   *skipped = totals.skipped;
   if (ntiles == 0) return SKY_OK;
   if (sc.tile_cap < ntiles) {
-    void* olds[] = {sc.tile2row, sc.tsum, sc.ttot, sc.nfh, sc.ranges};
+    void* olds[] = {sc.geom, sc.tsum, sc.ttot, sc.nfh, sc.ranges};
     for (void* p : olds)
       if (p) SKY_HIP(hipFree(p));
-    sc.tile2row = nullptr; sc.tsum = nullptr; sc.ttot = nullptr; sc.nfh = nullptr; sc.ranges = nullptr;
+    sc.geom = nullptr; sc.tsum = nullptr; sc.ttot = nullptr; sc.nfh = nullptr; sc.ranges = nullptr;
     sc.tile_cap = 0;
     const size_t cap = (size_t)ntiles + ntiles / 4 + 1024;
-    SKY_HIP(hipMalloc((void**)&sc.tile2row, cap * 4));
+    SKY_HIP(hipMalloc((void**)&sc.geom, cap * sizeof(TileGeom)));
     SKY_HIP(hipMalloc((void**)&sc.tsum, cap * sizeof(u128)));
     SKY_HIP(hipMalloc((void**)&sc.ttot, cap * sizeof(TileTotals)));
     SKY_HIP(hipMalloc((void**)&sc.nfh, cap * 4));
@@ -622,15 +638,15 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
     SKY_HIP(hipMalloc((void**)&sc.BH, (b_need + b_need / 4 + 1024) * 8));
     b_cap = b_need + b_need / 4 + 1024;
   }
-  hipLaunchKernelGGL(tiled_map_kernel, dim3(n), dim3(256), 0, st, sc.rows, n, sc.tile2row);
+  hipLaunchKernelGGL(tiled_map_kernel, dim3(n), dim3(256), 0, st, sc.rows, n, sc.geom);
   if (tm) SKY_TRY(tm->mark("tiled_rows", 0));
-  hipLaunchKernelGGL(tiled_sum_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.tsum);
+  hipLaunchKernelGGL(tiled_sum_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.geom, g->adjwgt, sc.tsum);
   if (tm) SKY_TRY(tm->mark("tiled_sum", edges));
   hipLaunchKernelGGL(tiled_ledger_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.tsum);
-  hipLaunchKernelGGL(tiled_totals_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.ttot);
+  hipLaunchKernelGGL(tiled_totals_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.geom, sc.rows, g->adjwgt, sc.ttot);
   if (tm) SKY_TRY(tm->mark("tiled_totals", edges));
   hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh, sc.ranges);
-  hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.tile2row, sc.rows, g->adjwgt, sc.BL,
+  hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.geom, sc.rows, g->adjwgt, sc.BL,
                      sc.BH, sc.nfh, sc.ranges, g->table, g->valid);
   if (tm) SKY_TRY(tm->mark("tiled_emit", edges));
   return SKY_OK;
