@@ -42,7 +42,8 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
     "lds_w2": "build_merge_kernel<64,2>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
-    "streamed": "huge_prefix_kernel+build_huge_kernel",
+    "streamed": "huge_prefix_kernel+build_huge_kernel", "stream": "build_stream_kernel",
+    "stream_deferred": "tile-parallel path for rows deferred by build_stream_kernel",
 }
 KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,2>" % (64 * nw) for nw in range(2, 17)})
 

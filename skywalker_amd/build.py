@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libskywalker_hip.so")
-SOURCES = ["sky_capi.hip", "sky_build.hip", "sky_build_tiled.hip", "sky_walk.hip", "sky_online.hip", "sky_sample.hip", "sky_gen.hip"]
+SOURCES = ["sky_capi.hip", "sky_build.hip", "sky_build_tiled.hip", "sky_build_stream.hip", "sky_walk.hip", "sky_online.hip", "sky_sample.hip", "sky_gen.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",

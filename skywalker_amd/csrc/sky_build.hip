@@ -41,7 +41,8 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
-  return nw <= 16 ? CLS_MW2 + (int)nw - 2 : CLS_HUGE;
+  if (nw <= 16) return CLS_MW2 + (int)nw - 2;
+  return d <= STREAM_MAX_DEG ? CLS_STREAM : CLS_HUGE;
 }
 
 // ---------------------------------------------------------------- binning
@@ -996,6 +997,22 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
   }
 
+  if (counts[CLS_STREAM]) {
+    const uint32_t cnt = counts[CLS_STREAM];
+    uint32_t skipped = 0;
+    if (g_row_merge) {
+      const RowRef* deferred = nullptr;
+      uint32_t nd = 0;
+      SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], cnt, &deferred, &nd));
+      if (tm) SKY_TRY(tm->mark("stream", host.edges[CLS_STREAM]));
+      SKY_TRY(stream_deferred_count(g, &nd));
+      if (nd) SKY_TRY(build_rows_tiled(g, deferred, nd, &skipped, nullptr, 0));  // more heavies than LDS holds
+    } else {
+      SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_STREAM], cnt, &skipped, nullptr, 0));
+    }
+    if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles is too small for rows of up to 65533 entries");
+    if (tm) SKY_TRY(tm->mark("stream_deferred", 0));
+  }
   if (counts[CLS_HUGE]) {
     const uint32_t cnt = counts[CLS_HUGE];
     uint32_t skipped = 0;

@@ -1,0 +1,316 @@
+// Alias tables of rows of 8190..65533 entries: one workgroup streams the row three times and
+// keeps the row's heavies in LDS.
+//
+// The table is the same pure function of the weights as everywhere else (see sky_build.hip).
+// Only the heavies of a row need random access: a light's alias is the first heavy whose surplus
+// prefix exceeds the light's exclusive deficit prefix, and a heavy's residual probability belongs
+// to the one light whose deficit interval (SL - D, SL] contains the heavy's surplus prefix.  So
+//   pass A  exact sum of the weights -> ledger
+//   pass B  classify, running surplus prefix; heavies compacted into LDS in slot order:
+//           {surplus prefix, slot}, 10 bytes each
+//   pass C  classify again, running deficit prefix; every light searches the heavy list once
+//           (alias) and finishes the heavies whose prefix falls into its interval (usually none,
+//           sometimes one); every heavy takes the next heavy of the list as alias, or {1, itself}
+//           when it is the last heavy or no light reaches it.
+// A heavy's probability and alias are separate 4-byte stores by different threads of the workgroup.
+// The second and third pass read the weights from L2.  Rows with more heavies than the LDS list
+// holds are appended to `deferred` and left untouched (the tile-parallel path builds them).
+#include "sky_build_common.h"
+#include "sky_graph.h"
+
+namespace sky {
+
+constexpr int ST_T = 512;                 // threads per row
+constexpr int ST_PER = 8;                 // consecutive slots per thread and chunk
+constexpr int ST_CH = ST_T * ST_PER;      // slots per chunk
+constexpr int ST_NW = ST_T / 64;
+constexpr uint32_t ST_CAP = 8064;         // heavies per row kept in LDS: two workgroups share a CU's 160 KB
+static_assert(STREAM_MAX_DEG + 3 <= 65536, "heavy slots are stored as 16-bit numbers");
+
+struct StreamRow {
+  uint32_t base, lead, span;
+};
+
+// The 8 weights of this thread in chunk c (span slots c*ST_CH + 8*tid ...), clamped, as doubles; 0 outside
+// the row.  Returns the mask of slots that belong to the row.
+__device__ __forceinline__ uint32_t load_chunk(const float* __restrict__ wgt, const StreamRow& r, uint32_t c, int tid,
+                                               double (&wd)[ST_PER]) {
+  uint32_t live = 0;
+#pragma unroll
+  for (int q = 0; q < ST_PER / 4; ++q) {
+    const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
+    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pos < r.span) x = *reinterpret_cast<const float4*>(wgt + r.base + pos);
+    const float xs[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t idx = pos + k;
+      const bool in = idx >= r.lead && idx < r.span;
+      if (in) live |= 1u << (q * 4 + k);
+      wd[q * 4 + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
+    }
+  }
+  return live;
+}
+
+// Exclusive prefix over the workgroup (thread order) of one u64 and one u32 per thread, plus totals.
+// Two barriers: the second one lets the caller reuse s_a / s_c right away.
+__device__ __forceinline__ void stream_excl(uint64_t a, uint32_t c, uint64_t* s_a, uint32_t* s_c, uint64_t& ex_a,
+                                            uint32_t& ex_c, uint64_t& tot_a, uint32_t& tot_c) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint64_t ia = group_scan_u64<64>(a);
+  const uint32_t ic = group_scan_u32<64>(c);
+  if (lane == 63) {
+    s_a[wave] = ia;
+    s_c[wave] = ic;
+  }
+  __syncthreads();
+  uint64_t ra = 0;
+  uint32_t rc = 0;
+  ex_a = ia - a;
+  ex_c = ic - c;
+#pragma unroll
+  for (int w = 0; w < ST_NW; ++w) {
+    if (w == wave) {
+      ex_a += ra;
+      ex_c += rc;
+    }
+    ra += s_a[w];
+    rc += s_c[w];
+  }
+  tot_a = ra;
+  tot_c = rc;
+  __syncthreads();
+}
+
+// For M keys at once: number of entries of the sorted LDS array a[0..n), n >= 1, that are <= key[m].
+// The M chains of dependent LDS reads advance in lockstep, so their latencies overlap.
+template <int M>
+__device__ __forceinline__ void count_le(const uint64_t* a, uint32_t n, const uint64_t (&key)[M], uint32_t (&out)[M]) {
+  const uint32_t hb = 1u << (31 - __clz((int)n));
+  uint32_t cur[M];
+  {
+    const uint64_t v = a[hb - 1];
+#pragma unroll
+    for (int m = 0; m < M; ++m) cur[m] = v <= key[m] ? n - hb : 0u;
+  }
+  for (uint32_t step = hb >> 1; step >= 1; step >>= 1) {
+    uint64_t v[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) v[m] = a[cur[m] + step - 1];
+#pragma unroll
+    for (int m = 0; m < M; ++m) cur[m] = v[m] <= key[m] ? cur[m] + step : cur[m];
+  }
+  uint64_t v[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) v[m] = a[cur[m]];
+#pragma unroll
+  for (int m = 0; m < M; ++m) out[m] = cur[m] + (v[m] <= key[m] ? 1u : 0u);
+}
+
+__global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __restrict__ vlist,
+                                                            const float* __restrict__ wgt,
+                                                            AliasEntry* __restrict__ table,
+                                                            int8_t* __restrict__ valid,
+                                                            RowRef* __restrict__ deferred,
+                                                            uint32_t* __restrict__ n_deferred) {
+  __shared__ uint64_t s_sh[ST_CAP];    // surplus prefix of the row's h-th heavy
+  __shared__ uint16_t s_slot[ST_CAP];  // its span slot
+  __shared__ WSum3 s_w[ST_NW];
+  __shared__ uint64_t s_a[ST_NW], s_d[ST_NW];
+  __shared__ uint32_t s_c[ST_NW];
+  const RowRef rr = vlist[blockIdx.x];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  StreamRow r;
+  r.base = rr.off & ~3u;
+  r.lead = rr.off - r.base;
+  r.span = r.lead + rr.d;
+  const uint32_t nch = (r.span + ST_CH - 1) / ST_CH;
+
+  // ---- pass A: exact sum
+  WSum3 sum{0.0, 0.0, 0.0};
+  for (uint32_t c = 0; c < nch; ++c) {
+    double wd[ST_PER];
+    load_chunk(wgt, r, c, tid, wd);
+#pragma unroll
+    for (int j = 0; j < ST_PER; ++j) wsum3_add(sum, wd[j]);
+  }
+  sum = group_sum_wsum3<64>(sum);
+  if (lane == 0) s_w[wave] = sum;
+  __syncthreads();
+  sum = s_w[0];
+#pragma unroll
+  for (int i = 1; i < ST_NW; ++i) {
+    sum.top += s_w[i].top;
+    sum.mid += s_w[i].mid;
+    sum.low += s_w[i].low;
+  }
+  if (sum.top + sum.mid + sum.low == 0.0) {
+    for (uint32_t c = 0; c < nch; ++c)
+#pragma unroll
+      for (int j = 0; j < ST_PER; ++j) {
+        const uint32_t idx = c * ST_CH + (uint32_t)ST_PER * tid + j;
+        if (idx >= r.lead && idx < r.span) table[r.base + idx] = AliasEntry{0.0f, SKY_INVALID};
+      }
+    if (tid == 0) valid[rr.v] = 0;
+    return;
+  }
+  const Ledger L = make_ledger_small(rr.d, wsum3_to_double(sum));
+
+  // ---- pass B: the heavies, in slot order, with their surplus prefix
+  uint64_t carry_u = 0, sd = 0;
+  uint32_t carry_c = 0;
+  bool overflow = false;
+  for (uint32_t c = 0; c < nch; ++c) {
+    double wd[ST_PER];
+    const uint32_t live = load_chunk(wgt, r, c, tid, wd);
+    uint64_t u[ST_PER];
+    uint64_t su = 0;
+    uint32_t heavy = 0;
+#pragma unroll
+    for (int j = 0; j < ST_PER; ++j) {
+      const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
+      if (e.heavy) {
+        su += e.amount;
+        heavy |= 1u << j;
+      } else {
+        sd += e.amount;
+      }
+      u[j] = su;
+    }
+    uint64_t ex_u, tot_u;
+    uint32_t ex_c, tot_c;
+    stream_excl(su, (uint32_t)__popc(heavy), s_a, s_c, ex_u, ex_c, tot_u, tot_c);
+    if (carry_c + tot_c > ST_CAP) {  // uniform
+      overflow = true;
+      break;
+    }
+    uint32_t rank = carry_c + ex_c;
+#pragma unroll
+    for (int j = 0; j < ST_PER; ++j)
+      if ((heavy >> j) & 1) {
+        s_sh[rank] = carry_u + ex_u + u[j];
+        s_slot[rank] = (uint16_t)(c * ST_CH + (uint32_t)ST_PER * tid + j);
+        ++rank;
+      }
+    carry_u += tot_u;
+    carry_c += tot_c;
+  }
+  if (overflow) {
+    if (tid == 0) deferred[atomicAdd(n_deferred, 1u)] = rr;
+    return;
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) sd += shfl_xor_u64(sd, m);
+  if (lane == 0) s_d[wave] = sd;
+  __syncthreads();  // the heavy list and s_d are complete
+  uint64_t total_l = 0;
+#pragma unroll
+  for (int i = 0; i < ST_NW; ++i) total_l += s_d[i];
+  const uint32_t nh = carry_c;
+  const uint64_t total_h = carry_u;
+  const uint32_t last_heavy = nh ? (uint32_t)s_slot[nh - 1] : NONE32;  // span slot
+
+  // ---- pass C: every entry
+  uint64_t carry_d = 0;
+  carry_c = 0;
+  for (uint32_t c = 0; c < nch; ++c) {
+    double wd[ST_PER];
+    const uint32_t live = load_chunk(wgt, r, c, tid, wd);
+    float op[ST_PER];
+    uint64_t key[ST_PER], dl[ST_PER];
+    uint32_t heavy = 0;
+    uint64_t run = 0;
+#pragma unroll
+    for (int j = 0; j < ST_PER; ++j) {
+      const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
+      op[j] = (float)e.p;
+      key[j] = run;
+      dl[j] = e.heavy ? 0 : e.amount;
+      run += dl[j];
+      if (e.heavy) heavy |= 1u << j;
+    }
+    uint64_t ex_d, tot_d;
+    uint32_t ex_c, tot_c;
+    stream_excl(run, (uint32_t)__popc(heavy), s_a, s_c, ex_d, ex_c, tot_d, tot_c);
+    uint32_t at[ST_PER];
+#pragma unroll
+    for (int j = 0; j < ST_PER; ++j) {
+      key[j] += carry_d + ex_d;  // deficits of the row before this slot
+      at[j] = 0;
+    }
+    if (nh) count_le<ST_PER>(s_sh, nh, key, at);  // heavies whose surplus prefix is <= key
+    const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
+#pragma unroll
+    for (int j = 0; j < ST_PER; ++j) {
+      if (!((live >> j) & 1)) continue;
+      const uint32_t idx = pos0 + j;
+      if ((heavy >> j) & 1) {
+        const uint32_t hr = carry_c + ex_c + (uint32_t)__popc(heavy & ((1u << j) - 1));
+        if (hr + 1 >= nh || s_sh[hr] > total_l) {
+          table[r.base + idx] = AliasEntry{1.0f, idx - r.lead};
+        } else {
+          table[r.base + idx].alias = (uint32_t)s_slot[hr + 1] - r.lead;
+        }
+      } else {
+        uint32_t b = at[j];
+        const uint32_t a = b < nh ? (uint32_t)s_slot[b] : (nh ? last_heavy : idx);
+        table[r.base + idx] = AliasEntry{op[j], a - r.lead};
+        // heavies whose surplus prefix lies in (key, key + D]: this light finishes them
+        const uint64_t sl = key[j] + dl[j];
+        while (b < nh && s_sh[b] <= sl) {
+          if (b + 1 < nh) table[r.base + s_slot[b]].prob = residual_prob(L.one + s_sh[b] - sl, L);
+          ++b;
+        }
+      }
+    }
+    carry_d += tot_d;
+    carry_c += tot_c;
+  }
+  (void)total_h;
+  if (tid == 0) valid[rr.v] = 1;
+}
+
+namespace {
+struct StreamScratch {
+  RowRef* deferred = nullptr;
+  uint32_t* n_deferred = nullptr;
+  uint32_t cap = 0;
+};
+StreamScratch g_stream;
+}  // namespace
+
+// Builds the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each).  Rows whose heavies do not fit the
+// LDS list are returned in *deferred (device array owned by this file, valid until the next call).
+int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n, const RowRef** deferred,
+                      uint32_t* n_deferred) {
+  StreamScratch& sc = g_stream;
+  *deferred = nullptr;
+  *n_deferred = 0;
+  if (n == 0) return SKY_OK;
+  hipStream_t st = g->stream;
+  if (sc.cap < n) {
+    if (sc.deferred) SKY_HIP(hipFree(sc.deferred));
+    sc.deferred = nullptr;
+    sc.cap = 0;
+    SKY_HIP(hipMalloc((void**)&sc.deferred, (size_t)n * sizeof(RowRef)));
+    sc.cap = n;
+  }
+  if (!sc.n_deferred) SKY_HIP(hipMalloc((void**)&sc.n_deferred, 4));
+  SKY_HIP(hipMemsetAsync(sc.n_deferred, 0, 4, st));
+  hipLaunchKernelGGL(build_stream_kernel, dim3(n), dim3(ST_T), 0, st, rows_list, g->adjwgt, g->table, g->valid,
+                     sc.deferred, sc.n_deferred);
+  *deferred = sc.deferred;
+  return SKY_OK;
+}
+
+// Number of rows the last build_rows_stream call deferred (synchronises the stream).
+int stream_deferred_count(sky_graph* g, uint32_t* n_deferred) {
+  *n_deferred = 0;
+  if (!g_stream.n_deferred) return SKY_OK;
+  SKY_HIP(hipMemcpyAsync(n_deferred, g_stream.n_deferred, 4, hipMemcpyDeviceToHost, g->stream));
+  SKY_HIP(hipStreamSynchronize(g->stream));
+  return SKY_OK;
+}
+
+}  // namespace sky

@@ -40,8 +40,9 @@ enum BuildClass : int {
   CLS_LDS_W2 = 8,  // deg <= 509       one wavefront, 8 entries per lane
   CLS_MW2 = 9,     // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
   CLS_MW16 = 23,   //                  class CLS_MW2 + nw - 2
-  CLS_HUGE = 24,   // deg > 8189       built tile by tile by the whole GPU
-  CLS_COUNT = 25
+  CLS_STREAM = 24, // deg <= 65533     one workgroup streams the row, its heavies stay in LDS
+  CLS_HUGE = 25,   // above            built tile by tile by the whole GPU
+  CLS_COUNT = 26
 };
 
 // One listed row of a degree class: the build kernels read where the row lies from the list itself
@@ -72,6 +73,10 @@ constexpr uint32_t TILED_TILE = 1024;  // slots per tile of the tile-parallel pa
 int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
                      uint64_t edges);
 void set_tiled_max_tiles(uint32_t n);
+constexpr uint32_t STREAM_MAX_DEG = 65533;  // longest row of the streaming class
+int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n, const RowRef** deferred,
+                      uint32_t* n_deferred);
+int stream_deferred_count(sky_graph* g, uint32_t* n_deferred);
 void set_row_merge(bool on);
 uint32_t tiled_max_tiles();
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,

@@ -143,3 +143,20 @@ def test_search_variant_of_the_row_kernels_gives_the_same_table(orc):
     finally:
         capi.set_option("row_merge", 1)
     build_and_compare(orc, xadj, adjncy, w, "row_merge=1")
+
+
+@pytest.mark.parametrize("dist", ["lognormal2", "uniform", "nearequal", "sparse", "fewlights", "fewheavies"])
+def test_rows_streamed_by_one_workgroup(orc, dist):
+    # rows of 8190..65533 entries: heavies kept in LDS ("fewlights" has more heavies than fit: those rows are
+    # handed to the tile-parallel path); 65534 is the first degree of the tile-parallel class
+    from helpers import weights
+    rng = np.random.default_rng(31)
+    degs = [8190, 8191, 7, 8193, 12288, 2, 12289, 16385, 1, 30000, 65533, 65534, 0, 9001]
+    xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=4096)
+    if dist == "fewlights":
+        w = np.where(rng.random(len(w)) < 0.01, 0.01, 1.01).astype(np.float32)
+    elif dist == "fewheavies":
+        w = np.where(rng.random(len(w)) < 0.001, 1000.0, 0.5).astype(np.float32)
+    else:
+        w = weights(len(w), rng, dist)
+    build_and_compare(orc, xadj, adjncy, w, "stream/" + dist)
