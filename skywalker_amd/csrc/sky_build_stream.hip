@@ -31,17 +31,29 @@ struct StreamRow {
   uint32_t base, lead, span;
 };
 
-// The 8 weights of this thread in chunk c (span slots c*ST_CH + 8*tid ...), clamped, as doubles; 0 outside
-// the row.  Returns the mask of slots that belong to the row.
-__device__ __forceinline__ uint32_t load_chunk(const float* __restrict__ wgt, const StreamRow& r, uint32_t c, int tid,
-                                               double (&wd)[ST_PER]) {
+// The 8 weights of this thread in chunk c (span slots c*ST_CH + 8*tid ...) as loaded; zeros past the row.
+struct RawChunk {
+  float4 q[ST_PER / 4];
+};
+__device__ __forceinline__ RawChunk fetch_chunk(const float* __restrict__ wgt, const StreamRow& r, uint32_t c,
+                                                int tid) {
+  RawChunk x;
+#pragma unroll
+  for (int q = 0; q < ST_PER / 4; ++q) {
+    const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
+    x.q[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pos < r.span) x.q[q] = *reinterpret_cast<const float4*>(wgt + r.base + pos);
+  }
+  return x;
+}
+// Clamped weights as doubles (0 outside the row) and the mask of slots that belong to the row.
+__device__ __forceinline__ uint32_t unpack_chunk(const RawChunk& x, const StreamRow& r, uint32_t c, int tid,
+                                                 double (&wd)[ST_PER]) {
   uint32_t live = 0;
 #pragma unroll
   for (int q = 0; q < ST_PER / 4; ++q) {
     const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
-    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (pos < r.span) x = *reinterpret_cast<const float4*>(wgt + r.base + pos);
-    const float xs[4] = {x.x, x.y, x.z, x.w};
+    const float xs[4] = {x.q[q].x, x.q[q].y, x.q[q].z, x.q[q].w};
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const uint32_t idx = pos + k;
@@ -129,12 +141,16 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
 
   // ---- pass A: exact sum
   WSum3 sum{0.0, 0.0, 0.0};
+  RawChunk nx = fetch_chunk(wgt, r, 0, tid);  // every loop below requests chunk c + 1 before it works on chunk c
   for (uint32_t c = 0; c < nch; ++c) {
+    const RawChunk cur = nx;
+    if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
     double wd[ST_PER];
-    load_chunk(wgt, r, c, tid, wd);
+    unpack_chunk(cur, r, c, tid, wd);
 #pragma unroll
     for (int j = 0; j < ST_PER; ++j) wsum3_add(sum, wd[j]);
   }
+  nx = fetch_chunk(wgt, r, 0, tid);
   sum = group_sum_wsum3<64>(sum);
   if (lane == 0) s_w[wave] = sum;
   __syncthreads();
@@ -162,8 +178,10 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   uint32_t carry_c = 0;
   bool overflow = false;
   for (uint32_t c = 0; c < nch; ++c) {
+    const RawChunk cur = nx;
+    if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
     double wd[ST_PER];
-    const uint32_t live = load_chunk(wgt, r, c, tid, wd);
+    const uint32_t live = unpack_chunk(cur, r, c, tid, wd);
     uint64_t u[ST_PER];
     uint64_t su = 0;
     uint32_t heavy = 0;
@@ -214,9 +232,12 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   // ---- pass C: every entry
   uint64_t carry_d = 0;
   carry_c = 0;
+  nx = fetch_chunk(wgt, r, 0, tid);
   for (uint32_t c = 0; c < nch; ++c) {
+    const RawChunk cur = nx;
+    if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
     double wd[ST_PER];
-    const uint32_t live = load_chunk(wgt, r, c, tid, wd);
+    const uint32_t live = unpack_chunk(cur, r, c, tid, wd);
     float op[ST_PER];
     uint64_t key[ST_PER], dl[ST_PER];
     uint32_t heavy = 0;
