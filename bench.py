@@ -37,14 +37,15 @@ TRAFFIC_PER_EDGE = {"tiled_emit": 20.8, "tiled_sum": 4.3, "tiled_totals": 4.4, "
                     "lds_w1": 14.5, "wave64": 16.6}
 WALK_TRAFFIC_PER_STEP = 398.6  # walk_offline_kernel, same source
 KERNEL_OF = {  # build_profile entry -> kernel symbol
-    "bin": "bin_count_kernel+bin_scatter_kernel", "g2": "build_group_kernel<2>", "g4": "build_group_kernel<4>",
-    "g8": "build_group_kernel<8>", "g16": "build_group_kernel<16>", "g32": "build_group_kernel<32>", "lds_w1": "build_merge_kernel<64,1>",
+    "bin": "bin_count_kernel+bin_scatter_kernel", "lds_w1": "build_merge_kernel<64,1>",
     "lds_w2": "build_merge_kernel<64,2>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
     "streamed": "huge_prefix_kernel+build_huge_kernel", "stream": "build_stream_kernel",
     "stream_deferred": "tile-parallel path for rows deferred by build_stream_kernel",
 }
+KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
+                  for g in (2, 4, 8, 16, 32) for x in ("", "x")})
 KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,2>" % (64 * nw) for nw in range(2, 17)})
 
 

@@ -33,11 +33,13 @@ namespace sky {
 __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d == 0) return CLS_EMPTY;
   if (d <= 2) return CLS_TINY;
+  // the 6-slot variants of the narrow groups (CLS_G2X .. CLS_G16X) cost more per edge than they gain in fill
   if (d <= 5) return CLS_G2;
   if (d <= 13) return CLS_G4;
   if (d <= 29) return CLS_G8;
   if (d <= 61) return CLS_G16;
   if (d <= 125) return CLS_G32;
+  if (d <= 191) return CLS_G32X;
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
@@ -151,41 +153,59 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
 }
 
 // ---------------------------------------------------------------- 2..32 lanes per row
-// G lanes share one row of at most 4 * G slots (counted from the row's 16-byte aligned start); every
-// lane holds one aligned quad of weights, so a wavefront carries 64 / G rows and the per-row steps
-// that do not depend on the row length (exact sum, ledger, scans) are paid once per 64 / G rows.
-// Prefix sums run over the group by DPP; SL and SH of every slot go to a per-group LDS strip
-// padded to 4 * G slots (slots outside the row add nothing), which each entry then searches
-// once with a fixed number of probes; the heavies' slots, compacted by rank, give "next heavy"
-// and "last heavy".  The rank rides in bits 52..63 of the SH scan.
+// G lanes share one row of at most PER * G slots, counted from the row's aligned start (16 bytes for
+// PER = 4, 8 bytes for PER = 6); every lane holds PER consecutive weights, so a wavefront carries
+// 64 / G rows and the per-row steps that do not depend on the row length (exact sum, ledger, scans)
+// are paid once per 64 / G rows.  Prefix sums run over the group by DPP; SL and SH of every slot go
+// to a per-group LDS strip padded to PER * G slots (slots outside the row add nothing), which each
+// entry then searches once with a fixed number of probes; the heavies' slots, compacted by rank,
+// give "next heavy" and "last heavy".  The rank rides in bits 52..63 of the SH scan.
 constexpr uint64_t GROUP_CNT = 1ull << 52;
 
-template <int G>
+template <int G, int PER>
 __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restrict__ vlist, uint32_t count,
                                                           const float* __restrict__ wgt,
                                                           AliasEntry* __restrict__ table,
                                                           int8_t* __restrict__ valid) {
-  constexpr uint32_t SLOTS = 4 * G;
-  __shared__ uint64_t s_pre[2048];  // [0, 1024): SL of every slot of the block; [1024, 2048): SH
-  __shared__ uint8_t s_hs[1024];    // per group: row-local slot of its h-th heavy
+  static_assert(PER == 4 || PER == 6, "a lane loads one float4 or three float2");
+  constexpr uint32_t SLOTS = PER * G;
+  constexpr uint32_t HB = PER == 4 ? SLOTS : SLOTS / 3 * 2;  // largest power of two <= SLOTS
+  constexpr uint32_t ALIGN = PER == 4 ? 4 : 2;               // the row's slots start at a multiple of this
+  constexpr uint32_t BLK = 256 * PER;                        // slots of one block's strips
+  __shared__ uint64_t s_pre[2 * BLK];  // [0, BLK): SL of every slot of the block; [BLK, 2 * BLK): SH
+  __shared__ uint8_t s_hs[BLK];        // per group: row-local slot of its h-th heavy
   const uint32_t grp = (blockIdx.x * 256u + threadIdx.x) / G;
   const int gl = threadIdx.x & (G - 1);
   const int lane = lane_id();
-  const uint32_t gbase = 4u * (threadIdx.x - gl);  // first LDS slot of the group
+  const uint32_t gbase = (uint32_t)PER * (threadIdx.x - gl);  // first LDS slot of the group
   RowRef rr{0, 0, 0, 0};
   if (grp < count) rr = vlist[grp];
   const uint32_t off = rr.off, d = rr.d;
-  const uint32_t base = off & ~3u, lead = off - base, span = d ? lead + d : 0;
-  const uint32_t pos = 4u * gl;
+  const uint32_t base = off & ~(ALIGN - 1), lead = off - base, span = d ? lead + d : 0;
+  const uint32_t pos = (uint32_t)PER * gl;
 
-  float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (pos < span) x = *reinterpret_cast<const float4*>(wgt + base + pos);
-  const float xs[4] = {x.x, x.y, x.z, x.w};
-  double wd[4];
+  float xs[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) xs[k] = 0.0f;
+  if (PER == 4) {
+    if (pos < span) {
+      const float4 x = *reinterpret_cast<const float4*>(wgt + base + pos);
+      xs[0] = x.x; xs[1] = x.y; xs[2] = x.z; xs[3] = x.w;
+    }
+  } else {
+#pragma unroll
+    for (int h = 0; h < PER / 2; ++h)
+      if (pos + 2 * h < span) {
+        const float2 x = *reinterpret_cast<const float2*>(wgt + base + pos + 2 * h);
+        xs[2 * h] = x.x;
+        xs[2 * h + 1] = x.y;
+      }
+  }
+  double wd[PER];
   uint32_t live = 0;
   WSum3 S{0.0, 0.0, 0.0};
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < PER; ++k) {
     const uint32_t idx = pos + k;
     const bool in = idx >= lead && idx < span;
     if (in) live |= 1u << k;
@@ -197,12 +217,12 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
   Ledger L = make_ledger_small(d, wsum3_to_double(S));
   if (!row_ok) L.scale = 0.0;
 
-  uint64_t dl[4], sl[4], sh[4];
-  float op[4];
+  uint64_t dl[PER], sl[PER], sh[PER];
+  float op[PER];
   uint32_t heavy = 0;
   uint64_t ra = 0, rb = 0;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < PER; ++k) {
     const Entry e = classify_small(wd[k], (live >> k) & 1, L);
     dl[k] = e.heavy ? 0 : e.amount;
     ra += dl[k];
@@ -215,11 +235,11 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
   const uint64_t ia = group_scan_u64<G>(ra), ib = group_scan_u64<G>(rb);
   const uint32_t nh = (uint32_t)(shfl_u64(ib, (lane - gl) + G - 1) >> 52);
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < PER; ++k) {
     sl[k] += ia - ra;
     sh[k] += ib - rb;
     s_pre[gbase + pos + k] = sl[k];
-    s_pre[1024 + gbase + pos + k] = sh[k] & (GROUP_CNT - 1);
+    s_pre[BLK + gbase + pos + k] = sh[k] & (GROUP_CNT - 1);
     if ((heavy >> k) & 1) s_hs[gbase + (uint32_t)(sh[k] >> 52) - 1] = (uint8_t)(pos + k - lead);
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -227,26 +247,27 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
   // light: first slot with SH > SL - D.  heavy: first slot with SL >= SH, i.e. SL > SH - 1.
-  uint32_t arr[4], at[4];
-  uint64_t key[4];
+  // The first probe narrows the answer to a window of HB slots that ends inside the strip.
+  uint32_t arr[PER], at[PER];
+  uint64_t key[PER];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < PER; ++k) {
     const bool hv = (heavy >> k) & 1;
-    arr[k] = gbase + (hv ? 0u : 1024u);
+    arr[k] = gbase + (hv ? 0u : BLK);
     key[k] = hv ? (sh[k] & (GROUP_CNT - 1)) - 1 : sl[k] - dl[k];
-    at[k] = 0;
+    at[k] = HB == SLOTS ? 0u : (s_pre[arr[k] + HB - 1] <= key[k] ? SLOTS - HB : 0u);
   }
 #pragma unroll
-  for (uint32_t step = SLOTS / 2; step >= 1; step >>= 1) {
-    uint64_t v[4];
+  for (uint32_t step = HB / 2; step >= 1; step >>= 1) {
+    uint64_t v[PER];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] = s_pre[arr[k] + at[k] + step - 1];
+    for (int k = 0; k < PER; ++k) v[k] = s_pre[arr[k] + at[k] + step - 1];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) at[k] += v[k] <= key[k] ? step : 0u;
+    for (int k = 0; k < PER; ++k) at[k] += v[k] <= key[k] ? step : 0u;
   }
-  uint32_t oa[4];
+  uint32_t oa[PER];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < PER; ++k) {
     const uint64_t v = s_pre[arr[k] + at[k]];
     const bool found = v > key[k];
     const uint32_t self = pos + k - lead;
@@ -267,13 +288,18 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
       oa[k] = SKY_INVALID;
     }
   }
-  if (pos < span) {
-    if (pos >= lead && pos + 4 <= span) {
-      store_entries4(table + base + pos, op, oa);
-    } else {
+  // pairs of entries start at multiples of 16 bytes
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if ((live >> k) & 1) table[base + pos + k] = AliasEntry{op[k], oa[k]};
+  for (int h = 0; h < PER / 2; ++h) {
+    const uint32_t m = (live >> (2 * h)) & 3u;
+    AliasEntry* t = table + base + pos + 2 * h;
+    if (m == 3u) {
+      *reinterpret_cast<uint4*>(t) =
+          make_uint4(__float_as_uint(op[2 * h]), oa[2 * h], __float_as_uint(op[2 * h + 1]), oa[2 * h + 1]);
+    } else if (m == 1u) {
+      t[0] = AliasEntry{op[2 * h], oa[2 * h]};
+    } else if (m == 2u) {
+      t[1] = AliasEntry{op[2 * h + 1], oa[2 * h + 1]};
     }
   }
   if (gl == 0 && d) valid[rr.v] = row_ok;
@@ -945,11 +971,16 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
   };
-  SKY_TRY(grp(CLS_G2, build_group_kernel<2>, 2, "g2"));
-  SKY_TRY(grp(CLS_G4, build_group_kernel<4>, 4, "g4"));
-  SKY_TRY(grp(CLS_G8, build_group_kernel<8>, 8, "g8"));
-  SKY_TRY(grp(CLS_G16, build_group_kernel<16>, 16, "g16"));
-  SKY_TRY(grp(CLS_G32, build_group_kernel<32>, 32, "g32"));
+  SKY_TRY(grp(CLS_G2, build_group_kernel<2, 4>, 2, "g2"));
+  SKY_TRY(grp(CLS_G2X, build_group_kernel<2, 6>, 2, "g2x"));
+  SKY_TRY(grp(CLS_G4, build_group_kernel<4, 4>, 4, "g4"));
+  SKY_TRY(grp(CLS_G4X, build_group_kernel<4, 6>, 4, "g4x"));
+  SKY_TRY(grp(CLS_G8, build_group_kernel<8, 4>, 8, "g8"));
+  SKY_TRY(grp(CLS_G8X, build_group_kernel<8, 6>, 8, "g8x"));
+  SKY_TRY(grp(CLS_G16, build_group_kernel<16, 4>, 16, "g16"));
+  SKY_TRY(grp(CLS_G16X, build_group_kernel<16, 6>, 16, "g16x"));
+  SKY_TRY(grp(CLS_G32, build_group_kernel<32, 4>, 32, "g32"));
+  SKY_TRY(grp(CLS_G32X, build_group_kernel<32, 6>, 32, "g32x"));
 
   auto lds = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
     const uint32_t cnt = counts[cls];

@@ -31,18 +31,23 @@ namespace sky {
 enum BuildClass : int {
   CLS_EMPTY = 0,   // deg 0            handled while binning
   CLS_TINY = 1,    // deg 1..2         one lane per vertex, handled while binning
-  CLS_G2 = 2,      // deg 3..5         2 lanes per row, one quad of slots per lane
-  CLS_G4 = 3,      // deg <= 13        4 lanes per row
-  CLS_G8 = 4,      // deg <= 29
-  CLS_G16 = 5,     // deg <= 61
-  CLS_G32 = 6,     // deg <= 125
-  CLS_LDS_W1 = 7,  // deg <= 253       one wavefront, LDS prefix arrays, 4 entries per lane
-  CLS_LDS_W2 = 8,  // deg <= 509       one wavefront, 8 entries per lane
-  CLS_MW2 = 9,     // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
-  CLS_MW16 = 23,   //                  class CLS_MW2 + nw - 2
-  CLS_STREAM = 24, // deg <= 65533     one workgroup streams the row, its heavies stay in LDS
-  CLS_HUGE = 25,   // above            built tile by tile by the whole GPU
-  CLS_COUNT = 26
+  CLS_G2 = 2,      // deg 3..5         2 lanes per row, 4 slots per lane
+  CLS_G2X = 3,     // deg <= 11        2 lanes, 6 slots per lane
+  CLS_G4 = 4,      // deg <= 13        4 lanes, 4 slots
+  CLS_G4X = 5,     // deg <= 23        4 lanes, 6 slots
+  CLS_G8 = 6,      // deg <= 29
+  CLS_G8X = 7,     // deg <= 47
+  CLS_G16 = 8,     // deg <= 61
+  CLS_G16X = 9,    // deg <= 95
+  CLS_G32 = 10,    // deg <= 125
+  CLS_G32X = 11,   // deg <= 191
+  CLS_LDS_W1 = 12, // deg <= 253       one wavefront, LDS prefix arrays, 4 entries per lane
+  CLS_LDS_W2 = 13, // deg <= 509       one wavefront, 8 entries per lane
+  CLS_MW2 = 14,    // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
+  CLS_MW16 = 28,   //                  class CLS_MW2 + nw - 2
+  CLS_STREAM = 29, // deg <= 65533     one workgroup streams the row, its heavies stay in LDS
+  CLS_HUGE = 30,   // above            built tile by tile by the whole GPU
+  CLS_COUNT = 31
 };
 
 // One listed row of a degree class: the build kernels read where the row lies from the list itself
