@@ -84,6 +84,34 @@ def test_cli_offline_deepwalk_matches_oracle(tmp_path, orc):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("table", [False, True])
+def test_cli_node2vec_matches_oracle(tmp_path, orc, table):
+    # --node2vec runs the rejection sampler on the first-order tables; --n2v_table the table per step
+    xadj, adjncy = orc.rmat_csr(11, 8, 7)
+    w = (orc.gen_weights(orc.W_UNIFORM, 7, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "n2v.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    cmd = [os.path.join(HOST, "skywalker"), "--node2vec", "--bias=1", "--input", p, "-n", "400", "--d", "15", "--p", "2",
+           "--q", "0.5", "--printresult", "--seed", "9"]
+    rc, out, err = run(cmd + (["--n2v_table"] if table else []))
+    assert rc == 0, err
+    lines = out.splitlines()
+    seeds = np.arange(400, dtype=np.uint32)
+    wf = w.astype(np.float32)
+    if table:
+        paths, lengths, sampled = orc.walk_online(xadj, adjncy, wf, 1, 2.0, 0.5, seeds, 15, 0.0, 9)
+    else:
+        prob, alias, valid = orc.alias_build(xadj, wf)
+        paths, lengths, sampled = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, 2.0, 0.5, seeds, 15, 0.0, 9)
+    for j in range(3):
+        i = lines.index("%drd path len %d " % (j, lengths[j]))
+        got = [int(x) for x in lines[i + 1].split()]
+        assert got == paths[j, :min(lengths[j], 16)].tolist()
+    sample_ms, mseps = (float(l.strip()) for l in lines[-2:])
+    assert abs(mseps - sampled / (sample_ms * 1e-3) / 1e6) <= 0.02 * mseps + 0.02
+
+
+@pytest.mark.gpu
 def test_cli_online_sage_and_csv(tmp_path, orc):
     xadj, adjncy = orc.rmat_csr(11, 8, 2)
     w = (orc.gen_weights(orc.W_UNIFORM, 2, len(adjncy), 1.0, 100.0)).astype(np.uint32)
