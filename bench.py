@@ -202,7 +202,7 @@ def main():
         for nm, ms, edges in r["profile"]:
             p = prof.setdefault(nm, [0.0, edges])
             p[0] += ms / len(rec)
-    dom = max(prof, key=lambda k: prof[k][0])
+    dom = max((k for k in prof if prof[k][1] > 0), key=lambda k: prof[k][0])  # brackets without edges are host round trips
     dom_ms, dom_edges = prof[dom]
     dom_bytes = BYTES_PER_EDGE.get(dom, 12) * dom_edges
     out = {

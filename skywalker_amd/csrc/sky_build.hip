@@ -969,7 +969,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, st, vlist + starts[cls],
                          cnt, g->adjwgt, g->table, g->valid);
     }
-    return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
+    return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
   SKY_TRY(grp(CLS_G2, build_group_kernel<2, 4>, 2, "g2"));
   SKY_TRY(grp(CLS_G2X, build_group_kernel<2, 6>, 2, "g2x"));
@@ -989,7 +989,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
                          g->table, g->valid);
     }
-    return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
+    return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
   auto mrg = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
     const uint32_t cnt = counts[cls];
@@ -998,7 +998,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
                          g->table, g->valid);
     }
-    return tm ? tm->mark(name, host.edges[cls]) : SKY_OK;
+    return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
   static const char* const mw_name[15] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9",
                                           "mw10", "mw11", "mw12", "mw13", "mw14", "mw15", "mw16"};
@@ -1028,21 +1028,18 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
   }
 
+  const RowRef* deferred = nullptr;
   if (counts[CLS_STREAM]) {
     const uint32_t cnt = counts[CLS_STREAM];
-    uint32_t skipped = 0;
     if (g_row_merge) {
-      const RowRef* deferred = nullptr;
       uint32_t nd = 0;
       SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], cnt, &deferred, &nd));
-      if (tm) SKY_TRY(tm->mark("stream", host.edges[CLS_STREAM]));
-      SKY_TRY(stream_deferred_count(g, &nd));
-      if (nd) SKY_TRY(build_rows_tiled(g, deferred, nd, &skipped, nullptr, 0));  // more heavies than LDS holds
     } else {
+      uint32_t skipped = 0;
       SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_STREAM], cnt, &skipped, nullptr, 0));
+      if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles is too small for rows of up to 65533 entries");
     }
-    if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles is too small for rows of up to 65533 entries");
-    if (tm) SKY_TRY(tm->mark("stream_deferred", 0));
+    if (tm) SKY_TRY(tm->mark("stream", host.edges[CLS_STREAM]));
   }
   if (counts[CLS_HUGE]) {
     const uint32_t cnt = counts[CLS_HUGE];
@@ -1074,7 +1071,17 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
                          g->table, g->valid);
     }
   }
-  if (tm) SKY_TRY(tm->mark("streamed", 0));
+  if (tm && counts[CLS_HUGE]) SKY_TRY(tm->mark("streamed", 0));
+  if (deferred) {  // rows the streaming kernel left alone (more heavies than its LDS list holds); asked last,
+                   // so that the host round trip does not idle the GPU between two classes
+    uint32_t nd = 0, skipped = 0;
+    SKY_TRY(stream_deferred_count(g, &nd));
+    if (nd) {
+      SKY_TRY(build_rows_tiled(g, deferred, nd, &skipped, nullptr, 0));
+      if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles is too small for rows of up to 65533 entries");
+      if (tm) SKY_TRY(tm->mark("stream_deferred", 0));
+    }
+  }
   return SKY_OK;
 }
 
