@@ -359,8 +359,12 @@ int orc_alias_check(const uint32_t* xadj, const float* w, const float* prob, con
     for (int64_t v = 0; v < (int64_t)V; ++v) {
       const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
       long double sum = 0;
-      for (uint32_t i = 0; i < deg; ++i) sum += (long double)clamp_weight(w[off + i]);
-      const bool ok = deg > 0 && sum > 0;
+      u128 fixed = 0;  // a row is valid iff its exact 2^-64 fixed-point sum is not zero (weights below 2^-64 add nothing)
+      for (uint32_t i = 0; i < deg; ++i) {
+        sum += (long double)clamp_weight(w[off + i]);
+        fixed += weight_fixed(clamp_weight(w[off + i]));
+      }
+      const bool ok = deg > 0 && fixed != 0;
       if ((valid[v] != 0) != ok) ++lbv;
       if (!ok) {
         for (uint32_t i = 0; i < deg; ++i)
@@ -375,7 +379,11 @@ int orc_alias_check(const uint32_t* xadj, const float* w, const float* prob, con
       orc_alias_reconstruct_row(prob + off, alias + off, deg, q.data());
       for (uint32_t i = 0; i < deg; ++i) {
         double t = (double)((long double)clamp_weight(w[off + i]) / sum);
-        double err = t > 0 ? std::fabs(q[i] - t) / t : (q[i] == 0 ? 0.0 : 1.0);
+        // shares of a bucket below 1e-30 are at the edge of what a float probability can hold (denormals,
+        // then zero): there only an absolute bound can be asked for
+        double err;
+        if (t * deg < 1e-30) err = q[i] * deg < 2e-30 ? 0.0 : 1.0;
+        else err = std::fabs(q[i] - t) / t;
         if (err > lworst) { lworst = err; lworst_v = (uint32_t)v; }
       }
     }

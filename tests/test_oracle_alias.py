@@ -150,3 +150,25 @@ def test_check_detects_a_wrong_table(orc):
     bad_alias = alias.copy()
     bad_alias[xadj[v] + 1] = (bad_alias[xadj[v] + 1] + 1) % (xadj[v + 1] - xadj[v])
     assert orc.alias_check(xadj, w, prob, bad_alias, valid)["max_rel_err"] > TOL
+
+
+def test_special_weight_values(orc):
+    # NaN, infinities, negatives and -0 count as zero; values above 2^32 as 2^32; weights below 2^-64 add nothing
+    # to the exact sum, so a row made only of them is invalid
+    w = np.array([np.nan, np.inf, -np.inf, -1.0, -0.0, 0.0, 1e-45, 2.0 ** -64, 3e-19, 2.0 ** 32, 2.0 ** 33, 3e38,
+                  1.0, 7.5], np.float32)
+    with np.errstate(all="ignore"):
+        prob, alias, valid = orc.alias_build_row(w)
+        clamped = np.where(np.isnan(w) | (w <= 0), 0.0, np.minimum(w.astype(np.float64), 2.0 ** 32))
+    assert valid == 1
+    q = orc.reconstruct_row(prob, alias)
+    t = clamped / clamped.sum()
+    big = t > 1e-20
+    assert np.allclose(q[big], t[big], rtol=1e-6, atol=0) and np.all(q[~big] < 1e-20)
+    # the four entries clamped to 2^32 (inf, 2^32, 2^33, 3e38) get equal shares
+    assert np.allclose(q[[1, 9, 10, 11]], q[1], rtol=1e-6, atol=0)
+    for tiny in ([1e-30, 1e-25], [1e-45], [2.0 ** -65, 0.0, -2.0]):
+        p2, a2, v2 = orc.alias_build_row(np.array(tiny, np.float32))
+        assert v2 == 0 and np.all(p2 == 0) and np.all(a2 == orc.INVALID)
+    p3, a3, v3 = orc.alias_build_row(np.array([2.0 ** -64, 2.0 ** -64], np.float32))
+    assert v3 == 1 and np.allclose(orc.reconstruct_row(p3, a3), [0.5, 0.5])
