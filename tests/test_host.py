@@ -84,6 +84,24 @@ def test_cli_offline_deepwalk_matches_oracle(tmp_path, orc):
 
 
 @pytest.mark.gpu
+def test_cli_unbiased_walk_is_the_unit_weight_walk(tmp_path, orc):
+    # --bias=0 ignores the weights of the file: uniform neighbour choice through the same tables
+    xadj, adjncy = orc.rmat_csr(11, 8, 3)
+    w = (orc.gen_weights(orc.W_UNIFORM, 3, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "u.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--bias=0", "--ol=0", "--input", p, "-n", "500",
+                        "--d", "12", "--printresult", "--seed", "4"])
+    assert rc == 0, err
+    lines = out.splitlines()
+    prob, alias, valid = orc.alias_build(xadj, np.ones(len(adjncy), np.float32))
+    paths, lengths, sampled = orc.walk_offline(xadj, adjncy, prob, alias, np.arange(500, dtype=np.uint32), 12, 0.0, 4)
+    for j in range(3):
+        i = lines.index("%drd path len %d " % (j, lengths[j]))
+        assert [int(x) for x in lines[i + 1].split()] == paths[j, :min(lengths[j], 13)].tolist()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("table", [False, True])
 def test_cli_node2vec_matches_oracle(tmp_path, orc, table):
     # --node2vec runs the rejection sampler on the first-order tables; --n2v_table the table per step
