@@ -57,6 +57,8 @@ DEFINE_double(pfr, 1.0, "UM prefetching ratio");
 DEFINE_bool(async, false, "using async execution");
 DEFINE_bool(replica, false, "same task for all gpus");
 DEFINE_bool(built, false, "has built table");
+DEFINE_string(savetable, "", "write the alias tables to this file after building them");
+DEFINE_string(loadtable, "", "read the alias tables from this file instead of building them");
 DEFINE_bool(gmem, false, "do not use shmem as buffer");
 DEFINE_bool(newsampler, true, "use new sampler");
 DEFINE_bool(csv, false, "CSV output");
@@ -118,8 +120,19 @@ int main(int argc, char* argv[]) {
   const bool online = FLAGS_ol;
   if (!online) {
     sampler.InitFullForConstruction(1, 0);
-    table_time = ConstructTable(sampler, 1, 0) * 1000;
-    LOG("Max construction time with %u gpu \t%.2f ms\n", 1, table_time);
+    if (!FLAGS_loadtable.empty()) {
+      if (!LoadTable(sampler, FLAGS_loadtable)) {
+        fprintf(stderr, "cannot use table file %s (missing, damaged, or of another graph)\n", FLAGS_loadtable.c_str());
+        return 1;
+      }
+    } else {
+      table_time = ConstructTable(sampler, 1, 0) * 1000;
+      LOG("Max construction time with %u gpu \t%.2f ms\n", 1, table_time);
+    }
+    if (!FLAGS_savetable.empty() && !SaveTable(sampler, FLAGS_savetable)) {
+      fprintf(stderr, "cannot write table file %s\n", FLAGS_savetable.c_str());
+      return 1;
+    }
     FLAGS_built = true;
   }
   if (!FLAGS_rw) {

@@ -212,6 +212,42 @@ inline float ConstructTable(Sampler& sampler, uint ngpu = 1, uint index = 0) {
   return (float)sec;
 }
 
+// Table persistence (the reference has none: every run rebuilds).  File: "SKYTBL01", V, E (u64 each), then
+// prob f32[E], alias u32[E], valid i8[V], little endian.
+inline bool SaveTable(Sampler& sampler, const std::string& path) {
+  const uint64_t V = sampler.ggraph.vtx_num, E = sampler.ggraph.edge_num;
+  std::vector<float> prob(E);
+  std::vector<uint32_t> alias(E);
+  std::vector<int8_t> valid(V);
+  SKY_RT_CALL(sky_alias_download(sampler.ggraph.handle, prob.data(), alias.data(), valid.data()));
+  FILE* f = fopen(path.c_str(), "wb");
+  if (!f) return false;
+  bool ok = fwrite("SKYTBL01", 1, 8, f) == 8 && fwrite(&V, 8, 1, f) == 1 && fwrite(&E, 8, 1, f) == 1;
+  ok = ok && fwrite(prob.data(), 4, E, f) == E && fwrite(alias.data(), 4, E, f) == E;
+  ok = ok && fwrite(valid.data(), 1, V, f) == V;
+  return fclose(f) == 0 && ok;
+}
+inline bool LoadTable(Sampler& sampler, const std::string& path) {
+  const uint64_t V = sampler.ggraph.vtx_num, E = sampler.ggraph.edge_num;
+  FILE* f = fopen(path.c_str(), "rb");
+  if (!f) return false;
+  char magic[8];
+  uint64_t fv = 0, fe = 0;
+  bool ok = fread(magic, 1, 8, f) == 8 && !memcmp(magic, "SKYTBL01", 8) && fread(&fv, 8, 1, f) == 1 &&
+            fread(&fe, 8, 1, f) == 1 && fv == V && fe == E;
+  std::vector<float> prob(ok ? E : 0);
+  std::vector<uint32_t> alias(ok ? E : 0);
+  std::vector<int8_t> valid(ok ? V : 0);
+  ok = ok && fread(prob.data(), 4, E, f) == E && fread(alias.data(), 4, E, f) == E && fread(valid.data(), 1, V, f) == V;
+  fclose(f);
+  if (!ok) return false;
+  SKY_RT_CALL(sky_alias_upload(sampler.ggraph.handle, prob.data(), alias.data(), valid.data()));
+  sampler.ggraph.Refresh();
+  sampler.alias_table = sampler.ggraph.alias_table;
+  sampler.valid = sampler.ggraph.valid;
+  return true;
+}
+
 inline float walk_common(Walker& walker, bool online, const char* who) {
   LOG("%s\n", who);
   double sec = 0;

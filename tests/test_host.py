@@ -84,6 +84,30 @@ def test_cli_offline_deepwalk_matches_oracle(tmp_path, orc):
 
 
 @pytest.mark.gpu
+def test_cli_saved_tables_give_the_same_walks(tmp_path, orc):
+    xadj, adjncy = orc.rmat_csr(11, 8, 5)
+    w = (orc.gen_weights(orc.W_UNIFORM, 5, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p, t = str(tmp_path / "t.w.gr"), str(tmp_path / "t.tbl")
+    write_gr(p, xadj, adjncy, w)
+    common = [os.path.join(HOST, "skywalker"), "--deepwalk", "--bias=1", "--ol=0", "--input", p, "-n", "300", "--d", "10",
+              "--printresult", "--seed", "6"]
+    rc, out1, err = run(common + ["--savetable", t])
+    assert rc == 0, err
+    raw = open(t, "rb").read()
+    V, E = len(xadj) - 1, len(adjncy)
+    assert raw[:8] == b"SKYTBL01" and struct.unpack("<2Q", raw[8:24]) == (V, E) and len(raw) == 24 + 8 * E + V
+    prob, alias, valid = orc.alias_build(xadj, w.astype(np.float32))
+    assert np.array_equal(np.frombuffer(raw, np.float32, E, 24).view(np.uint32), prob.view(np.uint32))
+    assert np.array_equal(np.frombuffer(raw, np.uint32, E, 24 + 4 * E), alias)
+    rc, out2, err = run(common + ["--loadtable", t])
+    assert rc == 0, err
+    keep = lambda o: [l for l in o.splitlines() if l.strip()][:-3]  # everything but the timing lines
+    assert keep(out1)[1:] == keep(out2)[1:] and len(keep(out1)) >= 7
+    rc, _, err = run(common + ["--loadtable", p])  # not a table file
+    assert rc != 0 and "cannot use table file" in err
+
+
+@pytest.mark.gpu
 def test_cli_unbiased_walk_is_the_unit_weight_walk(tmp_path, orc):
     # --bias=0 ignores the weights of the file: uniform neighbour choice through the same tables
     xadj, adjncy = orc.rmat_csr(11, 8, 3)
