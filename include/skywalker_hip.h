@@ -138,11 +138,14 @@ int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, co
  *      ctr_host[4n], key_host[2n] -> out_host[4n]. ---- */
 int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint32_t n, uint32_t* out_host);
 
-/* ---- tuning knobs (no counterpart in the reference).  "tiled_max_tiles": rows of more than 4093 entries are
+/* ---- tuning knobs (no counterpart in the reference).  "tiled_max_tiles": rows too long for one workgroup are
  *      built tile by tile (1024 entries per tile) up to this many tiles (default: no limit); longer rows
- *      are streamed by one workgroup each.  Tests lower it to exercise the streaming kernel.
- *      "row_merge" (default 1): rows of 62..4093 entries pair lights and heavies by a merge of their prefix
- *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table. ---- */
+ *      fall to a kernel in which one workgroup walks the whole row.  Tests lower it to exercise that kernel.
+ *      "row_merge" (default 1): rows of 62..8189 entries pair lights and heavies by a merge of their prefix
+ *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table.
+ *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:
+ *      0 builds, before every step, the rows the walkers stand on; 1 builds every row first and walks as
+ *      sky_walk_offline does; -1 takes whichever is estimated to be faster.  The paths are the same. ---- */
 int sky_set_option(const char* name, long value);
 
 /* ---- per-kernel timing of the last sky_alias_build_all on this graph, for roofline reporting:

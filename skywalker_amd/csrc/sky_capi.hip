@@ -319,6 +319,10 @@ int sky_set_option(const char* name, long value) {
     set_row_merge(value != 0);
     return SKY_OK;
   }
+  if (!strcmp(name, "online_full_build")) {
+    set_online_full_build((int)value);
+    return SKY_OK;
+  }
   return fail(SKY_ERR_ARG, std::string("sky_set_option: unknown option ") + name);
 }
 

@@ -76,6 +76,20 @@ int walk_online_node2vec(sky_graph* g, float p, float q, const uint32_t* seeds, 
                          float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
                          double* seconds);
 
+// -1: decide by the estimate below; 0: always build lazily, step by step; 1: always build every row first.
+static int g_online_full_build = -1;
+void set_online_full_build(int mode) { g_online_full_build = mode < 0 ? -1 : (mode ? 1 : 0); }
+
+// Estimated milliseconds of the two ways to serve a static-bias online walk.  A lazy round costs a
+// host round trip and a handful of small launches (about 1/8 ms measured), and the rounds together
+// build at most min(N * len, V) rows; the full build runs at about 1.3e8 edges per millisecond.
+static bool online_prefers_full_build(const sky_graph* g, uint32_t N, uint32_t len) {
+  if (g_online_full_build >= 0) return g_online_full_build == 1;
+  const double all_ms = (double)g->E / 1.3e8;
+  const double visited = std::min(1.0, (double)N * len / std::max(1u, g->V));
+  return 0.4 + all_ms < 0.125 * len + visited * all_ms;
+}
+
 int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
                 float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
                 double* seconds) {
@@ -83,6 +97,16 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
     return walk_node2vec_reject(g, p, q, seeds, N, len, stop_prob, seed, paths, lengths, sampled, seconds);
   if (bias_kind == SKY_BIAS_NODE2VEC)
     return walk_online_node2vec(g, p, q, seeds, N, len, stop_prob, seed, paths, lengths, sampled, seconds);
+  // Tables that already exist are used as they are.  Otherwise one build of every row, then the
+  // offline kernel, is taken when it is expected to cost less than len rounds of lazy builds, each
+  // of which waits for the host; the paths are the same either way.
+  double build_sec = 0;
+  if (!g->has_tables && N && len && online_prefers_full_build(g, N, len)) SKY_TRY(build_all_tables(g, &build_sec));
+  if (g->has_tables) {
+    SKY_TRY(walk_offline(g, seeds, N, len, stop_prob, seed, paths, lengths, sampled, seconds));
+    if (seconds) *seconds += build_sec;
+    return SKY_OK;
+  }
   hipStream_t st = g->stream;
   unsigned long long* d_sampled = nullptr;
   uint32_t *bitmap = nullptr, *list = nullptr, *d_cnt = nullptr;

@@ -96,6 +96,7 @@ __global__ __launch_bounds__(256) void sample_init_kernel(const uint32_t* __rest
 int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
                 uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds) {
   hipStream_t st = g->stream;
+  if (g->has_tables) online = false;  // every row is already there: nothing to build on the way
   std::vector<uint64_t> width(hops), off(hops), loff(hops, 0);
   uint64_t lps = 0, slen = 0, wd = 1;
   for (uint32_t h = 0; h < hops; ++h) {

@@ -90,13 +90,19 @@ def test_walk_does_not_depend_on_batch_composition(orc):
     assert np.array_equal(full[:1000], part)
 
 
-def test_online_static_walk_equals_offline_and_oracle(orc):
+@pytest.mark.parametrize("mode", [0, 1, -1])
+def test_online_static_walk_equals_offline_and_oracle(orc, mode):
+    # mode 0: rows built step by step as walkers reach them; 1: every row first; -1: the library chooses
     from skywalker_amd import capi
     xadj, adjncy = orc.rmat_csr(13, 8, 6)
     w = orc.gen_weights(orc.W_UNIFORM, 6, len(adjncy), 1.0, 100.0)
     seeds = orc.gen_seeds(3, 1 << 13, 2000)
     g = capi.Graph.upload(xadj, adjncy, w)
-    p_on, l_on, s_on, _ = g.walk_online(capi.BIAS_STATIC, 1.0, 1.0, seeds, 30, 0.1, 5)
+    capi.set_option("online_full_build", mode)
+    try:
+        p_on, l_on, s_on, _ = g.walk_online(capi.BIAS_STATIC, 1.0, 1.0, seeds, 30, 0.1, 5)
+    finally:
+        capi.set_option("online_full_build", -1)
     on = (p_on.to_host((2000, 31)), l_on.to_host())
     g.build_tables()
     p_off, l_off, s_off, _ = g.walk_offline(seeds, 30, 0.1, 5)
