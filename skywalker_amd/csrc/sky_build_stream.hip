@@ -24,7 +24,7 @@ constexpr int ST_T = 512;                 // threads per row
 constexpr int ST_PER = 8;                 // consecutive slots per thread and chunk
 constexpr int ST_CH = ST_T * ST_PER;      // slots per chunk
 constexpr int ST_NW = ST_T / 64;
-constexpr uint32_t ST_CAP = 8064;         // heavies per row kept in LDS: two workgroups share a CU's 160 KB
+constexpr uint32_t ST_CAP = 8063;         // heavies per row kept in LDS (and one sentinel): two workgroups share a CU's 160 KB
 static_assert(STREAM_MAX_DEG + 3 <= 65536, "heavy slots are stored as 16-bit numbers");
 
 struct StreamRow {
@@ -126,8 +126,8 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
                                                             int8_t* __restrict__ valid,
                                                             RowRef* __restrict__ deferred,
                                                             uint32_t* __restrict__ n_deferred) {
-  __shared__ uint64_t s_sh[ST_CAP];    // surplus prefix of the row's h-th heavy
-  __shared__ uint16_t s_slot[ST_CAP];  // its span slot
+  __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the row's h-th heavy
+  __shared__ uint16_t s_slot[ST_CAP + 1];  // its span slot
   __shared__ WSum3 s_w[ST_NW];
   __shared__ uint64_t s_a[ST_NW], s_d[ST_NW];
   __shared__ uint32_t s_c[ST_NW];
@@ -227,7 +227,10 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   for (int i = 0; i < ST_NW; ++i) total_l += s_d[i];
   const uint32_t nh = carry_c;
   const uint64_t total_h = carry_u;
-  const uint32_t last_heavy = nh ? (uint32_t)s_slot[nh - 1] : NONE32;  // span slot
+  if (tid == 0) {  // sentinel after the list; the first barrier of pass C publishes it
+    s_sh[nh] = ~0ull;
+    s_slot[nh] = nh ? s_slot[nh - 1] : (uint16_t)0;
+  }
 
   // ---- pass C: every entry
   uint64_t carry_d = 0;
@@ -239,14 +242,13 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
     double wd[ST_PER];
     const uint32_t live = unpack_chunk(cur, r, c, tid, wd);
     float op[ST_PER];
-    uint64_t key[ST_PER], dl[ST_PER];
+    uint64_t dl[ST_PER];
     uint32_t heavy = 0;
     uint64_t run = 0;
 #pragma unroll
     for (int j = 0; j < ST_PER; ++j) {
       const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
       op[j] = (float)e.p;
-      key[j] = run;
       dl[j] = e.heavy ? 0 : e.amount;
       run += dl[j];
       if (e.heavy) heavy |= 1u << j;
@@ -254,13 +256,18 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
     uint64_t ex_d, tot_d;
     uint32_t ex_c, tot_c;
     stream_excl(run, (uint32_t)__popc(heavy), s_a, s_c, ex_d, ex_c, tot_d, tot_c);
-    uint32_t at[ST_PER];
-#pragma unroll
-    for (int j = 0; j < ST_PER; ++j) {
-      key[j] += carry_d + ex_d;  // deficits of the row before this slot
-      at[j] = 0;
+    // b = heavies whose surplus prefix is <= the deficits before this thread's slots: one search; from
+    // there the thread's lights walk the list, each stopping at its own deficit prefix
+    uint64_t sl = carry_d + ex_d;
+    uint32_t b = 0;
+    if (nh) {
+      const uint64_t k1[1] = {sl};
+      uint32_t o1[1];
+      count_le<1>(s_sh, nh, k1, o1);
+      b = o1[0];
     }
-    if (nh) count_le<ST_PER>(s_sh, nh, key, at);  // heavies whose surplus prefix is <= key
+    uint64_t hv = s_sh[b];          // ~0 once the list is exhausted
+    uint32_t hslot = s_slot[b];     // then: the last heavy
     const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
 #pragma unroll
     for (int j = 0; j < ST_PER; ++j) {
@@ -274,14 +281,14 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
           table[r.base + idx].alias = (uint32_t)s_slot[hr + 1] - r.lead;
         }
       } else {
-        uint32_t b = at[j];
-        const uint32_t a = b < nh ? (uint32_t)s_slot[b] : (nh ? last_heavy : idx);
-        table[r.base + idx] = AliasEntry{op[j], a - r.lead};
-        // heavies whose surplus prefix lies in (key, key + D]: this light finishes them
-        const uint64_t sl = key[j] + dl[j];
-        while (b < nh && s_sh[b] <= sl) {
-          if (b + 1 < nh) table[r.base + s_slot[b]].prob = residual_prob(L.one + s_sh[b] - sl, L);
+        table[r.base + idx] = AliasEntry{op[j], (nh ? hslot : idx) - r.lead};
+        // heavies whose surplus prefix lies in (sl, sl + D]: this light finishes them
+        sl += dl[j];
+        while (hv <= sl) {
+          if (b + 1 < nh) table[r.base + hslot].prob = residual_prob(L.one + hv - sl, L);
           ++b;
+          hv = s_sh[b];
+          hslot = s_slot[b];
         }
       }
     }
