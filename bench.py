@@ -48,6 +48,7 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
 KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
                   for g in (2, 4, 8, 16, 32) for x in ("", "x")})
 KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,2>" % (64 * nw) for nw in range(2, 17)})
+KERNEL_OF["mw10"] = "build_merge_kernel<448,3>"
 
 
 def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sample=1_000_000):

@@ -521,7 +521,7 @@ constexpr uint64_t MERGE_CNT = 1ull << 52;
 constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
 
 template <int ROWT, int T>
-__global__ __launch_bounds__(ROWT, (ROWT >= 576 && ROWT <= 640 ? 6 : 4)) void build_merge_kernel(const RowRef* __restrict__ vlist,
+__global__ __launch_bounds__(ROWT, (ROWT == 576 ? 6 : 4)) void build_merge_kernel(const RowRef* __restrict__ vlist,
                                                            const uint32_t* __restrict__ xadj,
                                                            const float* __restrict__ wgt,
                                                            AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
@@ -920,7 +920,8 @@ int prepare_build_scratch(uint32_t max_rows) {
   if (!sc.lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
 #define SKY_BIG(NW) SKY_TRY(enable_big_lds(build_merge_kernel<64 * NW, 2>, (64 * NW * 8 + 2) * 14))
-    SKY_BIG(10); SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
+    SKY_TRY(enable_big_lds(build_merge_kernel<448, 3>, (448 * 12 + 2) * 14));
+    SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
 #undef SKY_BIG
     sc.lds_enabled = true;
   }
@@ -1007,7 +1008,10 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 2>, 64, 2, "lds_w2"));
 #define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 2>, 64 * NW, 2, mw_name[NW - 2]))
     SKY_MW(2); SKY_MW(3); SKY_MW(4); SKY_MW(5); SKY_MW(6); SKY_MW(7); SKY_MW(8); SKY_MW(9);
-    SKY_MW(10); SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
+    // rows of 4605..5117 entries: 7 wavefronts of 12 slots per thread.  Two workgroups of 10 wavefronts would
+    // have to fit 6 wavefronts per SIMD (80 registers, spills); 7 fit at 4 per SIMD
+    SKY_TRY(mrg(CLS_MW2 + 8, build_merge_kernel<448, 3>, 448, 3, mw_name[8]));
+    SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
 #undef SKY_MW
   } else {
     SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));

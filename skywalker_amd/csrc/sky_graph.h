@@ -44,7 +44,7 @@ enum BuildClass : int {
   CLS_LDS_W1 = 12, // deg <= 253       one wavefront, LDS prefix arrays, 4 entries per lane
   CLS_LDS_W2 = 13, // deg <= 509       one wavefront, 8 entries per lane
   CLS_MW2 = 14,    // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
-  CLS_MW16 = 28,   //                  class CLS_MW2 + nw - 2
+  CLS_MW16 = 28,   //                  class CLS_MW2 + nw - 2 (nw = 10: 7 wavefronts, 12 entries per thread)
   CLS_STREAM = 29, // deg <= 65533     one workgroup streams the row, its heavies stay in LDS
   CLS_HUGE = 30,   // above            built tile by tile by the whole GPU
   CLS_COUNT = 31
