@@ -32,6 +32,11 @@ struct StreamRow {
 };
 
 // The 8 weights of this thread in chunk c (span slots c*ST_CH + 8*tid ...) as loaded; zeros past the row.
+// Whether any slot of wavefront `wave` in chunk c lies inside the row's span.
+__device__ __forceinline__ bool wave_in_row(const StreamRow& r, uint32_t c, int wave) {
+  return c * ST_CH + (uint32_t)(ST_PER * 64) * (uint32_t)wave < r.span;
+}
+
 struct RawChunk {
   float4 q[ST_PER / 4];
 };
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the row's h-th heavy
   __shared__ uint16_t s_slot[ST_CAP + 1];  // its span slot
   __shared__ WSum3 s_w[ST_NW];
-  __shared__ uint64_t s_a[ST_NW], s_d[ST_NW];
+  __shared__ uint64_t s_a[ST_NW];
   __shared__ uint32_t s_c[ST_NW];
   const RowRef rr = vlist[blockIdx.x];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -145,6 +150,7 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   for (uint32_t c = 0; c < nch; ++c) {
     const RawChunk cur = nx;
     if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
+    if (!wave_in_row(r, c, wave)) continue;
     double wd[ST_PER];
     unpack_chunk(cur, r, c, tid, wd);
 #pragma unroll
@@ -173,32 +179,57 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   }
   const Ledger L = make_ledger_small(rr.d, wsum3_to_double(sum));
 
-  // ---- pass B: the heavies, in slot order, with their surplus prefix
-  uint64_t carry_u = 0, sd = 0;
+  // ---- pass B: the heavies, in slot order.  Whether an entry is heavy is a monotone function of its
+  // clamped weight (p = fl(w * scale) and t = fma(p, 2^F, -2^F) are monotone, heavy iff t >= 0.5), so one
+  // compare against the smallest heavy weight of this row decides it; the surplus is then computed for the
+  // heavies alone, from the compacted list.
+  uint32_t thr_bits;  // bit pattern of the smallest clamped weight that is heavy (above 2^32: none is)
+  {
+    auto is_heavy = [&](uint32_t bits) {
+      const double p = (double)__uint_as_float(bits) * L.scale;
+      return fma(p, L.fs, -L.fs) >= 0.5;
+    };
+    const double est = (1.0 + 0.5 * L.inv_fs) / L.scale;
+    constexpr uint32_t MAXW = 0x4F800000u;  // 2^32
+    uint32_t bits = est >= 4294967296.0 ? MAXW : __float_as_uint((float)est);
+    int guard = 0;
+    while (bits > 0 && is_heavy(bits - 1) && guard < 64) {
+      --bits;
+      ++guard;
+    }
+    while (bits <= MAXW && !is_heavy(bits) && guard < 64) {
+      ++bits;
+      ++guard;
+    }
+    if (guard >= 64) {  // the estimate is within a step or two of the boundary; anything else: leave the row
+      if (tid == 0) deferred[atomicAdd(n_deferred, 1u)] = rr;
+      return;
+    }
+    thr_bits = bits;
+  }
+  float* s_w32 = reinterpret_cast<float*>(s_sh);  // weight of heavy h in the low half of s_sh[h], until its prefix replaces it
   uint32_t carry_c = 0;
   bool overflow = false;
   for (uint32_t c = 0; c < nch; ++c) {
     const RawChunk cur = nx;
     if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
-    double wd[ST_PER];
-    const uint32_t live = unpack_chunk(cur, r, c, tid, wd);
-    uint64_t u[ST_PER];
-    uint64_t su = 0;
+    float cw[ST_PER];
     uint32_t heavy = 0;
+    if (wave_in_row(r, c, wave))
 #pragma unroll
-    for (int j = 0; j < ST_PER; ++j) {
-      const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
-      if (e.heavy) {
-        su += e.amount;
-        heavy |= 1u << j;
-      } else {
-        sd += e.amount;
+    for (int q = 0; q < ST_PER / 4; ++q) {
+      const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
+      const float xs[4] = {cur.q[q].x, cur.q[q].y, cur.q[q].z, cur.q[q].w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t idx = pos + k;
+        cw[q * 4 + k] = clamp_weight(xs[k]);
+        if (idx >= r.lead && idx < r.span && __float_as_uint(cw[q * 4 + k]) >= thr_bits) heavy |= 1u << (q * 4 + k);
       }
-      u[j] = su;
     }
     uint64_t ex_u, tot_u;
     uint32_t ex_c, tot_c;
-    stream_excl(su, (uint32_t)__popc(heavy), s_a, s_c, ex_u, ex_c, tot_u, tot_c);
+    stream_excl(0ull, (uint32_t)__popc(heavy), s_a, s_c, ex_u, ex_c, tot_u, tot_c);
     if (carry_c + tot_c > ST_CAP) {  // uniform
       overflow = true;
       break;
@@ -207,55 +238,78 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
 #pragma unroll
     for (int j = 0; j < ST_PER; ++j)
       if ((heavy >> j) & 1) {
-        s_sh[rank] = carry_u + ex_u + u[j];
+        s_w32[2 * rank] = cw[j];
         s_slot[rank] = (uint16_t)(c * ST_CH + (uint32_t)ST_PER * tid + j);
         ++rank;
       }
-    carry_u += tot_u;
     carry_c += tot_c;
   }
   if (overflow) {
     if (tid == 0) deferred[atomicAdd(n_deferred, 1u)] = rr;
     return;
   }
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) sd += shfl_xor_u64(sd, m);
-  if (lane == 0) s_d[wave] = sd;
-  __syncthreads();  // the heavy list and s_d are complete
-  uint64_t total_l = 0;
-#pragma unroll
-  for (int i = 0; i < ST_NW; ++i) total_l += s_d[i];
+  __syncthreads();  // the heavy list is complete
   const uint32_t nh = carry_c;
-  const uint64_t total_h = carry_u;
+  {
+    // surplus prefix of the list: 16 consecutive heavies per thread
+    constexpr int HP = 16;
+    static_assert(ST_CAP < (uint32_t)ST_T * HP, "one round covers the list");
+    uint64_t u[HP];
+    uint64_t su = 0;
+#pragma unroll
+    for (int k = 0; k < HP; ++k) {
+      const uint32_t h = (uint32_t)HP * tid + k;
+      if (h < nh) su += classify_fast((double)s_w32[2 * h], true, L).amount;
+      u[k] = su;
+    }
+    uint64_t ex_u, tot_u;
+    uint32_t ex_c, tot_c;
+    stream_excl(su, 0u, s_a, s_c, ex_u, ex_c, tot_u, tot_c);
+#pragma unroll
+    for (int k = 0; k < HP; ++k) {
+      const uint32_t h = (uint32_t)HP * tid + k;
+      if (h < nh) s_sh[h] = ex_u + u[k];
+    }
+  }
+  __syncthreads();
   if (tid == 0) {  // sentinel after the list; the first barrier of pass C publishes it
     s_sh[nh] = ~0ull;
     s_slot[nh] = nh ? s_slot[nh - 1] : (uint16_t)0;
   }
 
   // ---- pass C: every entry
-  uint64_t carry_d = 0;
+  uint64_t carry_d = 0;  // deficits so far; the row's total deficit after the last chunk
   carry_c = 0;
   nx = fetch_chunk(wgt, r, 0, tid);
   for (uint32_t c = 0; c < nch; ++c) {
     const RawChunk cur = nx;
     if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
-    double wd[ST_PER];
-    const uint32_t live = unpack_chunk(cur, r, c, tid, wd);
+    const bool on = wave_in_row(r, c, wave);  // a wavefront past the row's end only takes part in the scan
+    uint32_t live = 0;
     float op[ST_PER];
     uint64_t dl[ST_PER];
     uint32_t heavy = 0;
     uint64_t run = 0;
+    if (on) {
+      double wd[ST_PER];
+      live = unpack_chunk(cur, r, c, tid, wd);
 #pragma unroll
-    for (int j = 0; j < ST_PER; ++j) {
-      const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
-      op[j] = (float)e.p;
-      dl[j] = e.heavy ? 0 : e.amount;
-      run += dl[j];
-      if (e.heavy) heavy |= 1u << j;
+      for (int j = 0; j < ST_PER; ++j) {
+        const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
+        op[j] = (float)e.p;
+        dl[j] = e.heavy ? 0 : e.amount;
+        run += dl[j];
+        if (e.heavy) heavy |= 1u << j;
+      }
     }
     uint64_t ex_d, tot_d;
     uint32_t ex_c, tot_c;
     stream_excl(run, (uint32_t)__popc(heavy), s_a, s_c, ex_d, ex_c, tot_d, tot_c);
+    if (!on) {
+      carry_d += tot_d;
+      carry_c += tot_c;
+      continue;
+    }
     // b = heavies whose surplus prefix is <= the deficits before this thread's slots: one search; from
     // there the thread's lights walk the list, each stopping at its own deficit prefix
     uint64_t sl = carry_d + ex_d;
@@ -275,7 +329,7 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
       const uint32_t idx = pos0 + j;
       if ((heavy >> j) & 1) {
         const uint32_t hr = carry_c + ex_c + (uint32_t)__popc(heavy & ((1u << j) - 1));
-        if (hr + 1 >= nh || s_sh[hr] > total_l) {
+        if (hr + 1 >= nh) {
           table[r.base + idx] = AliasEntry{1.0f, idx - r.lead};
         } else {
           table[r.base + idx].alias = (uint32_t)s_slot[hr + 1] - r.lead;
@@ -295,7 +349,13 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
     carry_d += tot_d;
     carry_c += tot_c;
   }
-  (void)total_h;
+  // heavies no light has reached (surplus prefix beyond the row's total deficit) keep their bucket
+  __syncthreads();
+  for (uint32_t h = tid; h + 1 < nh; h += ST_T)
+    if (s_sh[h] > carry_d) {
+      const uint32_t slot = s_slot[h];
+      table[r.base + slot] = AliasEntry{1.0f, slot - r.lead};
+    }
   if (tid == 0) valid[rr.v] = 1;
 }
 
