@@ -44,7 +44,8 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 509) return CLS_LDS_W2;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
   if (nw <= 16) return CLS_MW2 + (int)nw - 2;
-  return d <= STREAM_MAX_DEG ? CLS_STREAM : CLS_HUGE;
+  if (d > STREAM_MAX_DEG) return CLS_HUGE;
+  return d > 24576u ? CLS_STREAM : CLS_STREAM_LAST;
 }
 
 // ---------------------------------------------------------------- binning
@@ -1033,8 +1034,14 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   }
 
   const RowRef* deferred = nullptr;
-  if (counts[CLS_STREAM]) {
-    const uint32_t cnt = counts[CLS_STREAM];
+  uint32_t stream_rows = 0;
+  uint64_t stream_edges = 0;
+  for (int c = CLS_STREAM; c <= CLS_STREAM_LAST; ++c) {
+    stream_rows += counts[c];
+    stream_edges += host.edges[c];
+  }
+  if (stream_rows) {  // one launch over the two lists, which lie back to back
+    const uint32_t cnt = stream_rows;
     if (g_row_merge) {
       uint32_t nd = 0;
       SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], cnt, &deferred, &nd));
@@ -1043,7 +1050,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_STREAM], cnt, &skipped, nullptr, 0));
       if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles is too small for rows of up to 65533 entries");
     }
-    if (tm) SKY_TRY(tm->mark("stream", host.edges[CLS_STREAM]));
+    if (tm) SKY_TRY(tm->mark("stream", stream_edges));
   }
   if (counts[CLS_HUGE]) {
     const uint32_t cnt = counts[CLS_HUGE];

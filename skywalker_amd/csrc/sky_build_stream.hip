@@ -71,7 +71,9 @@ __device__ __forceinline__ uint32_t unpack_chunk(const RawChunk& x, const Stream
 }
 
 // Exclusive prefix over the workgroup (thread order) of one u64 and one u32 per thread, plus totals.
-// Two barriers: the second one lets the caller reuse s_a / s_c right away.
+// One barrier: consecutive calls must alternate between two sets of s_a / s_c (a wavefront may start
+// the next call while others still read this one's sums; it cannot start the one after that before
+// every wavefront has passed the next call's barrier).
 __device__ __forceinline__ void stream_excl(uint64_t a, uint32_t c, uint64_t* s_a, uint32_t* s_c, uint64_t& ex_a,
                                             uint32_t& ex_c, uint64_t& tot_a, uint32_t& tot_c) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -97,7 +99,6 @@ __device__ __forceinline__ void stream_excl(uint64_t a, uint32_t c, uint64_t* s_
   }
   tot_a = ra;
   tot_c = rc;
-  __syncthreads();
 }
 
 // For M keys at once: number of entries of the sorted LDS array a[0..n), n >= 1, that are <= key[m].
@@ -134,8 +135,8 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the row's h-th heavy
   __shared__ uint16_t s_slot[ST_CAP + 1];  // its span slot
   __shared__ WSum3 s_w[ST_NW];
-  __shared__ uint64_t s_a[ST_NW];
-  __shared__ uint32_t s_c[ST_NW];
+  __shared__ uint64_t s_a[2][ST_NW];  // two sets of wavefront sums, used alternately
+  __shared__ uint32_t s_c[2][ST_NW];
   const RowRef rr = vlist[blockIdx.x];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   StreamRow r;
@@ -229,7 +230,7 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
     }
     uint64_t ex_u, tot_u;
     uint32_t ex_c, tot_c;
-    stream_excl(0ull, (uint32_t)__popc(heavy), s_a, s_c, ex_u, ex_c, tot_u, tot_c);
+    stream_excl(0ull, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_u, ex_c, tot_u, tot_c);
     if (carry_c + tot_c > ST_CAP) {  // uniform
       overflow = true;
       break;
@@ -264,7 +265,7 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
     }
     uint64_t ex_u, tot_u;
     uint32_t ex_c, tot_c;
-    stream_excl(su, 0u, s_a, s_c, ex_u, ex_c, tot_u, tot_c);
+    stream_excl(su, 0u, s_a[0], s_c[0], ex_u, ex_c, tot_u, tot_c);
 #pragma unroll
     for (int k = 0; k < HP; ++k) {
       const uint32_t h = (uint32_t)HP * tid + k;
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
     }
     uint64_t ex_d, tot_d;
     uint32_t ex_c, tot_c;
-    stream_excl(run, (uint32_t)__popc(heavy), s_a, s_c, ex_d, ex_c, tot_d, tot_c);
+    stream_excl(run, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
     if (!on) {
       carry_d += tot_d;
       carry_c += tot_c;

@@ -45,9 +45,11 @@ enum BuildClass : int {
   CLS_LDS_W2 = 13, // deg <= 509       one wavefront, 8 entries per lane
   CLS_MW2 = 14,    // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
   CLS_MW16 = 28,   //                  class CLS_MW2 + nw - 2 (nw = 10: 7 wavefronts, 12 entries per thread)
-  CLS_STREAM = 29, // deg <= 65533     one workgroup streams the row, its heavies stay in LDS
-  CLS_HUGE = 30,   // above            built tile by tile by the whole GPU
-  CLS_COUNT = 31
+  CLS_STREAM = 29, // deg 24577..65533  one workgroup streams the row, its heavies stay in LDS.  Two classes, the
+  CLS_STREAM_LAST = 30, // deg 8190..24576  longer rows first, listed back to back and built by one launch, which so
+                   //                  does not end on its longest rows
+  CLS_HUGE = 31,   // above            built tile by tile by the whole GPU
+  CLS_COUNT = 32
 };
 
 // One listed row of a degree class: the build kernels read where the row lies from the list itself
