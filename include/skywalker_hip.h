@@ -143,6 +143,9 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      fall to a kernel in which one workgroup walks the whole row.  Tests lower it to exercise that kernel.
  *      "row_merge" (default 1): rows of 62..8189 entries pair lights and heavies by a merge of their prefix
  *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table.
+ *      "stream_min_edges" (default 4000000): rows of 8190..65533 entries have a kernel of their own (one workgroup
+ *      streams a row); when a build holds no more than this many entries in such rows they go to the tile-parallel
+ *      path instead, which then needs no answer from the device in the middle of the build.  Tests set 0.
  *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:
  *      0 builds, before every step, the rows the walkers stand on; 1 builds every row first and walks as
  *      sky_walk_offline does; -1 takes whichever is estimated to be faster.  The paths are the same. ---- */

@@ -872,6 +872,8 @@ int enable_big_lds(K kernel, size_t bytes) {
 }
 
 }  // namespace
+static uint64_t g_stream_min_edges = 4000000;
+void set_stream_min_edges(uint64_t n) { g_stream_min_edges = n; }
 void set_row_merge(bool on) { g_row_merge = on; }
 
 int EventTimer::mark(const char* name, uint64_t e) {
@@ -1040,22 +1042,21 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     stream_rows += counts[c];
     stream_edges += host.edges[c];
   }
-  if (stream_rows) {  // one launch over the two lists, which lie back to back
-    const uint32_t cnt = stream_rows;
-    if (g_row_merge) {
-      uint32_t nd = 0;
-      SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], cnt, &deferred, &nd));
-    } else {
-      uint32_t skipped = 0;
-      SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_STREAM], cnt, &skipped, nullptr, 0));
-      if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles is too small for rows of up to 65533 entries");
-    }
+  // A small streaming class is not worth its own launch and the host round trip that asks for its deferred
+  // rows: its rows then go to the tile-parallel path together with the HUGE class that follows them in the list.
+  const bool stream_to_tiled = !g_row_merge || stream_edges <= g_stream_min_edges;
+  if (stream_rows && !stream_to_tiled) {  // one launch over the two lists, which lie back to back
+    uint32_t nd = 0;
+    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], stream_rows, &deferred, &nd));
     if (tm) SKY_TRY(tm->mark("stream", stream_edges));
   }
-  if (counts[CLS_HUGE]) {
-    const uint32_t cnt = counts[CLS_HUGE];
+  const uint32_t tiled_rows = counts[CLS_HUGE] + (stream_to_tiled ? stream_rows : 0);
+  const uint64_t tiled_edges = host.edges[CLS_HUGE] + (stream_to_tiled ? stream_edges : 0);
+  const RowRef* tiled_list = vlist + (stream_to_tiled ? starts[CLS_STREAM] : starts[CLS_HUGE]);
+  if (tiled_rows) {
+    const uint32_t cnt = tiled_rows;
     uint32_t skipped = 0;
-    SKY_TRY(build_rows_tiled(g, vlist + starts[CLS_HUGE], cnt, &skipped, tm, host.edges[CLS_HUGE]));
+    SKY_TRY(build_rows_tiled(g, tiled_list, cnt, &skipped, tm, tiled_edges));
     if (skipped) {  // rows with more tiles than the tile-parallel path takes: one workgroup streams each
       const uint32_t max_tiles = tiled_max_tiles();
       if (sc.huge_cap < cnt) {
@@ -1065,7 +1066,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
         SKY_HIP(hipMalloc((void**)&sc.huge_off, ((size_t)cnt + 1) * 8));
         sc.huge_cap = cnt;
       }
-      hipLaunchKernelGGL(huge_prefix_kernel, dim3(1), dim3(1024), 0, st, vlist + starts[CLS_HUGE], cnt, max_tiles,
+      hipLaunchKernelGGL(huge_prefix_kernel, dim3(1), dim3(1024), 0, st, tiled_list, cnt, max_tiles,
                          g->xadj, sc.huge_off, sc.huge_off + cnt);
       uint64_t total = 0;
       SKY_HIP(hipMemcpyAsync(&total, sc.huge_off + cnt, 8, hipMemcpyDeviceToHost, st));
@@ -1078,11 +1079,11 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
         sc.huge_scratch_cap = total;
       }
       hipLaunchKernelGGL(build_huge_kernel, dim3(std::min<uint32_t>(cnt, 512)), dim3(HUGE_T), 0, st,
-                         vlist + starts[CLS_HUGE], cnt, max_tiles, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch,
+                         tiled_list, cnt, max_tiles, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch,
                          g->table, g->valid);
+      if (tm) SKY_TRY(tm->mark("streamed", 0));
     }
   }
-  if (tm && counts[CLS_HUGE]) SKY_TRY(tm->mark("streamed", 0));
   if (deferred) {  // rows the streaming kernel left alone (more heavies than its LDS list holds); asked last,
                    // so that the host round trip does not idle the GPU between two classes
     uint32_t nd = 0, skipped = 0;

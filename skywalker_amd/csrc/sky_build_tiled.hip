@@ -147,6 +147,7 @@ __global__ __launch_bounds__(TL_T) void tiled_sum_kernel(const TileGeom* __restr
   __shared__ WSum3 s_w[TL_T / 64];
   const uint32_t tile = blockIdx.x;
   const TileGeom tg = geom[tile];
+  if (tg.span == 0) return;  // the grid may be larger than the number of tiles
   const TiledRow r = geom_row(tg, tile);
   const int tid = threadIdx.x;
   float w[TL_Q][4];
@@ -201,6 +202,7 @@ __global__ __launch_bounds__(TL_T) void tiled_totals_kernel(const TileGeom* __re
   __shared__ uint32_t s_f[TL_T / 64], s_l[TL_T / 64];
   const uint32_t tile = blockIdx.x;
   const TileGeom tg = geom[tile];
+  if (tg.span == 0) return;
   const int tid = threadIdx.x;
   const uint32_t t = tg.T;
   float w[TL_Q][4];
@@ -431,6 +433,7 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const TileGeom* __rest
   __shared__ uint32_t s_fh[TL_Q][NW];
   const uint32_t tile = blockIdx.x;
   const TileGeom tg = geom[tile];
+  if (tg.span == 0) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t T = tg.T;
 
@@ -587,7 +590,10 @@ uint32_t tiled_max_tiles() { return g_tiled_max_tiles; }
 void set_tiled_max_tiles(uint32_t n) { g_tiled_max_tiles = std::min<uint32_t>(std::max<uint32_t>(n, 1), TILED_MAX_TILES); }
 
 // Builds the rows of `rows_list` (device, n entries) that have at most the configured number of
-// tiles; *skipped receives how many rows were left for the streaming kernel.
+// tiles; *skipped receives how many rows were left for the streaming kernel.  `edges` is the number of
+// entries of the listed rows when the caller knows it (0 otherwise): the tile grids are then sized by
+// the bound edges / TILE + 2 n, with empty records for the tiles that do not exist, and the host does
+// not wait for the device to count them.
 int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
                      uint64_t edges) {
   hipStream_t st = g->stream;
@@ -605,12 +611,19 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
   SKY_HIP(hipMemsetAsync(sc.totals, 0, sizeof(TiledCounters), st));
   hipLaunchKernelGGL(tiled_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, st, rows_list, n, g->xadj,
                      g_tiled_max_tiles, sc.rows, sc.totals);
-  TiledCounters totals = {};
-  SKY_HIP(hipMemcpyAsync(&totals, sc.totals, sizeof(totals), hipMemcpyDeviceToHost, st));
-  SKY_HIP(hipStreamSynchronize(st));
-  const uint32_t ntiles = (uint32_t)totals.next;
-  const uint32_t nslots = (uint32_t)(totals.next >> 32);  // 256 per block of rows
-  *skipped = totals.skipped;
+  const bool bounded = edges != 0 && g_tiled_max_tiles == TILED_MAX_TILES && edges / TILE + 2ull * n < (1ull << 31);
+  uint32_t ntiles, nslots;
+  if (bounded) {
+    ntiles = (uint32_t)(edges / TILE + 2ull * n);
+    nslots = 256u * ((n + 255) / 256);
+  } else {
+    TiledCounters totals = {};
+    SKY_HIP(hipMemcpyAsync(&totals, sc.totals, sizeof(totals), hipMemcpyDeviceToHost, st));
+    SKY_HIP(hipStreamSynchronize(st));
+    ntiles = (uint32_t)totals.next;
+    nslots = (uint32_t)(totals.next >> 32);  // 256 per block of rows
+    *skipped = totals.skipped;
+  }
   if (ntiles == 0) return SKY_OK;
   if (sc.tile_cap < ntiles) {
     void* olds[] = {sc.geom, sc.tsum, sc.ttot, sc.nfh, sc.ranges};
@@ -638,6 +651,7 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
     SKY_HIP(hipMalloc((void**)&sc.BH, (b_need + b_need / 4 + 1024) * 8));
     b_cap = b_need + b_need / 4 + 1024;
   }
+  if (bounded) SKY_HIP(hipMemsetAsync(sc.geom, 0, (size_t)ntiles * sizeof(TileGeom), st));  // span 0: no such tile
   hipLaunchKernelGGL(tiled_map_kernel, dim3(n), dim3(256), 0, st, sc.rows, n, sc.geom);
   if (tm) SKY_TRY(tm->mark("tiled_rows", 0));
   hipLaunchKernelGGL(tiled_sum_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.geom, g->adjwgt, sc.tsum);

@@ -319,6 +319,11 @@ int sky_set_option(const char* name, long value) {
     set_row_merge(value != 0);
     return SKY_OK;
   }
+  if (!strcmp(name, "stream_min_edges")) {
+    if (value < 0) return fail(SKY_ERR_ARG, "sky_set_option: stream_min_edges must be >= 0");
+    set_stream_min_edges((uint64_t)value);
+    return SKY_OK;
+  }
   if (!strcmp(name, "online_full_build")) {
     set_online_full_build((int)value);
     return SKY_OK;
