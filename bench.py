@@ -145,6 +145,7 @@ def main():
     import numpy as np
 
     cfg = CONFIGS[args.config]
+    capi.set_option("build_profile", 1)  # HIP events between the build kernels: the roofline needs each one's duration
     if args.calibrate:
         words = 1 << 28
         a = capi.DeviceArray(words, np.uint32, fill=1)

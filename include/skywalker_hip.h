@@ -146,13 +146,16 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      "stream_min_edges" (default 4000000): rows of 8190..65533 entries have a kernel of their own (one workgroup
  *      streams a row); when a build holds no more than this many entries in such rows they go to the tile-parallel
  *      path instead, which then needs no answer from the device in the middle of the build.  Tests set 0.
+ *      "build_profile" (default 0): 1 records a HIP event after every kernel of sky_alias_build_all for
+ *      sky_last_build_profile (about 3 microseconds each; a small graph pays 20 % of its build for them).
  *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:
  *      0 builds, before every step, the rows the walkers stand on; 1 builds every row first and walks as
  *      sky_walk_offline does; -1 takes whichever is estimated to be faster.  The paths are the same. ---- */
 int sky_set_option(const char* name, long value);
 
 /* ---- per-kernel timing of the last sky_alias_build_all on this graph, for roofline reporting:
- *      names[i] is a static string, ms[i] its HIP-event duration.  Returns the number of entries. ---- */
+ *      names[i] is a static string, ms[i] its HIP-event duration.  Returns the number of entries: one
+ *      ("build") unless the option "build_profile" was 1 during the build. ---- */
 int sky_last_build_profile(const sky_graph* g, const char** names, float* ms, uint64_t* edges, int max_entries);
 
 #ifdef __cplusplus

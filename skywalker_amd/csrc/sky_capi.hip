@@ -324,6 +324,10 @@ int sky_set_option(const char* name, long value) {
     set_stream_min_edges((uint64_t)value);
     return SKY_OK;
   }
+  if (!strcmp(name, "build_profile")) {
+    set_build_profile(value != 0);
+    return SKY_OK;
+  }
   if (!strcmp(name, "online_full_build")) {
     set_online_full_build((int)value);
     return SKY_OK;

@@ -86,6 +86,7 @@ int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n, const R
 int stream_deferred_count(sky_graph* g, uint32_t* n_deferred);
 void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);
+void set_build_profile(bool on);
 void set_online_full_build(int mode);
 uint32_t tiled_max_tiles();
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,

@@ -187,3 +187,26 @@ def test_special_weight_values_in_every_kind_of_row(orc):
     # rows made of nothing but contributions that vanish: invalid rows in every class
     w2 = np.where(rng.random(len(w)) < 0.5, np.float32(1e-30), np.float32(-3.0)).astype(np.float32)
     build_and_compare(orc, xadj, adjncy, w2, "all-vanishing rows")
+
+
+def test_build_profile_is_opt_in(orc):
+    # without the option one bracket spans the build; with it every launched class has its own entry
+    from skywalker_amd import capi
+    g = capi.Graph.rmat(14, 16, 3, capi.W_UNIFORM, 1.0, 100.0, 3)
+    sec = g.build_tables()
+    prof = g.build_profile()
+    assert [p[0] for p in prof] == ["build"] and prof[0][2] == g.E
+    assert abs(prof[0][1] * 1e-3 - sec) < 1e-6
+    before = g.tables()
+    capi.set_option("build_profile", 1)
+    try:
+        sec = g.build_tables()
+    finally:
+        capi.set_option("build_profile", 0)
+    prof = g.build_profile()
+    assert prof[0][0] == "bin" and len(prof) > 3
+    assert abs(sum(p[1] for p in prof) * 1e-3 - sec) < 1e-5  # the brackets tile the build
+    after = g.tables()
+    g.free()
+    for a, b in zip(before, after):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
