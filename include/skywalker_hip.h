@@ -103,7 +103,9 @@ int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t*
 int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, const int8_t* valid);
 
 /* ---- start vertices uniform over [0,V): Philox(seed; i). seeds_device[N]. The reference uses 0..N-1
- *      (include/sampler.cuh:494-503); sequential seeds are simply uploaded by the caller. ---- */
+ *      (include/sampler.cuh:494-503); sequential seeds are simply uploaded by the caller.  The walk and
+ *      sample calls below accept any 32-bit value as a start vertex: one that is not below V is recorded in its
+ *      slot and never left (length 0, no children), it is not an error. ---- */
 int sky_gen_seeds(uint64_t seed, uint32_t V, uint32_t N, uint32_t* seeds_device);
 
 /* ---- biased walk on prebuilt tables: replaces OfflineWalk(Walker&) (src/offline_walk.cu:181-230, kernels

@@ -409,7 +409,7 @@ int orc_alias_check(const uint32_t* xadj, const float* w, const float* prob, con
 //   next = adjncy[off + cand]
 // paths is walker-major, N x (len+1) (sampler_result.cuh:607-612); slots past
 // length[i] are not written.
-int orc_walk_offline(const uint32_t* xadj, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
+int orc_walk_offline(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
                      const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed, uint32_t* paths,
                      uint32_t* lengths, uint64_t* sampled) {
   uint64_t total = 0;
@@ -419,7 +419,7 @@ int orc_walk_offline(const uint32_t* xadj, const uint32_t* adjncy, const float* 
     uint32_t v = seeds[i];
     path[0] = v;
     uint32_t s = 0;
-    for (; s < len; ++s) {
+    for (; s < len && v < V; ++s) {  // a start vertex that does not exist is recorded and never left
       uint32_t r[4];
       philox(seed, (uint32_t)i, s, 0, DOM_WALK, r);
       if (stop_prob > 0.0f && u24(r[2]) < stop_prob) break;
@@ -456,7 +456,7 @@ static inline float node2vec_weight(const uint32_t* xadj, const uint32_t* adjncy
 }
 
 // bias_kind 0: static edge weights (DeepWalk / PPR); 1: node2vec second order.
-int orc_walk_online(const uint32_t* xadj, const uint32_t* adjncy, const float* w, int bias_kind, float p, float q,
+int orc_walk_online(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* w, int bias_kind, float p, float q,
                     const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed, uint32_t* paths,
                     uint32_t* lengths, uint64_t* sampled) {
   uint64_t total = 0;
@@ -472,7 +472,7 @@ int orc_walk_online(const uint32_t* xadj, const uint32_t* adjncy, const float* w
       bool has_prev = false;
       path[0] = v;
       uint32_t s = 0;
-      for (; s < len; ++s) {
+      for (; s < len && v < V; ++s) {
         uint32_t r[4];
         philox(seed, (uint32_t)i, s, 0, DOM_WALK, r);
         if (stop_prob > 0.0f && u24(r[2]) < stop_prob) break;
@@ -505,7 +505,7 @@ int orc_walk_online(const uint32_t* xadj, const uint32_t* adjncy, const float* w
 // it when u24(r_t[3]) * fmax < f(nbr), f = 1/p if nbr is the previous vertex, 1 if adjacent to it, 1/q
 // otherwise, fmax = max(1/p, 1, 1/q).  After 65536 rejections the last candidate is taken.  The law of
 // the accepted neighbour is w * f / sum(w * f), the same as a draw from the second-order table.
-int orc_walk_node2vec_reject(const uint32_t* xadj, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
+int orc_walk_node2vec_reject(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
                              float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob,
                              uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled) {
   const float fp = 1.0f / p, fq = 1.0f / q;
@@ -518,7 +518,7 @@ int orc_walk_node2vec_reject(const uint32_t* xadj, const uint32_t* adjncy, const
     bool has_prev = false;
     path[0] = v;
     uint32_t s = 0;
-    for (; s < len; ++s) {
+    for (; s < len && v < V; ++s) {
       uint32_t r[4];
       philox(seed, (uint32_t)i, s, 0, DOM_WALK, r);
       if (stop_prob > 0.0f && u24(r[2]) < stop_prob) break;
@@ -565,7 +565,7 @@ int orc_walk_node2vec_reject(const uint32_t* xadj, const uint32_t* adjncy, const
 // A parent with an invalid row (zero total weight) yields no children (CheckValid, offline_sample.cu:86).
 // Slots that receive no vertex are not written.
 // online != 0 rebuilds each parent's table from w with the sweep instead of reading prob/alias.
-static int sample_impl(const uint32_t* xadj, const uint32_t* adjncy, const float* w, const float* prob,
+static int sample_impl(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* w, const float* prob,
                        const uint32_t* alias, int online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout,
                        uint32_t hops, uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled) {
   // fanout[0..hops-1], fanout[0] == 1
@@ -596,6 +596,7 @@ static int sample_impl(const uint32_t* xadj, const uint32_t* adjncy, const float
         for (uint64_t s = 0; s < width[h]; ++s) {
           if (!filled[s]) continue;
           const uint32_t v = d[off[h] + s];
+          if (v >= V) continue;  // a seed that does not exist has no children
           const uint32_t o = xadj[v], deg = xadj[v + 1] - o;
           if (deg == 0) continue;
           const float* pr = prob ? prob + o : nullptr;
@@ -636,16 +637,16 @@ static int sample_impl(const uint32_t* xadj, const uint32_t* adjncy, const float
   return 0;
 }
 
-int orc_sample_offline(const uint32_t* xadj, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
+int orc_sample_offline(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
                        const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops, uint64_t seed,
                        uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled) {
-  return sample_impl(xadj, adjncy, nullptr, prob, alias, 0, seeds, N, fanout, hops, seed, data, sample_lengths,
+  return sample_impl(xadj, V, adjncy, nullptr, prob, alias, 0, seeds, N, fanout, hops, seed, data, sample_lengths,
                      sampled);
 }
-int orc_sample_online(const uint32_t* xadj, const uint32_t* adjncy, const float* w, const uint32_t* seeds, uint32_t N,
+int orc_sample_online(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* w, const uint32_t* seeds, uint32_t N,
                       const uint32_t* fanout, uint32_t hops, uint64_t seed, uint32_t* data, uint32_t* sample_lengths,
                       uint64_t* sampled) {
-  return sample_impl(xadj, adjncy, w, nullptr, nullptr, 1, seeds, N, fanout, hops, seed, data, sample_lengths,
+  return sample_impl(xadj, V, adjncy, w, nullptr, nullptr, 1, seeds, N, fanout, hops, seed, data, sample_lengths,
                      sampled);
 }
 

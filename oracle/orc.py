@@ -44,15 +44,15 @@ def lib():
     L.orc_alias_reconstruct_row.argtypes = [_f32p, _u32p, C.c_uint32, _f64p]
     L.orc_alias_reconstruct_row.restype = None
     L.orc_alias_check.argtypes = [_u32p, _f32p, _f32p, _u32p, _i8p, C.c_uint32, _f64p]
-    L.orc_walk_offline.argtypes = [_u32p, _u32p, _f32p, _u32p, _u32p, C.c_uint32, C.c_uint32, C.c_float, C.c_uint64,
+    L.orc_walk_offline.argtypes = [_u32p, C.c_uint32, _u32p, _f32p, _u32p, _u32p, C.c_uint32, C.c_uint32, C.c_float, C.c_uint64,
                                    _u32p, _u32p, C.POINTER(C.c_uint64)]
-    L.orc_walk_online.argtypes = [_u32p, _u32p, _f32p, C.c_int, C.c_float, C.c_float, _u32p, C.c_uint32, C.c_uint32,
+    L.orc_walk_online.argtypes = [_u32p, C.c_uint32, _u32p, _f32p, C.c_int, C.c_float, C.c_float, _u32p, C.c_uint32, C.c_uint32,
                                   C.c_float, C.c_uint64, _u32p, _u32p, C.POINTER(C.c_uint64)]
-    L.orc_walk_node2vec_reject.argtypes = [_u32p, _u32p, _f32p, _u32p, C.c_float, C.c_float, _u32p, C.c_uint32, C.c_uint32,
+    L.orc_walk_node2vec_reject.argtypes = [_u32p, C.c_uint32, _u32p, _f32p, _u32p, C.c_float, C.c_float, _u32p, C.c_uint32, C.c_uint32,
                                            C.c_float, C.c_uint64, _u32p, _u32p, C.POINTER(C.c_uint64)]
-    L.orc_sample_offline.argtypes = [_u32p, _u32p, _f32p, _u32p, _u32p, C.c_uint32, _u32p, C.c_uint32, C.c_uint64,
+    L.orc_sample_offline.argtypes = [_u32p, C.c_uint32, _u32p, _f32p, _u32p, _u32p, C.c_uint32, _u32p, C.c_uint32, C.c_uint64,
                                      _u32p, _u32p, C.POINTER(C.c_uint64)]
-    L.orc_sample_online.argtypes = [_u32p, _u32p, _f32p, _u32p, C.c_uint32, _u32p, C.c_uint32, C.c_uint64, _u32p,
+    L.orc_sample_online.argtypes = [_u32p, C.c_uint32, _u32p, _f32p, _u32p, C.c_uint32, _u32p, C.c_uint32, C.c_uint64, _u32p,
                                     _u32p, C.POINTER(C.c_uint64)]
     L.orc_num_threads.restype = C.c_int
     _lib = L
@@ -138,7 +138,7 @@ def walk_offline(xadj, adjncy, prob, alias, seeds, length, stop_prob, seed):
     paths = np.full((N, length + 1), FILL, np.uint32)
     lengths = np.zeros(N, np.uint32)
     sampled = C.c_uint64(0)
-    lib().orc_walk_offline(xadj, adjncy, prob, alias, np.ascontiguousarray(seeds, np.uint32), N, length, stop_prob,
+    lib().orc_walk_offline(xadj, len(xadj) - 1, adjncy, prob, alias, np.ascontiguousarray(seeds, np.uint32), N, length, stop_prob,
                            seed, paths, lengths, C.byref(sampled))
     return paths, lengths, sampled.value
 
@@ -148,7 +148,7 @@ def walk_online(xadj, adjncy, w, bias_kind, p, q, seeds, length, stop_prob, seed
     paths = np.full((N, length + 1), FILL, np.uint32)
     lengths = np.zeros(N, np.uint32)
     sampled = C.c_uint64(0)
-    lib().orc_walk_online(xadj, adjncy, np.ascontiguousarray(w, np.float32), bias_kind, p, q,
+    lib().orc_walk_online(xadj, len(xadj) - 1, adjncy, np.ascontiguousarray(w, np.float32), bias_kind, p, q,
                           np.ascontiguousarray(seeds, np.uint32), N, length, stop_prob, seed, paths, lengths,
                           C.byref(sampled))
     return paths, lengths, sampled.value
@@ -159,7 +159,7 @@ def walk_node2vec_reject(xadj, adjncy, prob, alias, p, q, seeds, length, stop_pr
     paths = np.full((N, length + 1), FILL, np.uint32)
     lengths = np.zeros(N, np.uint32)
     sampled = C.c_uint64(0)
-    lib().orc_walk_node2vec_reject(xadj, adjncy, prob, alias, p, q, np.ascontiguousarray(seeds, np.uint32), N, length,
+    lib().orc_walk_node2vec_reject(xadj, len(xadj) - 1, adjncy, prob, alias, p, q, np.ascontiguousarray(seeds, np.uint32), N, length,
                                    stop_prob, seed, paths, lengths, C.byref(sampled))
     return paths, lengths, sampled.value
 
@@ -184,7 +184,7 @@ def sample_offline(xadj, adjncy, prob, alias, seeds, fanout, seed):
     data = np.full((N, lps), FILL, np.uint32)
     sl = np.zeros((N, slen), np.uint32)
     sampled = C.c_uint64(0)
-    lib().orc_sample_offline(xadj, adjncy, prob, alias, np.ascontiguousarray(seeds, np.uint32), N, fan, len(fan),
+    lib().orc_sample_offline(xadj, len(xadj) - 1, adjncy, prob, alias, np.ascontiguousarray(seeds, np.uint32), N, fan, len(fan),
                              seed, data, sl, C.byref(sampled))
     return data, sl, sampled.value
 
@@ -196,7 +196,7 @@ def sample_online(xadj, adjncy, w, seeds, fanout, seed):
     data = np.full((N, lps), FILL, np.uint32)
     sl = np.zeros((N, slen), np.uint32)
     sampled = C.c_uint64(0)
-    lib().orc_sample_online(xadj, adjncy, np.ascontiguousarray(w, np.float32),
+    lib().orc_sample_online(xadj, len(xadj) - 1, adjncy, np.ascontiguousarray(w, np.float32),
                             np.ascontiguousarray(seeds, np.uint32), N, fan, len(fan), seed, data, sl,
                             C.byref(sampled))
     return data, sl, sampled.value

@@ -13,11 +13,15 @@
 namespace sky {
 
 __global__ __launch_bounds__(256) void walk_init_kernel(const uint32_t* __restrict__ seeds, uint32_t N, uint32_t len,
-                                                        uint32_t* __restrict__ paths, uint32_t* __restrict__ lengths) {
+                                                        uint32_t V, uint32_t* __restrict__ paths,
+                                                        uint32_t* __restrict__ lengths) {
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
   if (i >= N) return;
-  paths[(size_t)i * (len + 1)] = seeds[i];
-  lengths[i] = len;  // "still walking"; a walker that stops at step s stores s < len
+  const uint32_t v = seeds[i];
+  paths[(size_t)i * (len + 1)] = v;
+  // "still walking"; a walker that stops at step s stores s < len.  A start vertex that does not exist
+  // is recorded and never left.
+  lengths[i] = v < V ? len : 0u;
 }
 
 // Stop test and dead-end test of step s; collects the vertices whose table is still missing.
@@ -130,7 +134,7 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
     const uint32_t blocks = (N + 255) / 256;
     if (N) {
       SKY_HIP(hipMemsetAsync(bitmap, 0, (size_t)words * 4, st));
-      hipLaunchKernelGGL(walk_init_kernel, dim3(blocks), dim3(256), 0, st, seeds, N, len, paths, lengths);
+      hipLaunchKernelGGL(walk_init_kernel, dim3(blocks), dim3(256), 0, st, seeds, N, len, g->V, paths, lengths);
       for (uint32_t s = 0; s < len; ++s) {
         SKY_HIP(hipMemsetAsync(d_cnt, 0, 8, st));
         hipLaunchKernelGGL(walk_collect_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, N, len, s, stop_prob, seed,
@@ -394,7 +398,7 @@ int walk_online_node2vec(sky_graph* g, float p, float q, const uint32_t* seeds, 
     SKY_TRY(tm.mark("start", 0));
     if (N) {
       const uint32_t blocks = (N + 255) / 256;
-      hipLaunchKernelGGL(walk_init_kernel, dim3(blocks), dim3(256), 0, st, seeds, N, len, paths, lengths);
+      hipLaunchKernelGGL(walk_init_kernel, dim3(blocks), dim3(256), 0, st, seeds, N, len, g->V, paths, lengths);
       for (uint32_t s = 0; s < len; ++s)
         hipLaunchKernelGGL(n2v_step_kernel, dim3(N), dim3(N2V_T), 0, st, g->xadj, g->adjncy, g->adjwgt, len, s, p, q,
                            stop_prob, seed, paths, lengths);

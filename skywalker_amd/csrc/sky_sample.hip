@@ -31,7 +31,8 @@ __device__ __forceinline__ bool slot_filled(const HopGeom& g, const uint32_t* sl
 __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restrict__ xadj,
                                                          const uint32_t* __restrict__ adjncy,
                                                          const AliasEntry* __restrict__ table, uint64_t total,
-                                                         HopGeom g, uint64_t seed, uint32_t* __restrict__ data,
+                                                         uint32_t V, HopGeom g, uint64_t seed,
+                                                         uint32_t* __restrict__ data,
                                                          uint32_t* __restrict__ sl,
                                                          unsigned long long* __restrict__ sampled) {
   const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
@@ -43,7 +44,11 @@ __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restr
     const uint32_t i = (uint32_t)(rem % g.k);
     if (slot_filled(g, sl, si, s)) {
       const uint32_t v = data[si * g.lps + g.off + s];
-      const uint32_t o = xadj[v], deg = xadj[v + 1] - o;
+      uint32_t o = 0, deg = 0;
+      if (v < V) {  // a seed that does not exist has no children
+        o = xadj[v];
+        deg = xadj[v + 1] - o;
+      }
       if (deg != 0 && table[o].alias != SKY_INVALID) {
         uint32_t* out = data + si * g.lps + g.off_next + s * g.k;
         uint32_t cnt;
@@ -74,7 +79,7 @@ __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restr
 // during this call: first setter of the vertex's bit appends it.
 __global__ __launch_bounds__(256) void frontier_collect_kernel(const uint32_t* __restrict__ data,
                                                                const uint32_t* __restrict__ sl, uint64_t total,
-                                                               HopGeom g, uint32_t* __restrict__ bitmap,
+                                                               uint32_t V, HopGeom g, uint32_t* __restrict__ bitmap,
                                                                uint32_t* __restrict__ list,
                                                                uint32_t* __restrict__ count) {
   const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
@@ -82,6 +87,7 @@ __global__ __launch_bounds__(256) void frontier_collect_kernel(const uint32_t* _
   const uint64_t si = tid / g.width, s = tid % g.width;
   if (!slot_filled(g, sl, si, s)) return;
   const uint32_t v = data[si * g.lps + g.off + s];
+  if (v >= V) return;
   const uint32_t bit = 1u << (v & 31);
   if (atomicOr(&bitmap[v >> 5], bit) & bit) return;
   list[atomicAdd(count, 1u)] = v;
@@ -151,7 +157,7 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
         const uint64_t slots = (uint64_t)N * hg.width;
         SKY_HIP(hipMemsetAsync(d_count, 0, 4, st));
         hipLaunchKernelGGL(frontier_collect_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, st, data,
-                           sample_lengths, slots, hg, bitmap, list, d_count);
+                           sample_lengths, slots, g->V, hg, bitmap, list, d_count);
         uint32_t cnt = 0;
         SKY_HIP(hipMemcpyAsync(&cnt, d_count, 4, hipMemcpyDeviceToHost, st));
         SKY_HIP(hipStreamSynchronize(st));
@@ -160,7 +166,7 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
       const uint64_t total = (uint64_t)N * hg.width * hg.k;
       if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");
       hipLaunchKernelGGL(sample_hop_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, g->xadj,
-                         g->adjncy, g->table, total, hg, seed, data, sample_lengths, d_sampled);
+                         g->adjncy, g->table, total, g->V, hg, seed, data, sample_lengths, d_sampled);
     }
     SKY_TRY(tm.mark("sample", 0));
     SKY_TRY(tm.finish(nullptr, seconds));

@@ -15,7 +15,7 @@ constexpr int WALK_BLOCK = 256;
 
 __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
     const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
-    const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t len,
+    const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t V, uint32_t len,
     float stop_prob, uint64_t seed, uint32_t* __restrict__ paths, uint32_t* __restrict__ lengths,
     unsigned long long* __restrict__ sampled) {
   const uint32_t i = blockIdx.x * WALK_BLOCK + threadIdx.x;
@@ -24,7 +24,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
     uint32_t* path = paths + (size_t)i * (len + 1);
     uint32_t v = seeds[i];
     path[0] = v;
-    for (; s < len; ++s) {
+    for (; s < len && v < V; ++s) {  // a start vertex that does not exist is recorded and never left
       const u32x4 r = philox(seed, i, s, 0, DOM_WALK);
       if (stop_prob > 0.0f && u24(r.z) < stop_prob) break;
       const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
@@ -57,7 +57,7 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   SKY_HIP(hipEventRecord(e0, st));
   if (N)
     hipLaunchKernelGGL(walk_offline_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st, g->xadj,
-                       g->adjncy, g->table, seeds, N, len, stop_prob, seed, paths, lengths, d_sampled);
+                       g->adjncy, g->table, seeds, N, g->V, len, stop_prob, seed, paths, lengths, d_sampled);
   SKY_HIP(hipEventRecord(e1, st));
   SKY_HIP(hipStreamSynchronize(st));
   SKY_HIP(hipGetLastError());
@@ -94,8 +94,8 @@ __device__ __forceinline__ bool row_has(const uint32_t* __restrict__ row, uint32
 
 __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_kernel(
     const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
-    const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t len, float fp,
-    float fq, float fmax, float stop_prob, uint64_t seed, uint32_t* __restrict__ paths,
+    const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t V, uint32_t len,
+    float fp, float fq, float fmax, float stop_prob, uint64_t seed, uint32_t* __restrict__ paths,
     uint32_t* __restrict__ lengths, unsigned long long* __restrict__ sampled) {
   const uint32_t i = blockIdx.x * WALK_BLOCK + threadIdx.x;
   uint32_t s = 0;
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_kernel(
     uint32_t* path = paths + (size_t)i * (len + 1);
     uint32_t v = seeds[i], prev = 0, prev_off = 0, prev_deg = 0;
     path[0] = v;
-    for (; s < len; ++s) {
+    for (; s < len && v < V; ++s) {
       u32x4 r = philox(seed, i, s, 0, DOM_WALK);
       if (stop_prob > 0.0f && u24(r.z) < stop_prob) break;
       const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
@@ -155,7 +155,7 @@ int walk_node2vec_reject(sky_graph* g, float p, float q, const uint32_t* seeds, 
     SKY_TRY(tm.mark("start", 0));
     if (N)
       hipLaunchKernelGGL(walk_n2v_reject_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st,
-                         g->xadj, g->adjncy, g->table, seeds, N, len, fp, fq, fmax, stop_prob, seed, paths, lengths,
+                         g->xadj, g->adjncy, g->table, seeds, N, g->V, len, fp, fq, fmax, stop_prob, seed, paths, lengths,
                          d_sampled);
     SKY_TRY(tm.mark("walk", 0));
     double sec = 0;

@@ -67,3 +67,26 @@ def test_per_parent_draw_frequencies(orc):
     draws = data.to_host((N, 11))[:, 1:].ravel()
     assert sampled == N * 10
     assert chi_square_p(np.bincount(draws, minlength=d + 1)[1:], w.astype(np.float64) / w.sum(dtype=np.float64)) > 0.01
+
+
+def test_seeds_that_do_not_exist_have_no_children(orc):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(10, 8, 5)
+    V = len(xadj) - 1
+    w = orc.gen_weights(orc.W_UNIFORM, 5, len(adjncy), 1.0, 10.0)
+    seeds = orc.gen_seeds(6, V, 200)
+    seeds[::5] = V
+    seeds[1] = 0xFFFFFFFF
+    fanout = [1, 4, 3]
+    lps, slen = capi.sample_layout(fanout)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    d_on, sl_on, s_on, _ = g.sample_online(seeds, fanout, 3)
+    on = (d_on.to_host((200, lps)), sl_on.to_host((200, slen)))
+    g.build_tables()
+    d_off, sl_off, s_off, _ = g.sample_offline(seeds, fanout, 3)
+    off = (d_off.to_host((200, lps)), sl_off.to_host((200, slen)))
+    g.free()
+    odata, osl, osampled = orc.sample_online(xadj, adjncy, w, seeds, fanout, 3)
+    for got, s in ((on, s_on), (off, s_off)):
+        assert np.array_equal(got[0], odata) and np.array_equal(got[1], osl) and s == osampled
+    assert np.all(osl[seeds >= V] == 0)

@@ -198,3 +198,42 @@ def test_node2vec_rejection_second_step_law(orc):
     law /= law.sum()
     assert second[2] == 0 and sampled == 2 * N
     assert chi_square_p(second[[0, 1, 3, 4]], law[[0, 1, 3, 4]]) > 0.01
+
+
+def test_start_vertices_that_do_not_exist_never_move(orc):
+    # same rule as the oracle's, in every walk kernel: the seed is recorded, the length is 0
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(10, 8, 3)
+    V = len(xadj) - 1
+    w = orc.gen_weights(orc.W_UNIFORM, 3, len(adjncy), 1.0, 10.0)
+    seeds = orc.gen_seeds(2, V, 300)
+    seeds[::7] = V
+    seeds[3::11] = 0xFFFFFFFF
+    seeds[5] = V + 1
+
+    def host(r, length):
+        out = (r[0].to_host((len(seeds), length + 1)), r[1].to_host(), r[2])
+        r[0].free()
+        r[1].free()
+        return out
+
+    g = capi.Graph.upload(xadj, adjncy, w)
+    capi.set_option("online_full_build", 0)
+    try:
+        lazy = host(g.walk_online(capi.BIAS_STATIC, 1.0, 1.0, seeds, 12, 0.05, 9), 12)
+    finally:
+        capi.set_option("online_full_build", -1)
+    n2v = host(g.walk_online(capi.BIAS_NODE2VEC, 2.0, 0.5, seeds, 12, 0.05, 9), 12)
+    g.build_tables()
+    prob, alias, _ = g.tables()
+    off = host(g.walk_offline(seeds, 12, 0.05, 9), 12)
+    rej = host(g.walk_online(capi.BIAS_NODE2VEC_REJECT, 2.0, 0.5, seeds, 12, 0.05, 9), 12)
+    g.free()
+    want = orc.walk_offline(xadj, adjncy, prob, alias, seeds, 12, 0.05, 9)
+    for got in (off, lazy):
+        assert np.array_equal(got[1], want[1]) and np.array_equal(got[0], want[0]) and got[2] == want[2]
+    want = orc.walk_online(xadj, adjncy, w, 1, 2.0, 0.5, seeds, 12, 0.05, 9)
+    assert np.array_equal(n2v[1], want[1]) and np.array_equal(n2v[0], want[0]) and n2v[2] == want[2]
+    want = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, 2.0, 0.5, seeds, 12, 0.05, 9)
+    assert np.array_equal(rej[1], want[1]) and np.array_equal(rej[0], want[0]) and rej[2] == want[2]
+    assert np.all(off[1][seeds >= V] == 0)

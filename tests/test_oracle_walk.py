@@ -254,3 +254,29 @@ def test_sample_draw_law_and_online_equals_offline(orc):
                         w.astype(np.float64) / w.sum(dtype=np.float64)) > 0.01
     d2, sl2, s2 = orc.sample_online(xadj, adjncy, w, np.zeros(N, np.uint32), [1, 8], 3)
     assert np.array_equal(data, d2) and np.array_equal(sl, sl2) and sampled == s2
+
+
+def test_start_vertices_that_do_not_exist_never_move(orc):
+    # every walk and the sampler record such a seed and stop there: length 0, no children
+    xadj, adjncy = orc.rmat_csr(8, 8, 3)
+    V = len(xadj) - 1
+    w = orc.gen_weights(orc.W_UNIFORM, 3, len(adjncy), 1.0, 10.0)
+    prob, alias, _ = orc.alias_build(xadj, w)
+    seeds = np.array([5, V, 7, 0xFFFFFFFF, V + 1000, 9], np.uint32)
+    bad = seeds >= V
+    runs = [orc.walk_offline(xadj, adjncy, prob, alias, seeds, 6, 0.0, 1),
+            orc.walk_online(xadj, adjncy, w, 0, 1.0, 1.0, seeds, 6, 0.0, 1),
+            orc.walk_online(xadj, adjncy, w, 1, 2.0, 0.5, seeds, 6, 0.0, 1),
+            orc.walk_node2vec_reject(xadj, adjncy, prob, alias, 2.0, 0.5, seeds, 6, 0.0, 1)]
+    for paths, lengths, sampled in runs:
+        assert np.array_equal(paths[:, 0], seeds)
+        assert np.all(lengths[bad] == 0) and np.all(paths[bad, 1:] == orc.FILL)
+        assert sampled == int(lengths.sum())
+    good = runs[0]
+    ref = orc.walk_offline(xadj, adjncy, prob, alias, seeds[~bad], 6, 0.0, 1)
+    assert np.array_equal(good[1][~bad] > 0, ref[1] > 0)  # the others walk as usual (walker ids differ, so not the same paths)
+    for data, sl, sampled in (orc.sample_offline(xadj, adjncy, prob, alias, seeds, [1, 3, 2], 1),
+                              orc.sample_online(xadj, adjncy, w, seeds, [1, 3, 2], 1)):
+        assert np.array_equal(data[:, 0], seeds)
+        assert np.all(data[bad, 1:] == orc.FILL) and np.all(sl[bad] == 0)
+        assert sampled == int(sl.sum())
