@@ -38,8 +38,8 @@ TRAFFIC_PER_EDGE = {"stream": 19.0, "mw10": 12.1, "mw9": 16.8, "mw4": 12.2, "mw3
                     "tiled_emit": 24.4, "tiled_sum": 4.3, "tiled_totals": 4.3}
 WALK_TRAFFIC_PER_STEP = 398.5  # walk_offline_kernel, same source
 KERNEL_OF = {  # build_profile entry -> kernel symbol
-    "bin": "bin_count_kernel+bin_scatter_kernel", "lds_w1": "build_merge_kernel<64,1>",
-    "lds_w2": "build_merge_kernel<64,2>",
+    "bin": "bin_count_kernel+bin_scatter_kernel", "lds_w1": "build_merge_kernel<64,4>",
+    "lds_w2": "build_merge_kernel<64,8>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
     "streamed": "huge_prefix_kernel+build_huge_kernel", "stream": "build_stream_kernel",
@@ -47,8 +47,9 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
 }
 KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
                   for g in (2, 4, 8, 16, 32) for x in ("", "x")})
-KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,2>" % (64 * nw) for nw in range(2, 17)})
-KERNEL_OF["mw10"] = "build_merge_kernel<448,3>"
+KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,8>" % (64 * nw) for nw in range(2, 17)})
+KERNEL_OF["mw10"] = "build_merge_kernel<512,10>"
+KERNEL_OF["mw3"] = "build_merge_kernel<256,6>"
 
 
 def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sample=1_000_000):

@@ -521,12 +521,15 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const RowRef* __restric
 constexpr uint64_t MERGE_CNT = 1ull << 52;
 constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
 
-template <int ROWT, int T>
+template <int ROWT, int PER>
 __global__ __launch_bounds__(ROWT, (ROWT == 576 ? 6 : 4)) void build_merge_kernel(const RowRef* __restrict__ vlist,
                                                            const uint32_t* __restrict__ xadj,
                                                            const float* __restrict__ wgt,
                                                            AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
-  constexpr int PER = 4 * T;  // consecutive slots per thread, counted from the row's 16-byte aligned start
+  // PER consecutive slots per thread, counted from the row's 16-byte aligned start; a thread moves them as
+  // quads when PER is a multiple of 4, as pairs otherwise (its first slot is then only 8-byte aligned)
+  constexpr int VEC = PER % 4 == 0 ? 4 : 2;
+  static_assert(PER % VEC == 0 && PER <= 16, "whole vectors, and `live` has one bit per slot");
   constexpr int CAP = ROWT * PER;
   constexpr int NW = ROWT / 64;
   constexpr uint32_t TOP = CAP + 1;  // heavy h lives at index TOP - h of the value array and of the result array
@@ -551,18 +554,25 @@ __global__ __launch_bounds__(ROWT, (ROWT == 576 ? 6 : 4)) void build_merge_kerne
   WSum3 sum{0.0, 0.0, 0.0};
   if (wave_on) {
 #pragma unroll
-    for (int t = 0; t < T; ++t) {
-      const uint32_t pos = pos0 + 4u * t;
-      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (pos < span) x = *reinterpret_cast<const float4*>(wgt + base + pos);
-      const float xs[4] = {x.x, x.y, x.z, x.w};
+    for (int t = 0; t < PER / VEC; ++t) {
+      const uint32_t pos = pos0 + (uint32_t)(VEC * t);
+      float xs[4] = {0.f, 0.f, 0.f, 0.f};
+      if (pos < span) {
+        if constexpr (VEC == 4) {
+          const float4 x = *reinterpret_cast<const float4*>(wgt + base + pos);
+          xs[0] = x.x; xs[1] = x.y; xs[2] = x.z; xs[3] = x.w;
+        } else {
+          const float2 x = *reinterpret_cast<const float2*>(wgt + base + pos);
+          xs[0] = x.x; xs[1] = x.y;
+        }
+      }
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < VEC; ++k) {
         const uint32_t idx = pos + k;
         const bool in = idx >= lead && idx < span;
-        if (in) live |= 1u << (t * 4 + k);
-        wd[t * 4 + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
-        wsum3_add(sum, wd[t * 4 + k]);
+        if (in) live |= 1u << (t * VEC + k);
+        wd[t * VEC + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
+        wsum3_add(sum, wd[t * VEC + k]);
       }
     }
     sum = group_sum_wsum3<64>(sum);
@@ -687,16 +697,21 @@ __global__ __launch_bounds__(ROWT, (ROWT == 576 ? 6 : 4)) void build_merge_kerne
       }
     }
 #pragma unroll
-    for (int t = 0; t < T; ++t) {
-      const uint32_t pos = pos0 + 4u * t;
-      if (pos >= lead && pos + 4 <= span) {
-        const float p4[4] = {op[4 * t], op[4 * t + 1], op[4 * t + 2], op[4 * t + 3]};
-        const uint32_t a4[4] = {oa[4 * t], oa[4 * t + 1], oa[4 * t + 2], oa[4 * t + 3]};
-        store_entries4(table + base + pos, p4, a4);
+    for (int t = 0; t < PER / VEC; ++t) {
+      const uint32_t pos = pos0 + (uint32_t)(VEC * t);
+      if (pos >= lead && pos + VEC <= span) {
+        if constexpr (VEC == 4) {
+          const float p4[4] = {op[4 * t], op[4 * t + 1], op[4 * t + 2], op[4 * t + 3]};
+          const uint32_t a4[4] = {oa[4 * t], oa[4 * t + 1], oa[4 * t + 2], oa[4 * t + 3]};
+          store_entries4(table + base + pos, p4, a4);
+        } else {
+          *reinterpret_cast<uint4*>(table + base + pos) =
+              make_uint4(__float_as_uint(op[2 * t]), oa[2 * t], __float_as_uint(op[2 * t + 1]), oa[2 * t + 1]);
+        }
       } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if ((live >> (t * 4 + k)) & 1) table[base + pos + k] = AliasEntry{op[4 * t + k], oa[4 * t + k]};
+        for (int k = 0; k < VEC; ++k)
+          if ((live >> (t * VEC + k)) & 1) table[base + pos + k] = AliasEntry{op[VEC * t + k], oa[VEC * t + k]};
       }
     }
   }
@@ -924,8 +939,8 @@ int prepare_build_scratch(uint32_t max_rows) {
   if (!sc.blk_cnt) SKY_HIP(hipMalloc((void**)&sc.blk_cnt, (size_t)BIN_BLOCKS * CLS_COUNT * 4));
   if (!sc.lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
-#define SKY_BIG(NW) SKY_TRY(enable_big_lds(build_merge_kernel<64 * NW, 2>, (64 * NW * 8 + 2) * 14))
-    SKY_TRY(enable_big_lds(build_merge_kernel<448, 3>, (448 * 12 + 2) * 14));
+#define SKY_BIG(NW) SKY_TRY(enable_big_lds(build_merge_kernel<64 * NW, 8>, (64 * NW * 8 + 2) * 14))
+    SKY_TRY(enable_big_lds(build_merge_kernel<512, 10>, (512 * 10 + 2) * 14));
     SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
 #undef SKY_BIG
     sc.lds_enabled = true;
@@ -997,10 +1012,10 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
-  auto mrg = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
+  auto mrg = [&](int cls, auto kernel, int rowt, int per, const char* name) -> int {
     const uint32_t cnt = counts[cls];
     if (cnt) {
-      const size_t bytes = ((size_t)rowt * 4 * t + 2) * 14;
+      const size_t bytes = ((size_t)rowt * per + 2) * 14;
       hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
                          g->table, g->valid);
     }
@@ -1009,13 +1024,17 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   static const char* const mw_name[15] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9",
                                           "mw10", "mw11", "mw12", "mw13", "mw14", "mw15", "mw16"};
   if (g_row_merge) {
-    SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 1>, 64, 1, "lds_w1"));
-    SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 2>, 64, 2, "lds_w2"));
-#define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 2>, 64 * NW, 2, mw_name[NW - 2]))
-    SKY_MW(2); SKY_MW(3); SKY_MW(4); SKY_MW(5); SKY_MW(6); SKY_MW(7); SKY_MW(8); SKY_MW(9);
-    // rows of 4605..5117 entries: 7 wavefronts of 12 slots per thread.  Two workgroups of 10 wavefronts would
-    // have to fit 6 wavefronts per SIMD (80 registers, spills); 7 fit at 4 per SIMD
-    SKY_TRY(mrg(CLS_MW2 + 8, build_merge_kernel<448, 3>, 448, 3, mw_name[8]));
+    SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 4>, 64, 4, "lds_w1"));
+    SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 8>, 64, 8, "lds_w2"));
+#define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 8>, 64 * NW, 8, mw_name[NW - 2]))
+    SKY_MW(2);
+    // rows of 1022..1533 entries: 4 wavefronts of 6 slots per thread rather than 3 of 8 (13 % faster: every
+    // SIMD of the CU gets the same number of wavefronts of a workgroup)
+    SKY_TRY(mrg(CLS_MW2 + 1, build_merge_kernel<256, 6>, 256, 6, mw_name[1]));
+    SKY_MW(4); SKY_MW(5); SKY_MW(6); SKY_MW(7); SKY_MW(8); SKY_MW(9);
+    // rows of 4605..5117 entries: 8 wavefronts of 10 slots per thread.  Two workgroups of 10 wavefronts would
+    // have to fit 6 wavefronts per SIMD (80 registers, spills); 8 fit at 4 per SIMD, every SIMD alike
+    SKY_TRY(mrg(CLS_MW2 + 8, build_merge_kernel<512, 10>, 512, 10, mw_name[8]));
     SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
 #undef SKY_MW
   } else {
