@@ -48,8 +48,8 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
 KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
                   for g in (2, 4, 8, 16, 32) for x in ("", "x")})
 KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,8>" % (64 * nw) for nw in range(2, 17)})
-KERNEL_OF["mw10"] = "build_merge_kernel<512,10>"
-KERNEL_OF["mw3"] = "build_merge_kernel<256,6>"
+KERNEL_OF.update({"mw3": "build_merge_kernel<256,6>", "mw5": "build_merge_kernel<256,10>", "mw6": "build_merge_kernel<512,6>",
+                  "mw7": "build_merge_kernel<256,14>", "mw9": "build_merge_kernel<768,6>", "mw10": "build_merge_kernel<512,10>"})
 
 
 def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sample=1_000_000):

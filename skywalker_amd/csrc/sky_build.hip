@@ -522,7 +522,7 @@ constexpr uint64_t MERGE_CNT = 1ull << 52;
 constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
 
 template <int ROWT, int PER>
-__global__ __launch_bounds__(ROWT, (ROWT == 576 ? 6 : 4)) void build_merge_kernel(const RowRef* __restrict__ vlist,
+__global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __restrict__ vlist,
                                                            const uint32_t* __restrict__ xadj,
                                                            const float* __restrict__ wgt,
                                                            AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
@@ -941,6 +941,7 @@ int prepare_build_scratch(uint32_t max_rows) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
 #define SKY_BIG(NW) SKY_TRY(enable_big_lds(build_merge_kernel<64 * NW, 8>, (64 * NW * 8 + 2) * 14))
     SKY_TRY(enable_big_lds(build_merge_kernel<512, 10>, (512 * 10 + 2) * 14));
+    SKY_TRY(enable_big_lds(build_merge_kernel<768, 6>, (768 * 6 + 2) * 14));
     SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
 #undef SKY_BIG
     sc.lds_enabled = true;
@@ -1027,13 +1028,19 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 4>, 64, 4, "lds_w1"));
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 8>, 64, 8, "lds_w2"));
 #define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 8>, 64 * NW, 8, mw_name[NW - 2]))
+    // Class nw holds rows that fit 512 nw slots.  Where a shape with an even number of slots per thread and a
+    // multiple of 4 wavefronts covers that span exactly, it is used instead of nw wavefronts of 8 slots: every
+    // SIMD of the CU then carries the same number of a workgroup's wavefronts, and 6..10 slots per thread need
+    // 70..110 registers (measured on rows of one class each: 13 % faster for nw = 3, 24 % for 5, 41 % for 6,
+    // 2 % for 7, 31 % for 9, 28 % for 10, where 10 wavefronts of 8 slots also spill).
     SKY_MW(2);
-    // rows of 1022..1533 entries: 4 wavefronts of 6 slots per thread rather than 3 of 8 (13 % faster: every
-    // SIMD of the CU gets the same number of wavefronts of a workgroup)
     SKY_TRY(mrg(CLS_MW2 + 1, build_merge_kernel<256, 6>, 256, 6, mw_name[1]));
-    SKY_MW(4); SKY_MW(5); SKY_MW(6); SKY_MW(7); SKY_MW(8); SKY_MW(9);
-    // rows of 4605..5117 entries: 8 wavefronts of 10 slots per thread.  Two workgroups of 10 wavefronts would
-    // have to fit 6 wavefronts per SIMD (80 registers, spills); 8 fit at 4 per SIMD, every SIMD alike
+    SKY_MW(4);
+    SKY_TRY(mrg(CLS_MW2 + 3, build_merge_kernel<256, 10>, 256, 10, mw_name[3]));
+    SKY_TRY(mrg(CLS_MW2 + 4, build_merge_kernel<512, 6>, 512, 6, mw_name[4]));
+    SKY_TRY(mrg(CLS_MW2 + 5, build_merge_kernel<256, 14>, 256, 14, mw_name[5]));
+    SKY_MW(8);
+    SKY_TRY(mrg(CLS_MW2 + 7, build_merge_kernel<768, 6>, 768, 6, mw_name[7]));
     SKY_TRY(mrg(CLS_MW2 + 8, build_merge_kernel<512, 10>, 512, 10, mw_name[8]));
     SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
 #undef SKY_MW
