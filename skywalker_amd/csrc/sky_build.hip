@@ -69,13 +69,21 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
   }
   __syncthreads();
   const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
+  uint32_t tiny_edges = 0;  // rows of 1..2 entries, the commonest kind of a power-law graph, stay out of the LDS atomics
   for (uint32_t i = lo + threadIdx.x; i < hi; i += 256u) {
     const uint32_t v = src ? src[i] : i;
     const uint32_t d = xadj[v + 1] - xadj[v];
     const int c = degree_class(d);
-    if (c >= CLS_G2) atomicAdd(&s_cnt[c], 1u);
-    if (c >= CLS_TINY) atomicAdd(&s_edges[c], (unsigned long long)d);
+    if (c >= CLS_G2) {
+      atomicAdd(&s_cnt[c], 1u);
+      atomicAdd(&s_edges[c], (unsigned long long)d);
+    } else {
+      tiny_edges += d;  // 0 for an empty row
+    }
   }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) tiny_edges += (uint32_t)__shfl_xor((int)tiny_edges, m, 64);
+  if ((threadIdx.x & 63) == 0 && tiny_edges) atomicAdd(&s_edges[CLS_TINY], (unsigned long long)tiny_edges);
   __syncthreads();
   if (threadIdx.x < CLS_COUNT) {
     blk_cnt[blockIdx.x * CLS_COUNT + threadIdx.x] = s_cnt[threadIdx.x];
@@ -125,21 +133,24 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
       if (c == CLS_EMPTY) {
         valid[v] = 0;
       } else if (c == CLS_TINY) {
+        // a weight adds to the exact sum iff it is at least 2^-64
+        constexpr float UNIT = 5.421010862427522170037e-20f;  // 2^-64
         const float w0 = clamp_weight(wgt[off]);
         if (d == 1) {
-          const u128 q = weight_fixed(w0);
-          const bool ok = (q.lo | q.hi) != 0;
+          const bool ok = w0 >= UNIT;
           table[off] = AliasEntry{ok ? 1.0f : 0.0f, ok ? 0u : SKY_INVALID};
           valid[v] = ok;
         } else {
           const float w1 = clamp_weight(wgt[off + 1]);
-          const u128 s = add128(weight_fixed(w0), weight_fixed(w1));
-          if ((s.lo | s.hi) == 0) {
+          if (!(w0 >= UNIT || w1 >= UNIT)) {
             table[off] = table[off + 1] = AliasEntry{0.0f, SKY_INVALID};
             valid[v] = 0;
           } else {
-            const Ledger L = make_ledger(2, s);
-            const Entry e0 = classify(w0, L), e1 = classify(w1, L);
+            WSum3 S{0.0, 0.0, 0.0};
+            wsum3_add(S, (double)w0);
+            wsum3_add(S, (double)w1);
+            const Ledger L = make_ledger_small(2, wsum3_to_double(S));
+            const Entry e0 = classify_small((double)w0, true, L), e1 = classify_small((double)w1, true, L);
             // a lone heavy is the last heavy: it keeps its bucket and tops up the light
             table[off] = AliasEntry{e0.heavy ? 1.0f : (float)e0.p, (!e0.heavy && e1.heavy) ? 1u : 0u};
             table[off + 1] = AliasEntry{e1.heavy ? 1.0f : (float)e1.p, (!e1.heavy && e0.heavy) ? 0u : 1u};
