@@ -33,7 +33,7 @@ namespace sky {
 __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d == 0) return CLS_EMPTY;
   if (d <= 2) return CLS_TINY;
-  // the 6-slot variants of the narrow groups (CLS_G2X .. CLS_G16X) cost more per edge than they gain in fill
+  // 6-slot variants of the narrower groups cost more per edge than they gain in fill
   if (d <= 5) return CLS_G2;
   if (d <= 13) return CLS_G4;
   if (d <= 29) return CLS_G8;
@@ -1005,13 +1005,9 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
   SKY_TRY(grp(CLS_G2, build_group_kernel<2, 4>, 2, "g2"));
-  SKY_TRY(grp(CLS_G2X, build_group_kernel<2, 6>, 2, "g2x"));
   SKY_TRY(grp(CLS_G4, build_group_kernel<4, 4>, 4, "g4"));
-  SKY_TRY(grp(CLS_G4X, build_group_kernel<4, 6>, 4, "g4x"));
   SKY_TRY(grp(CLS_G8, build_group_kernel<8, 4>, 8, "g8"));
-  SKY_TRY(grp(CLS_G8X, build_group_kernel<8, 6>, 8, "g8x"));
   SKY_TRY(grp(CLS_G16, build_group_kernel<16, 4>, 16, "g16"));
-  SKY_TRY(grp(CLS_G16X, build_group_kernel<16, 6>, 16, "g16x"));
   SKY_TRY(grp(CLS_G32, build_group_kernel<32, 4>, 32, "g32"));
   SKY_TRY(grp(CLS_G32X, build_group_kernel<32, 6>, 32, "g32x"));
 

@@ -29,27 +29,23 @@ namespace sky {
 
 // Degree classes of the offline build.  Upper bounds are inclusive.
 enum BuildClass : int {
-  CLS_EMPTY = 0,   // deg 0            handled while binning
-  CLS_TINY = 1,    // deg 1..2         one lane per vertex, handled while binning
-  CLS_G2 = 2,      // deg 3..5         2 lanes per row, 4 slots per lane
-  CLS_G2X = 3,     // deg <= 11        2 lanes, 6 slots per lane
-  CLS_G4 = 4,      // deg <= 13        4 lanes, 4 slots
-  CLS_G4X = 5,     // deg <= 23        4 lanes, 6 slots
-  CLS_G8 = 6,      // deg <= 29
-  CLS_G8X = 7,     // deg <= 47
-  CLS_G16 = 8,     // deg <= 61
-  CLS_G16X = 9,    // deg <= 95
-  CLS_G32 = 10,    // deg <= 125
-  CLS_G32X = 11,   // deg <= 191
-  CLS_LDS_W1 = 12, // deg <= 253       one wavefront, LDS prefix arrays, 4 entries per lane
-  CLS_LDS_W2 = 13, // deg <= 509       one wavefront, 8 entries per lane
-  CLS_MW2 = 14,    // deg <= 512 * nw - 3, nw = 2..16: one workgroup of nw wavefronts, 8 entries per thread;
-  CLS_MW16 = 28,   //                  class CLS_MW2 + nw - 2 (nw = 10: 7 wavefronts, 12 entries per thread)
-  CLS_STREAM = 29, // deg 24577..65533  one workgroup streams the row, its heavies stay in LDS.  Two classes, the
-  CLS_STREAM_LAST = 30, // deg 8190..24576  longer rows first, listed back to back and built by one launch, which so
-                   //                  does not end on its longest rows
-  CLS_HUGE = 31,   // above            built tile by tile by the whole GPU
-  CLS_COUNT = 32
+  CLS_EMPTY = 0,    // deg 0            handled while binning
+  CLS_TINY = 1,     // deg 1..2         one lane per vertex, handled while binning
+  CLS_G2 = 2,       // deg 3..5         2 lanes per row, 4 slots per lane
+  CLS_G4 = 3,       // deg <= 13        4 lanes
+  CLS_G8 = 4,       // deg <= 29        8 lanes
+  CLS_G16 = 5,      // deg <= 61        16 lanes
+  CLS_G32 = 6,      // deg <= 125       32 lanes
+  CLS_G32X = 7,     // deg <= 191       32 lanes, 6 slots per lane
+  CLS_LDS_W1 = 8,   // deg <= 253       one wavefront per row, 4 slots per lane
+  CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
+  CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..16 (class CLS_MW2 + nw - 2): one workgroup per row whose
+  CLS_MW16 = 24,    //                  threads cover 512 * nw slots
+  CLS_STREAM = 25,  // deg 24577..65533 one workgroup streams the row, its heavies stay in LDS.  Two classes, the
+  CLS_STREAM_LAST = 26,  // deg 8190..24576  longer rows first, listed back to back and built by one launch, which so
+                    //                  does not end on its longest rows
+  CLS_HUGE = 27,    // above            built tile by tile by the whole GPU
+  CLS_COUNT = 28
 };
 
 // One listed row of a degree class: the build kernels read where the row lies from the list itself
