@@ -210,3 +210,39 @@ def test_build_profile_is_opt_in(orc):
     g.free()
     for a, b in zip(before, after):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def test_degenerate_inputs(orc):
+    # a graph without edges, a graph without vertices, no walkers, zero steps: every entry point returns
+    # cleanly and the counts are zero
+    from skywalker_amd import capi
+    for V in (0, 1, 300):
+        xadj = np.zeros(V + 1, np.uint32)
+        g = capi.Graph.upload(xadj, np.zeros(0, np.uint32), np.zeros(0, np.float32))
+        assert g.V == V and g.E == 0
+        g.build_tables()
+        prob, alias, valid = g.tables()
+        assert len(prob) == 0 and len(alias) == 0 and len(valid) == V and not valid.any()
+        seeds = np.arange(min(V, 5), dtype=np.uint32)
+        for length in (0, 4):
+            p, l, sampled, _ = g.walk_offline(seeds, length, 0.0, 1)
+            assert sampled == 0 and not l.to_host().any()
+            assert np.array_equal(p.to_host((len(seeds), length + 1))[:, 0], seeds)
+            p, l, sampled, _ = g.walk_online(capi.BIAS_STATIC, 1.0, 1.0, seeds, length, 0.0, 1)
+            assert sampled == 0 and not l.to_host().any()
+            p, l, sampled, _ = g.walk_online(capi.BIAS_NODE2VEC_REJECT, 2.0, 0.5, seeds, length, 0.0, 1)
+            assert sampled == 0 and not l.to_host().any()
+        d, sl, sampled, _ = g.sample_offline(seeds, [1, 3, 2], 1)
+        assert sampled == 0 and not sl.to_host().any()
+        d, sl, sampled, _ = g.sample_online(seeds, [1, 3, 2], 1)
+        assert sampled == 0 and not sl.to_host().any()
+        g.free()
+    # an ordinary graph, no walkers
+    xadj, adjncy = orc.rmat_csr(8, 4, 1)
+    g = capi.Graph.upload(xadj, adjncy, None)  # unit weights
+    g.build_tables()
+    none = np.zeros(0, np.uint32)
+    assert g.walk_offline(none, 5, 0.0, 1)[2] == 0
+    assert g.walk_online(capi.BIAS_NODE2VEC, 2.0, 0.5, none, 5, 0.0, 1)[2] == 0
+    assert g.sample_offline(none, [1, 2], 1)[2] == 0
+    g.free()
