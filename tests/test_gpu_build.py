@@ -246,3 +246,30 @@ def test_degenerate_inputs(orc):
     assert g.walk_online(capi.BIAS_NODE2VEC, 2.0, 0.5, none, 5, 0.0, 1)[2] == 0
     assert g.sample_offline(none, [1, 2], 1)[2] == 0
     g.free()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_mixtures_of_every_class(orc, seed):
+    # both ends of every degree class plus random rows of every size, a different weight law per seed,
+    # special values sprinkled into some
+    from helpers import weights
+    rng = np.random.default_rng(1000 + seed)
+    ends = [0, 1, 2, 3, 5, 6, 13, 14, 29, 30, 61, 62, 125, 126, 191, 192, 253, 254, 509, 8190, 24576, 24577, 65533, 65534]
+    for nw in range(2, 17):
+        ends += [512 * (nw - 1) - 2, 512 * nw - 3]
+    degs = ends + list(rng.integers(0, 70, 3000)) + list(rng.integers(60, 600, 600)) + \
+        list(rng.integers(500, 8300, 260)) + list(rng.integers(8000, 66000, 12)) + list(rng.integers(66000, 400000, 2))
+    degs = np.array(degs)
+    rng.shuffle(degs)
+    xadj = np.zeros(len(degs) + 1, np.uint32)
+    xadj[1:] = np.cumsum(degs)
+    E = int(xadj[-1])
+    adjncy = rng.integers(0, len(degs), E).astype(np.uint32)
+    dist = ["lognormal", "uniform", "lognormal2", "nearequal", "sparse", "unit", "equal"][seed % 7]
+    w = weights(E, rng, dist)
+    if seed % 3 == 0:
+        pick = rng.random(E) < 0.001
+        special = np.array([0.0, -1.0, np.inf, np.nan, 1e-30, 2.0 ** -64, 2.0 ** 32, 1e38], np.float32)
+        w[pick] = special[rng.integers(0, len(special), pick.sum())]
+    with np.errstate(all="ignore"):
+        build_and_compare(orc, xadj, adjncy, w, "mixture %d/%s" % (seed, dist))
