@@ -11,7 +11,10 @@
  *   - every function returns 0 on success or a negative sky_status; the message of
  *     the last failure on the calling thread is available from sky_last_error().
  *   - a sky_graph owns the device-resident CSR and, after sky_alias_build_all, the
- *     alias tables.  One host thread per sky_graph; calls are synchronous.
+ *     alias tables.  One host thread per sky_graph; calls are synchronous.  The scratch memory of the table
+ *     build and the options of sky_set_option belong to the process, not to a graph: calls that build tables
+ *     (sky_alias_build_all, sky_walk_online, sky_sample_online) must not overlap, whatever graphs they are for,
+ *     like the reference's entry functions, which share the default stream.
  *   - "device pointer" arguments are HIP device addresses on the current device
  *     (from sky_device_malloc, or any other allocator of the same process).
  *   - `seconds` outputs report the kernel region only (launch to completion,
