@@ -159,6 +159,7 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
         }
       } else {
         vlist[atomicAdd(&s_cur[c], 1u)] = RowRef{v, off, d, 0};
+        valid[v] = 1;  // written here, next to its neighbours' flags; the row's kernel clears it if the row has no weight
       }
     }
   }
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
       t[1] = AliasEntry{op[2 * h + 1], oa[2 * h + 1]};
     }
   }
-  if (gl == 0 && d) valid[rr.v] = row_ok;
+  if (gl == 0 && d && !row_ok) valid[rr.v] = 0;  // the binning pass has set it
 }
 
 // ---------------------------------------------------------------- one row per workgroup, prefix arrays in LDS
@@ -516,7 +517,6 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const RowRef* __restric
         }
     }
   }
-  if (tid == 0) valid[v] = 1;
 }
 
 // ---------------------------------------------------------------- one row per workgroup, pairing by merge
@@ -726,7 +726,6 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
       }
     }
   }
-  if (tid == 0) valid[v] = 1;
 }
 
 // ---------------------------------------------------------------- rows beyond LDS: global scratch
@@ -835,7 +834,6 @@ __global__ __launch_bounds__(HUGE_T) void build_huge_kernel(const RowRef* __rest
       }
       table[off + i] = AliasEntry{op, oa};
     }
-    if (tid == 0) valid[v] = 1;
     __syncthreads();
   }
 }

@@ -357,7 +357,6 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
       const uint32_t slot = s_slot[h];
       table[r.base + slot] = AliasEntry{1.0f, slot - r.lead};
     }
-  if (tid == 0) valid[rr.v] = 1;
 }
 
 namespace {

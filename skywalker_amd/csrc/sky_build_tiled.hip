@@ -565,7 +565,6 @@ __global__ __launch_bounds__(TL_T) void tiled_emit_kernel(const TileGeom* __rest
         }
     }
   }
-  if (T == 0 && tid == 0) valid[r.v] = 1;
 }
 
 // ---------------------------------------------------------------- host driver
