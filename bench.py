@@ -43,7 +43,6 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
     "streamed": "huge_prefix_kernel+build_huge_kernel", "stream": "build_stream_kernel",
-    "stream_deferred": "tile-parallel path for rows deferred by build_stream_kernel",
 }
 KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
                   for g in (2, 4, 8, 16, 32) for x in ("", "x")})

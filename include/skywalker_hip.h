@@ -149,8 +149,8 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      "row_merge" (default 1): rows of 62..8189 entries pair lights and heavies by a merge of their prefix
  *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table.
  *      "stream_min_edges" (default 4000000): rows of 8190..65533 entries have a kernel of their own (one workgroup
- *      streams a row); when a build holds no more than this many entries in such rows they go to the tile-parallel
- *      path instead, which then needs no answer from the device in the middle of the build.  Tests set 0.
+ *      streams a row); when a build holds no more than this many entries in such rows, too few to fill the GPU
+ *      with one workgroup each, they go to the tile-parallel path instead.  Tests set 0.
  *      "build_profile" (default 0): 1 records a HIP event after every kernel of sky_alias_build_all for
  *      sky_last_build_profile (about 3 microseconds each; a small graph pays 20 % of its build for them).
  *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:

@@ -1068,19 +1068,17 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
   }
 
-  const RowRef* deferred = nullptr;
   uint32_t stream_rows = 0;
   uint64_t stream_edges = 0;
   for (int c = CLS_STREAM; c <= CLS_STREAM_LAST; ++c) {
     stream_rows += counts[c];
     stream_edges += host.edges[c];
   }
-  // A small streaming class is not worth its own launch and the host round trip that asks for its deferred
-  // rows: its rows then go to the tile-parallel path together with the HUGE class that follows them in the list.
+  // A small streaming class is not worth its own launch: its rows then go to the tile-parallel path together
+  // with the HUGE class that follows them in the list.
   const bool stream_to_tiled = !g_row_merge || stream_edges <= g_stream_min_edges;
   if (stream_rows && !stream_to_tiled) {  // one launch over the two lists, which lie back to back
-    uint32_t nd = 0;
-    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], stream_rows, &deferred, &nd));
+    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], stream_rows));
     if (tm) SKY_TRY(tm->mark("stream", stream_edges));
   }
   const uint32_t tiled_rows = counts[CLS_HUGE] + (stream_to_tiled ? stream_rows : 0);
@@ -1115,16 +1113,6 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
                          tiled_list, cnt, max_tiles, sc.huge_off, g->xadj, g->adjwgt, sc.huge_scratch,
                          g->table, g->valid);
       if (tm) SKY_TRY(tm->mark("streamed", 0));
-    }
-  }
-  if (deferred) {  // rows the streaming kernel left alone (more heavies than its LDS list holds); asked last,
-                   // so that the host round trip does not idle the GPU between two classes
-    uint32_t nd = 0, skipped = 0;
-    SKY_TRY(stream_deferred_count(g, &nd));
-    if (nd) {
-      SKY_TRY(build_rows_tiled(g, deferred, nd, &skipped, nullptr, 0));
-      if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles is too small for rows of up to 65533 entries");
-      if (tm) SKY_TRY(tm->mark("stream_deferred", 0));
     }
   }
   return SKY_OK;

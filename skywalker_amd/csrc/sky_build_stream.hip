@@ -1,20 +1,22 @@
-// Alias tables of rows of 8190..65533 entries: one workgroup streams the row three times and
-// keeps the row's heavies in LDS.
+// Alias tables of rows of 8190..65533 entries: one workgroup streams the row and keeps a window of
+// the row's heavies in LDS.
 //
 // The table is the same pure function of the weights as everywhere else (see sky_build.hip).
 // Only the heavies of a row need random access: a light's alias is the first heavy whose surplus
 // prefix exceeds the light's exclusive deficit prefix, and a heavy's residual probability belongs
 // to the one light whose deficit interval (SL - D, SL] contains the heavy's surplus prefix.  So
-//   pass A  exact sum of the weights -> ledger
-//   pass B  classify, running surplus prefix; heavies compacted into LDS in slot order:
-//           {surplus prefix, slot}, 10 bytes each
-//   pass C  classify again, running deficit prefix; every light searches the heavy list once
-//           (alias) and finishes the heavies whose prefix falls into its interval (usually none,
-//           sometimes one); every heavy takes the next heavy of the list as alias, or {1, itself}
-//           when it is the last heavy or no light reaches it.
-// A heavy's probability and alias are separate 4-byte stores by different threads of the workgroup.
-// The second and third pass read the weights from L2.  Rows with more heavies than the LDS list
-// holds are appended to `deferred` and left untouched (the tile-parallel path builds them).
+//   pass A   exact sum of the weights -> ledger
+//   collect  the next ST_CAP heavies in slot order into LDS, {surplus prefix, slot}, 10 bytes each,
+//            and the slot of the heavy after them, if there is one; each takes the next heavy as
+//            alias, the row's last heavy keeps {1, itself}
+//   emit     classify every entry, running deficit prefix; a light whose alias lies in the window
+//            gets its entry, and every light finishes the window's heavies that fall into its
+//            deficit interval (usually none, sometimes one)
+// Rows with more heavies than one window holds repeat collect and emit: both move through the row
+// in slot order and only come back to the chunk in which the previous window ended, because the
+// alias ranks of the lights and the slots of the heavies both grow along the row.  Heavies no light
+// reaches keep {1, itself}.  A heavy's probability and alias are separate 4-byte stores by
+// different threads of the workgroup.  After the first pass the weights come from L2.
 #include "sky_build_common.h"
 #include "sky_graph.h"
 
@@ -126,17 +128,23 @@ __device__ __forceinline__ void count_le(const uint64_t* a, uint32_t n, const ui
   for (int m = 0; m < M; ++m) out[m] = cur[m] + (v[m] <= key[m] ? 1u : 0u);
 }
 
-__global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __restrict__ vlist,
+// Values that every lane holds alike, moved to scalar registers (the compiler cannot see that sums read
+// back from LDS are the same in every lane).
+__device__ __forceinline__ uint32_t uniform_u32(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ uint64_t uniform_u64(uint64_t x) {
+  return ((uint64_t)uniform_u32((uint32_t)(x >> 32)) << 32) | uniform_u32((uint32_t)x);
+}
+
+__global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __restrict__ vlist,
                                                             const float* __restrict__ wgt,
                                                             AliasEntry* __restrict__ table,
-                                                            int8_t* __restrict__ valid,
-                                                            RowRef* __restrict__ deferred,
-                                                            uint32_t* __restrict__ n_deferred) {
-  __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the row's h-th heavy
-  __shared__ uint16_t s_slot[ST_CAP + 1];  // its span slot
+                                                            int8_t* __restrict__ valid) {
+  __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the window's h-th heavy, then a sentinel
+  __shared__ uint16_t s_slot[ST_CAP + 1];  // its span slot; after them the slot lights beyond the window take
   __shared__ WSum3 s_w[ST_NW];
   __shared__ uint64_t s_a[2][ST_NW];  // two sets of wavefront sums, used alternately
   __shared__ uint32_t s_c[2][ST_NW];
+  __shared__ uint32_t s_next;  // slot of the first heavy after the window
   const RowRef rr = vlist[blockIdx.x];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   StreamRow r;
@@ -157,7 +165,6 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
 #pragma unroll
     for (int j = 0; j < ST_PER; ++j) wsum3_add(sum, wd[j]);
   }
-  nx = fetch_chunk(wgt, r, 0, tid);
   sum = group_sum_wsum3<64>(sum);
   if (lane == 0) s_w[wave] = sum;
   __syncthreads();
@@ -180,11 +187,11 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
   }
   const Ledger L = make_ledger_small(rr.d, wsum3_to_double(sum));
 
-  // ---- pass B: the heavies, in slot order.  Whether an entry is heavy is a monotone function of its
-  // clamped weight (p = fl(w * scale) and t = fma(p, 2^F, -2^F) are monotone, heavy iff t >= 0.5), so one
-  // compare against the smallest heavy weight of this row decides it; the surplus is then computed for the
-  // heavies alone, from the compacted list.
+  // Whether an entry is heavy is a monotone function of its clamped weight (p = fl(w * scale) and
+  // t = fma(p, 2^F, -2^F) are monotone, heavy iff t >= 0.5), so one compare against the smallest heavy weight
+  // of this row decides it; the surplus is then computed for the heavies alone, from the compacted list.
   uint32_t thr_bits;  // bit pattern of the smallest clamped weight that is heavy (above 2^32: none is)
+  bool thr_ok;        // false: the boundary was not found where it must be; every entry is classified in full
   {
     auto is_heavy = [&](uint32_t bits) {
       const double p = (double)__uint_as_float(bits) * L.scale;
@@ -202,202 +209,204 @@ __global__ __launch_bounds__(ST_T) void build_stream_kernel(const RowRef* __rest
       ++bits;
       ++guard;
     }
-    if (guard >= 64) {  // the estimate is within a step or two of the boundary; anything else: leave the row
-      if (tid == 0) deferred[atomicAdd(n_deferred, 1u)] = rr;
-      return;
-    }
+    thr_ok = guard < 64;  // the estimate is within a step or two of the boundary
     thr_bits = bits;
   }
   float* s_w32 = reinterpret_cast<float*>(s_sh);  // weight of heavy h in the low half of s_sh[h], until its prefix replaces it
-  uint32_t carry_c = 0;
-  bool overflow = false;
-  for (uint32_t c = 0; c < nch; ++c) {
-    const RawChunk cur = nx;
-    if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
-    float cw[ST_PER];
-    uint32_t heavy = 0;
-    if (wave_in_row(r, c, wave))
-#pragma unroll
-    for (int q = 0; q < ST_PER / 4; ++q) {
-      const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
-      const float xs[4] = {cur.q[q].x, cur.q[q].y, cur.q[q].z, cur.q[q].w};
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const uint32_t idx = pos + k;
-        cw[q * 4 + k] = clamp_weight(xs[k]);
-        if (idx >= r.lead && idx < r.span && __float_as_uint(cw[q * 4 + k]) >= thr_bits) heavy |= 1u << (q * 4 + k);
-      }
-    }
-    uint64_t ex_u, tot_u;
-    uint32_t ex_c, tot_c;
-    stream_excl(0ull, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_u, ex_c, tot_u, tot_c);
-    if (carry_c + tot_c > ST_CAP) {  // uniform
-      overflow = true;
-      break;
-    }
-    uint32_t rank = carry_c + ex_c;
-#pragma unroll
-    for (int j = 0; j < ST_PER; ++j)
-      if ((heavy >> j) & 1) {
-        s_w32[2 * rank] = cw[j];
-        s_slot[rank] = (uint16_t)(c * ST_CH + (uint32_t)ST_PER * tid + j);
-        ++rank;
-      }
-    carry_c += tot_c;
-  }
-  if (overflow) {
-    if (tid == 0) deferred[atomicAdd(n_deferred, 1u)] = rr;
-    return;
-  }
-  __syncthreads();  // the heavy list is complete
-  const uint32_t nh = carry_c;
-  {
-    // surplus prefix of the list: 16 consecutive heavies per thread
-    constexpr int HP = 16;
-    static_assert(ST_CAP < (uint32_t)ST_T * HP, "one round covers the list");
-    uint64_t u[HP];
-    uint64_t su = 0;
-#pragma unroll
-    for (int k = 0; k < HP; ++k) {
-      const uint32_t h = (uint32_t)HP * tid + k;
-      if (h < nh) su += classify_fast((double)s_w32[2 * h], true, L).amount;
-      u[k] = su;
-    }
-    uint64_t ex_u, tot_u;
-    uint32_t ex_c, tot_c;
-    stream_excl(su, 0u, s_a[0], s_c[0], ex_u, ex_c, tot_u, tot_c);
-#pragma unroll
-    for (int k = 0; k < HP; ++k) {
-      const uint32_t h = (uint32_t)HP * tid + k;
-      if (h < nh) s_sh[h] = ex_u + u[k];
-    }
-  }
-  __syncthreads();
-  if (tid == 0) {  // sentinel after the list; the first barrier of pass C publishes it
-    s_sh[nh] = ~0ull;
-    s_slot[nh] = nh ? s_slot[nh - 1] : (uint16_t)0;
-  }
 
-  // ---- pass C: every entry
-  uint64_t carry_d = 0;  // deficits so far; the row's total deficit after the last chunk
-  carry_c = 0;
-  nx = fetch_chunk(wgt, r, 0, tid);
-  for (uint32_t c = 0; c < nch; ++c) {
-    const RawChunk cur = nx;
-    if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
-    const bool on = wave_in_row(r, c, wave);  // a wavefront past the row's end only takes part in the scan
-    uint32_t live = 0;
-    float op[ST_PER];
-    uint64_t dl[ST_PER];
-    uint32_t heavy = 0;
-    uint64_t run = 0;
-    if (on) {
-      double wd[ST_PER];
-      live = unpack_chunk(cur, r, c, tid, wd);
+  // window state: collecting resumes at chunk cb (cnt_cb heavies lie before it), emitting at chunk cc
+  // (def_cc deficits lie before it)
+  uint32_t hb = 0;     // rank of the window's first heavy
+  uint64_t sh_lo = 0;  // surplus prefix of the heavies before the window
+  uint32_t cb = 0, cnt_cb = 0, cc = 0;
+  uint64_t def_cc = 0;
+  for (;;) {
+    // ---- collect: heavies of ranks [hb, hb + ST_CAP) and the slot of rank hb + ST_CAP
+    bool more = false;
+    uint32_t cnt = cnt_cb, next_cb = nch, next_cnt_cb = 0;
+    nx = fetch_chunk(wgt, r, cb, tid);
+    for (uint32_t c = cb; c < nch; ++c) {
+      const RawChunk cur = nx;
+      if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
+      float cw[ST_PER];
+      uint32_t heavy = 0;
+      if (wave_in_row(r, c, wave))
 #pragma unroll
-      for (int j = 0; j < ST_PER; ++j) {
-        const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
-        op[j] = (float)e.p;
-        dl[j] = e.heavy ? 0 : e.amount;
-        run += dl[j];
-        if (e.heavy) heavy |= 1u << j;
-      }
-    }
-    uint64_t ex_d, tot_d;
-    uint32_t ex_c, tot_c;
-    stream_excl(run, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
-    if (!on) {
-      carry_d += tot_d;
-      carry_c += tot_c;
-      continue;
-    }
-    // b = heavies whose surplus prefix is <= the deficits before this thread's slots: one search; from
-    // there the thread's lights walk the list, each stopping at its own deficit prefix
-    uint64_t sl = carry_d + ex_d;
-    uint32_t b = 0;
-    if (nh) {
-      const uint64_t k1[1] = {sl};
-      uint32_t o1[1];
-      count_le<1>(s_sh, nh, k1, o1);
-      b = o1[0];
-    }
-    uint64_t hv = s_sh[b];          // ~0 once the list is exhausted
-    uint32_t hslot = s_slot[b];     // then: the last heavy
-    const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
+        for (int q = 0; q < ST_PER / 4; ++q) {
+          const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
+          const float xs[4] = {cur.q[q].x, cur.q[q].y, cur.q[q].z, cur.q[q].w};
 #pragma unroll
-    for (int j = 0; j < ST_PER; ++j) {
-      if (!((live >> j) & 1)) continue;
-      const uint32_t idx = pos0 + j;
-      if ((heavy >> j) & 1) {
-        const uint32_t hr = carry_c + ex_c + (uint32_t)__popc(heavy & ((1u << j) - 1));
-        if (hr + 1 >= nh) {
-          table[r.base + idx] = AliasEntry{1.0f, idx - r.lead};
-        } else {
-          table[r.base + idx].alias = (uint32_t)s_slot[hr + 1] - r.lead;
+          for (int k = 0; k < 4; ++k) {
+            const uint32_t idx = pos + k;
+            cw[q * 4 + k] = clamp_weight(xs[k]);
+            const bool hv = thr_ok ? __float_as_uint(cw[q * 4 + k]) >= thr_bits
+                                   : classify_fast((double)cw[q * 4 + k], true, L).heavy;
+            if (idx >= r.lead && idx < r.span && hv) heavy |= 1u << (q * 4 + k);
+          }
         }
-      } else {
-        table[r.base + idx] = AliasEntry{op[j], (nh ? hslot : idx) - r.lead};
-        // heavies whose surplus prefix lies in (sl, sl + D]: this light finishes them
-        sl += dl[j];
-        while (hv <= sl) {
-          if (b + 1 < nh) table[r.base + hslot].prob = residual_prob(L.one + hv - sl, L);
-          ++b;
-          hv = s_sh[b];
-          hslot = s_slot[b];
+      uint64_t ex_u, tot_u;
+      uint32_t ex_c, tot_c;
+      stream_excl(0ull, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_u, ex_c, tot_u, tot_c);
+      uint32_t rank = cnt + ex_c;
+#pragma unroll
+      for (int j = 0; j < ST_PER; ++j)
+        if ((heavy >> j) & 1) {
+          const uint32_t slot = c * ST_CH + (uint32_t)ST_PER * tid + j;
+          if (rank >= hb && rank < hb + ST_CAP) {
+            s_w32[2 * (rank - hb)] = cw[j];
+            s_slot[rank - hb] = (uint16_t)slot;
+          } else if (rank == hb + ST_CAP) {
+            s_next = slot;
+          }
+          ++rank;
         }
+      tot_c = uniform_u32(tot_c);
+      if (cnt + tot_c > hb + ST_CAP) {  // uniform: the window is full and another heavy follows in this chunk
+        more = true;
+        next_cb = c;
+        next_cnt_cb = cnt;
+        break;
       }
+      cnt += tot_c;
     }
-    carry_d += tot_d;
-    carry_c += tot_c;
-  }
-  // heavies no light has reached (surplus prefix beyond the row's total deficit) keep their bucket
-  __syncthreads();
-  for (uint32_t h = tid; h + 1 < nh; h += ST_T)
-    if (s_sh[h] > carry_d) {
+    const uint32_t nw = more ? ST_CAP : cnt - hb;
+    __syncthreads();  // the window's weights and slots, and s_next, are complete
+    const uint32_t next_slot = more ? uniform_u32(s_next) : NONE32;
+    uint64_t sh_hi;  // surplus prefix of the window's last heavy
+    {
+      // surplus prefix of the window: 16 consecutive heavies per thread
+      constexpr int HP = 16;
+      static_assert(ST_CAP < (uint32_t)ST_T * HP, "one round covers the window");
+      uint64_t u[HP];
+      uint64_t su = 0;
+#pragma unroll
+      for (int k = 0; k < HP; ++k) {
+        const uint32_t h = (uint32_t)HP * tid + k;
+        if (h < nw) su += classify_fast((double)s_w32[2 * h], true, L).amount;
+        u[k] = su;
+      }
+      uint64_t ex_u, tot_u;
+      uint32_t ex_c, tot_c;
+      stream_excl(su, 0u, s_a[0], s_c[0], ex_u, ex_c, tot_u, tot_c);
+#pragma unroll
+      for (int k = 0; k < HP; ++k) {
+        const uint32_t h = (uint32_t)HP * tid + k;
+        if (h < nw) s_sh[h] = sh_lo + ex_u + u[k];
+      }
+      sh_hi = sh_lo + uniform_u64(tot_u);
+    }
+    // every heavy takes the next heavy as alias; the row's last heavy keeps its bucket
+    for (uint32_t h = tid; h < nw; h += ST_T) {
       const uint32_t slot = s_slot[h];
-      table[r.base + slot] = AliasEntry{1.0f, slot - r.lead};
+      const uint32_t nxt = h + 1 < nw ? (uint32_t)s_slot[h + 1] : next_slot;
+      if (nxt != NONE32) {
+        table[r.base + slot].alias = nxt - r.lead;
+      } else {
+        table[r.base + slot] = AliasEntry{1.0f, slot - r.lead};
+      }
     }
-}
+    if (tid == 0) {  // after the list: a sentinel, and the slot that lights beyond the window's last heavy take
+      s_sh[nw] = ~0ull;
+      s_slot[nw] = more ? (uint16_t)next_slot : (nw ? s_slot[nw - 1] : (uint16_t)0);
+    }
+    const bool any_heavy = hb + nw != 0;
+    const bool whole_row = hb == 0 && !more;  // the usual case: one window holds every heavy of the row
+    __syncthreads();
 
-namespace {
-struct StreamScratch {
-  RowRef* deferred = nullptr;
-  uint32_t* n_deferred = nullptr;
-  uint32_t cap = 0;
-};
-StreamScratch g_stream;
-}  // namespace
-
-// Builds the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each).  Rows whose heavies do not fit the
-// LDS list are returned in *deferred (device array owned by this file, valid until the next call).
-int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n, const RowRef** deferred,
-                      uint32_t* n_deferred) {
-  StreamScratch& sc = g_stream;
-  *deferred = nullptr;
-  *n_deferred = 0;
-  if (n == 0) return SKY_OK;
-  hipStream_t st = g->stream;
-  if (sc.cap < n) {
-    if (sc.deferred) SKY_HIP(hipFree(sc.deferred));
-    sc.deferred = nullptr;
-    sc.cap = 0;
-    SKY_HIP(hipMalloc((void**)&sc.deferred, (size_t)n * sizeof(RowRef)));
-    sc.cap = n;
+    // ---- emit: chunks from cc on, until the deficits before a chunk reach the window's last surplus prefix
+    uint64_t carry_d = def_cc;
+    uint32_t last_c = cc;        // the last chunk worked on, where the next window starts again
+    uint64_t last_def = def_cc;  // deficits before it
+    bool reached_end = true;
+    nx = fetch_chunk(wgt, r, cc, tid);
+    for (uint32_t c = cc; c < nch; ++c) {
+      if (more && carry_d >= sh_hi) {  // uniform: the lights from here on belong to later windows
+        reached_end = false;
+        break;
+      }
+      last_c = c;
+      last_def = carry_d;
+      const RawChunk cur = nx;
+      if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
+      const bool on = wave_in_row(r, c, wave);  // a wavefront past the row's end only takes part in the scan
+      uint32_t live = 0;
+      float op[ST_PER];
+      uint64_t dl[ST_PER];
+      uint32_t heavy = 0;
+      uint64_t run = 0;
+      if (on) {
+        double wd[ST_PER];
+        live = unpack_chunk(cur, r, c, tid, wd);
+#pragma unroll
+        for (int j = 0; j < ST_PER; ++j) {
+          const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
+          op[j] = (float)e.p;
+          dl[j] = e.heavy ? 0 : e.amount;
+          run += dl[j];
+          if (e.heavy) heavy |= 1u << j;
+        }
+      }
+      uint64_t ex_d, tot_d;
+      uint32_t ex_c, tot_c;
+      stream_excl(run, 0u, s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
+      if (on) {
+        // b = window heavies whose surplus prefix is <= the deficits before this thread's slots: one search;
+        // from there the thread's lights walk the list, each stopping at its own deficit prefix
+        uint64_t sl = carry_d + ex_d;
+        uint32_t b = 0;
+        if (nw) {
+          const uint64_t k1[1] = {sl};
+          uint32_t o1[1];
+          count_le<1>(s_sh, nw, k1, o1);
+          b = o1[0];
+        }
+        uint64_t hv = s_sh[b];       // ~0 once the window is exhausted
+        uint32_t hslot = s_slot[b];  // then: the first heavy after the window, or the row's last heavy
+        const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
+#pragma unroll
+        for (int j = 0; j < ST_PER; ++j) {
+          if (!((live >> j) & 1) || ((heavy >> j) & 1)) continue;
+          const uint32_t idx = pos0 + j;
+          // the light's alias is the first heavy whose surplus prefix exceeds sl: in this window iff
+          // sh_lo <= sl < sh_hi, or beyond every heavy of the row
+          if (whole_row || (sl >= sh_lo && (sl < sh_hi || !more)))
+            table[r.base + idx] = AliasEntry{op[j], (any_heavy ? hslot : idx) - r.lead};
+          // heavies of the window whose surplus prefix lies in (sl, sl + D]: this light finishes them
+          sl += dl[j];
+          while (hv <= sl) {
+            if (b + 1 < nw || more) table[r.base + hslot].prob = residual_prob(L.one + hv - sl, L);
+            ++b;
+            hv = s_sh[b];
+            hslot = s_slot[b];
+          }
+        }
+      }
+      carry_d += uniform_u64(tot_d);
+    }
+    if (reached_end) {  // carry_d is the row's total deficit: heavies beyond it are reached by no light
+      __syncthreads();
+      for (uint32_t h = tid; h < nw; h += ST_T)
+        if (s_sh[h] > carry_d && (h + 1 < nw || more)) {
+          const uint32_t slot = s_slot[h];
+          table[r.base + slot] = AliasEntry{1.0f, slot - r.lead};
+        }
+    }
+    if (!more) break;
+    hb += nw;
+    sh_lo = sh_hi;
+    cb = next_cb;
+    cnt_cb = next_cnt_cb;
+    cc = last_c;
+    def_cc = last_def;
+    __syncthreads();  // the lists are rewritten by the next window
   }
-  if (!sc.n_deferred) SKY_HIP(hipMalloc((void**)&sc.n_deferred, 4));
-  SKY_HIP(hipMemsetAsync(sc.n_deferred, 0, 4, st));
-  hipLaunchKernelGGL(build_stream_kernel, dim3(n), dim3(ST_T), 0, st, rows_list, g->adjwgt, g->table, g->valid,
-                     sc.deferred, sc.n_deferred);
-  *deferred = sc.deferred;
-  return SKY_OK;
 }
 
-// Number of rows the last build_rows_stream call deferred (synchronises the stream).
-int stream_deferred_count(sky_graph* g, uint32_t* n_deferred) {
-  *n_deferred = 0;
-  if (!g_stream.n_deferred) return SKY_OK;
-  SKY_HIP(hipMemcpyAsync(n_deferred, g_stream.n_deferred, 4, hipMemcpyDeviceToHost, g->stream));
-  SKY_HIP(hipStreamSynchronize(g->stream));
+// Builds the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each).
+int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n) {
+  if (n == 0) return SKY_OK;
+  hipLaunchKernelGGL(build_stream_kernel, dim3(n), dim3(ST_T), 0, g->stream, rows_list, g->adjwgt, g->table,
+                     g->valid);
   return SKY_OK;
 }
 

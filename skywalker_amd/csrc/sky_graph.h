@@ -77,9 +77,7 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
                      uint64_t edges);
 void set_tiled_max_tiles(uint32_t n);
 constexpr uint32_t STREAM_MAX_DEG = 65533;  // longest row of the streaming class
-int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n, const RowRef** deferred,
-                      uint32_t* n_deferred);
-int stream_deferred_count(sky_graph* g, uint32_t* n_deferred);
+int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n);
 void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);
 void set_build_profile(bool on);

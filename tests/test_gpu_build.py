@@ -157,8 +157,8 @@ def test_search_variant_of_the_row_kernels_gives_the_same_table(orc):
 
 @pytest.mark.parametrize("dist", ["lognormal2", "uniform", "nearequal", "sparse", "fewlights", "fewheavies"])
 def test_rows_streamed_by_one_workgroup(orc, dist):
-    # rows of 8190..65533 entries: heavies kept in LDS ("fewlights" has more heavies than fit: those rows are
-    # handed to the tile-parallel path); 65534 is the first degree of the tile-parallel class
+    # rows of 8190..65533 entries: a window of 8063 heavies kept in LDS ("fewlights" and "uniform" have rows with
+    # up to eight windows, "nearequal" rows without a heavy); 65534 is the first degree of the tile-parallel class
     from helpers import weights
     rng = np.random.default_rng(31)
     degs = [8190, 8191, 7, 8193, 12288, 2, 12289, 16385, 1, 30000, 65533, 65534, 0, 9001]
