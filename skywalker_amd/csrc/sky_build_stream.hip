@@ -277,21 +277,24 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       // surplus prefix of the window: 16 consecutive heavies per thread
       constexpr int HP = 16;
       static_assert(ST_CAP < (uint32_t)ST_T * HP, "one round covers the window");
-      uint64_t u[HP];
+      // (the amounts are computed twice rather than kept: 32 registers less at the kernel's widest point)
       uint64_t su = 0;
 #pragma unroll
       for (int k = 0; k < HP; ++k) {
         const uint32_t h = (uint32_t)HP * tid + k;
         if (h < nw) su += classify_fast((double)s_w32[2 * h], true, L).amount;
-        u[k] = su;
       }
       uint64_t ex_u, tot_u;
       uint32_t ex_c, tot_c;
       stream_excl(su, 0u, s_a[0], s_c[0], ex_u, ex_c, tot_u, tot_c);
+      uint64_t acc = sh_lo + ex_u;
 #pragma unroll
       for (int k = 0; k < HP; ++k) {
         const uint32_t h = (uint32_t)HP * tid + k;
-        if (h < nw) s_sh[h] = sh_lo + ex_u + u[k];
+        if (h < nw) {
+          acc += classify_fast((double)s_w32[2 * h], true, L).amount;  // read before s_sh[h] takes its place
+          s_sh[h] = acc;
+        }
       }
       sh_hi = sh_lo + uniform_u64(tot_u);
     }
