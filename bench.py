@@ -33,7 +33,7 @@ CONFIGS = {
 BYTES_PER_EDGE = {"tiled_sum": 4, "tiled_totals": 4, "bin": 12}
 # HBM bytes per edge measured with rocprofv3 --pmc FETCH_SIZE (x2.0, calibrated on copy_u32_kernel) and WRITE_SIZE
 # (x1.0); see profiles/c5_build_traffic.md
-TRAFFIC_PER_EDGE = {"stream": 24.4, "mw10": 12.1, "mw9": 12.1, "mw4": 12.2, "mw3": 12.2, "mw2": 12.6, "lds_w2": 12.6,
+TRAFFIC_PER_EDGE = {"stream": 19.2, "mw10": 12.1, "mw9": 12.1, "mw4": 12.2, "mw3": 12.2, "mw2": 12.6, "lds_w2": 12.6,
                     "lds_w1": 14.6, "g32x": 13.0, "g32": 13.8, "g16": 14.8, "g8": 19.2, "g4": 24.1, "g2": 34.5,
                     "tiled_emit": 24.4, "tiled_sum": 4.3, "tiled_totals": 4.3}
 WALK_TRAFFIC_PER_STEP = 398.5  # walk_offline_kernel, same source

@@ -298,8 +298,12 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       }
       sh_hi = sh_lo + uniform_u64(tot_u);
     }
-    // every heavy takes the next heavy as alias; the row's last heavy keeps its bucket
-    for (uint32_t h = tid; h < nw; h += ST_T) {
+    const bool any_heavy = hb + nw != 0;
+    const bool whole_row = hb == 0 && !more;  // the usual case: one window holds every heavy of the row
+    // every heavy takes the next heavy as alias; the row's last heavy keeps its bucket.  When the window holds
+    // the whole row the emit pass meets every heavy and writes this beside the entries of its neighbours
+    // (a store of its own here costs a second write of the line); otherwise it is written from the list.
+    for (uint32_t h = tid; h < nw && !whole_row; h += ST_T) {
       const uint32_t slot = s_slot[h];
       const uint32_t nxt = h + 1 < nw ? (uint32_t)s_slot[h + 1] : next_slot;
       if (nxt != NONE32) {
@@ -312,12 +316,11 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       s_sh[nw] = ~0ull;
       s_slot[nw] = more ? (uint16_t)next_slot : (nw ? s_slot[nw - 1] : (uint16_t)0);
     }
-    const bool any_heavy = hb + nw != 0;
-    const bool whole_row = hb == 0 && !more;  // the usual case: one window holds every heavy of the row
     __syncthreads();
 
     // ---- emit: chunks from cc on, until the deficits before a chunk reach the window's last surplus prefix
     uint64_t carry_d = def_cc;
+    uint32_t carry_c = 0;        // heavies before the chunk (kept for whole_row only, where cc = 0)
     uint32_t last_c = cc;        // the last chunk worked on, where the next window starts again
     uint64_t last_def = def_cc;  // deficits before it
     bool reached_end = true;
@@ -351,7 +354,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       }
       uint64_t ex_d, tot_d;
       uint32_t ex_c, tot_c;
-      stream_excl(run, 0u, s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
+      stream_excl(run, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
       if (on) {
         // b = window heavies whose surplus prefix is <= the deficits before this thread's slots: one search;
         // from there the thread's lights walk the list, each stopping at its own deficit prefix
@@ -368,8 +371,19 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
         const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
-          if (!((live >> j) & 1) || ((heavy >> j) & 1)) continue;
+          if (!((live >> j) & 1)) continue;
           const uint32_t idx = pos0 + j;
+          if ((heavy >> j) & 1) {
+            if (whole_row) {
+              const uint32_t hr = carry_c + ex_c + (uint32_t)__popc(heavy & ((1u << j) - 1));
+              if (hr + 1 < nw) {
+                table[r.base + idx].alias = (uint32_t)s_slot[hr + 1] - r.lead;
+              } else {
+                table[r.base + idx] = AliasEntry{1.0f, idx - r.lead};
+              }
+            }
+            continue;
+          }
           // the light's alias is the first heavy whose surplus prefix exceeds sl: in this window iff
           // sh_lo <= sl < sh_hi, or beyond every heavy of the row
           if (whole_row || (sl >= sh_lo && (sl < sh_hi || !more)))
@@ -385,6 +399,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
         }
       }
       carry_d += uniform_u64(tot_d);
+      carry_c += uniform_u32(tot_c);
     }
     if (reached_end) {  // carry_d is the row's total deficit: heavies beyond it are reached by no light
       __syncthreads();
