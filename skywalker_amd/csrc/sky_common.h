@@ -70,8 +70,8 @@ __device__ __forceinline__ u128 add128(u128 a, u128 b) {
   return r;
 }
 __device__ __forceinline__ float clamp_weight(float w) {
-  if (!(w > 0.0f)) return 0.0f;  // zero, negatives, NaN
-  return w > 4294967296.0f ? 4294967296.0f : w;
+  // zero, negatives and NaN give +0 (the maximum of a NaN and a number is the number), values above 2^32 give 2^32
+  return fminf(fmaxf(w, 0.0f), 4294967296.0f);
 }
 // floor(w * 2^64) of a clamped weight.
 __device__ __forceinline__ u128 weight_fixed(float w) {
