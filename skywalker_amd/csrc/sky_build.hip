@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
     const uint32_t idx = pos + k;
-    const bool in = idx >= lead && idx < span;
+    const bool in = idx - lead < d;  // one unsigned compare: slots before the row wrap around
     if (in) live |= 1u << k;
     wd[k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
     wsum3_add(S, wd[k]);
@@ -362,7 +362,7 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const RowRef* __restric
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const uint32_t idx = pos + k;
-      const bool in = idx >= lead && idx < span;
+      const bool in = idx - lead < d;  // one unsigned compare: slots before the row wrap around
       if (in) live |= 1u << (t * 4 + k);
       w[t][k] = in ? clamp_weight(xs[k]) : 0.0f;
       sum = add128(sum, weight_fixed(w[t][k]));
@@ -580,7 +580,7 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
 #pragma unroll
       for (int k = 0; k < VEC; ++k) {
         const uint32_t idx = pos + k;
-        const bool in = idx >= lead && idx < span;
+        const bool in = idx - lead < d;  // one unsigned compare: slots before the row wrap around
         if (in) live |= 1u << (t * VEC + k);
         wd[t * VEC + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
         wsum3_add(sum, wd[t * VEC + k]);

@@ -64,7 +64,7 @@ __device__ __forceinline__ uint32_t unpack_chunk(const RawChunk& x, const Stream
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const uint32_t idx = pos + k;
-      const bool in = idx >= r.lead && idx < r.span;
+      const bool in = idx - r.lead < r.span - r.lead;
       if (in) live |= 1u << (q * 4 + k);
       wd[q * 4 + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
     }
@@ -241,7 +241,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
             cw[q * 4 + k] = clamp_weight(xs[k]);
             const bool hv = thr_ok ? __float_as_uint(cw[q * 4 + k]) >= thr_bits
                                    : classify_fast((double)cw[q * 4 + k], true, L).heavy;
-            if (idx >= r.lead && idx < r.span && hv) heavy |= 1u << (q * 4 + k);
+            if (idx - r.lead < r.span - r.lead && hv) heavy |= 1u << (q * 4 + k);
           }
         }
       uint64_t ex_u, tot_u;

@@ -73,11 +73,11 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ wgt, const T
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const uint32_t idx = pos + k;
-      w[q][k] = (idx >= r.lead && idx < r.span) ? clamp_weight(xs[k]) : 0.0f;
+      w[q][k] = idx - r.lead < r.span - r.lead ? clamp_weight(xs[k]) : 0.0f;
     }
   }
 }
-__device__ __forceinline__ bool in_row(const TiledRow& r, uint32_t idx) { return idx >= r.lead && idx < r.span; }
+__device__ __forceinline__ bool in_row(const TiledRow& r, uint32_t idx) { return idx - r.lead < r.span - r.lead; }
 
 // ---------------------------------------------------------------- row and tile bookkeeping
 struct TiledCounters {
