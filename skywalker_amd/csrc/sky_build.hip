@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
     const uint32_t idx = pos + k;
     const bool in = idx - lead < d;  // one unsigned compare: slots before the row wrap around
     if (in) live |= 1u << k;
-    wd[k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
+    wd[k] = (double)masked_weight(xs[k], in);
     wsum3_add(S, wd[k]);
   }
   S = group_sum_wsum3<G>(S);
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
         const uint32_t idx = pos + k;
         const bool in = idx - lead < d;  // one unsigned compare: slots before the row wrap around
         if (in) live |= 1u << (t * VEC + k);
-        wd[t * VEC + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
+        wd[t * VEC + k] = (double)masked_weight(xs[k], in);
         wsum3_add(sum, wd[t * VEC + k]);
       }
     }

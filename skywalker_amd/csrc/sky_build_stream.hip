@@ -66,7 +66,7 @@ __device__ __forceinline__ uint32_t unpack_chunk(const RawChunk& x, const Stream
       const uint32_t idx = pos + k;
       const bool in = idx - r.lead < r.span - r.lead;
       if (in) live |= 1u << (q * 4 + k);
-      wd[q * 4 + k] = (double)(in ? clamp_weight(xs[k]) : 0.0f);
+      wd[q * 4 + k] = (double)masked_weight(xs[k], in);
     }
   }
   return live;

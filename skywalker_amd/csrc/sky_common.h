@@ -70,8 +70,14 @@ __device__ __forceinline__ u128 add128(u128 a, u128 b) {
   return r;
 }
 __device__ __forceinline__ float clamp_weight(float w) {
-  // zero, negatives and NaN give +0 (the maximum of a NaN and a number is the number), values above 2^32 give 2^32
-  return fminf(fmaxf(w, 0.0f), 4294967296.0f);
+  // median of (w, 0, 2^32): zero, negatives and NaN give +0 (a NaN operand makes the instruction return the
+  // smallest of the other two), values above 2^32 give 2^32
+  return __builtin_amdgcn_fmed3f(w, 0.0f, 4294967296.0f);
+}
+// The clamped weight of a slot of the row, +0 for a slot outside it: the upper bound carries the mask, which
+// costs one 32-bit select instead of two on the converted double.
+__device__ __forceinline__ float masked_weight(float w, bool in) {
+  return __builtin_amdgcn_fmed3f(w, 0.0f, in ? 4294967296.0f : 0.0f);
 }
 // floor(w * 2^64) of a clamped weight.
 __device__ __forceinline__ u128 weight_fixed(float w) {
