@@ -178,12 +178,14 @@ __device__ __forceinline__ Ledger make_ledger_small(uint32_t deg, double sum /* 
   return L;
 }
 // classify for rows of fewer than 2^12 entries (|t| < 2^52, F = 40): same values as classify, fewer
-// instructions.  `in` false gives a light of deficit 0.  fma(p, fs, -fs) == (p - 1) * fs because fs is a
-// power of two; max(t, 1) before rounding == max(rint(t), 1) for a heavy.
+// instructions.  `in` false gives a light of deficit 0.  max(t, 1) before rounding == max(rint(t), 1) for a
+// heavy.  (p - 1) * fs as written: the product with a power of two is exact, so one rounding as in classify;
+// a subtraction with an inline constant and a multiplication, where a fused form needs its addend moved
+// into the destination first.
 __device__ __forceinline__ Entry classify_small(double wd, bool in, const Ledger& L) {
   Entry e;
   e.p = in ? wd * L.scale : 1.0;
-  const double t = fma(e.p, L.fs, -L.fs);
+  const double t = (e.p - 1.0) * L.fs;
   e.heavy = t >= 0.5;
   const double a = fmax(e.heavy ? t : -t, e.heavy ? 1.0 : 0.0);
   e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) - 0x4330000000000000ull;
@@ -194,7 +196,7 @@ __device__ __forceinline__ Entry classify_small(double wd, bool in, const Ledger
 __device__ __forceinline__ Entry classify_fast(double wd, bool in, const Ledger& L) {
   Entry e;
   e.p = in ? wd * L.scale : 1.0;
-  const double t = fma(e.p, L.fs, -L.fs);
+  const double t = (e.p - 1.0) * L.fs;
   e.heavy = t >= 0.5;
   const double a = fmax(e.heavy ? t : -t, e.heavy ? 1.0 : 0.0);
   if (a < 4503599627370496.0)
@@ -271,8 +273,9 @@ __device__ __forceinline__ uint32_t dpp0(uint32_t v) {
 }
 template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ uint64_t dpp0_u64(uint64_t v) {
-  const uint32_t lo = dpp0<CTRL, ROW_MASK>((uint32_t)v), hi = dpp0<CTRL, ROW_MASK>((uint32_t)(v >> 32));
-  return ((uint64_t)hi << 32) | lo;
+  // the 64-bit form keeps the two moved halves a register pair, so that the addition that follows is one
+  // instruction (halves joined by shift and or end up as two additions)
+  return (uint64_t)__builtin_amdgcn_update_dpp((uint64_t)0, v, CTRL, ROW_MASK, 0xF, true);
 }
 constexpr int DPP_ROW_SHR1 = 0x111, DPP_ROW_SHR2 = 0x112, DPP_ROW_SHR4 = 0x114, DPP_ROW_SHR8 = 0x118;
 constexpr int DPP_ROW_BCAST15 = 0x142, DPP_ROW_BCAST31 = 0x143;
