@@ -236,8 +236,8 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
   uint64_t ra = 0, rb = 0;
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
-    const Entry e = classify_small(wd[k], (live >> k) & 1, L);
-    dl[k] = e.heavy ? 0 : e.amount;
+    const Entry e = classify_small_unmasked(wd[k], L);
+    dl[k] = (e.heavy || !((live >> k) & 1)) ? 0 : e.amount;
     ra += dl[k];
     rb += e.heavy ? (e.amount | GROUP_CNT) : 0;
     sl[k] = ra;
@@ -619,8 +619,9 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
     uint64_t dl[PER], dh[PER], sl[PER], sh[PER];
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const Entry e = PACKED ? classify_small(wd[j], (live >> j) & 1, L) : classify_fast(wd[j], (live >> j) & 1, L);
-      dl[j] = e.heavy ? 0 : e.amount;
+      const bool in = (live >> j) & 1;
+      const Entry e = PACKED ? classify_small_unmasked(wd[j], L) : classify_fast(wd[j], in, L);
+      dl[j] = (e.heavy || !in) ? 0 : e.amount;
       dh[j] = e.heavy ? (PACKED ? (e.amount | MERGE_CNT) : e.amount) : 0;
       op[j] = (float)e.p;
       if (e.heavy) heavy |= 1u << j;

@@ -191,6 +191,18 @@ __device__ __forceinline__ Entry classify_small(double wd, bool in, const Ledger
   e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) - 0x4330000000000000ull;
   return e;
 }
+// classify_small without the row mask: a slot outside the row arrives with weight +0 and comes out as a
+// light with a deficit of 2^F, which the caller drops (two selects on a double saved per entry; the
+// caller's own selects take the mask for free, as a scalar AND of lane masks).
+__device__ __forceinline__ Entry classify_small_unmasked(double wd, const Ledger& L) {
+  Entry e;
+  e.p = wd * L.scale;
+  const double t = (e.p - 1.0) * L.fs;
+  e.heavy = t >= 0.5;
+  const double a = fmax(e.heavy ? t : -t, e.heavy ? 1.0 : 0.0);
+  e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) - 0x4330000000000000ull;
+  return e;
+}
 // classify with fewer instructions for any row: same values.  The 2^52 rounding shortcut covers every
 // amount below 2^52; larger ones are integers already and take the (rare, branched) general conversion.
 __device__ __forceinline__ Entry classify_fast(double wd, bool in, const Ledger& L) {
