@@ -643,10 +643,7 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
       const uint32_t li = pos0 + j - lead;
       const bool hv = (heavy >> j) & 1;
       s_v[hv ? TOP + 1 - hc : li - hc] = hv ? (PACKED ? (sh[j] & (MERGE_CNT - 1)) : sh[j]) : sl[j];
-      if (hv) {
-        s_hs[hc - 1] = (uint16_t)li;
-        if (hc == 1) s_res[0] = li;  // the first light starts in the first heavy
-      }
+      if (hv) s_hs[hc - 1] = (uint16_t)li;
     }
   }
   if (tid == 0) {
@@ -656,6 +653,7 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
   __syncthreads();
 
   if (nh) {
+    if (tid == 0) s_res[0] = s_hs[0];  // the first light starts in the first heavy
     // merged positions [k0, k0 + PER) belong to this thread; a lights and k0 - a heavies come before them
     const uint32_t k0 = pos0;
     if (k0 < d) {
