@@ -187,7 +187,7 @@ __device__ __forceinline__ Entry classify_small(double wd, bool in, const Ledger
   e.p = in ? wd * L.scale : 1.0;
   const double t = (e.p - 1.0) * L.fs;
   e.heavy = t >= 0.5;
-  const double a = fmax(e.heavy ? t : -t, e.heavy ? 1.0 : 0.0);
+  const double a = fmax(fabs(t), e.heavy ? 1.0 : 0.0);  // |t| < 0.5 for a light with t > 0: rounds to the deficit 0
   e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) - 0x4330000000000000ull;
   return e;
 }
@@ -199,7 +199,7 @@ __device__ __forceinline__ Entry classify_small_unmasked(double wd, const Ledger
   e.p = wd * L.scale;
   const double t = (e.p - 1.0) * L.fs;
   e.heavy = t >= 0.5;
-  const double a = fmax(e.heavy ? t : -t, e.heavy ? 1.0 : 0.0);
+  const double a = fmax(fabs(t), e.heavy ? 1.0 : 0.0);  // |t| < 0.5 for a light with t > 0: rounds to the deficit 0
   e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) - 0x4330000000000000ull;
   return e;
 }
@@ -210,7 +210,7 @@ __device__ __forceinline__ Entry classify_fast(double wd, bool in, const Ledger&
   e.p = in ? wd * L.scale : 1.0;
   const double t = (e.p - 1.0) * L.fs;
   e.heavy = t >= 0.5;
-  const double a = fmax(e.heavy ? t : -t, e.heavy ? 1.0 : 0.0);
+  const double a = fmax(fabs(t), e.heavy ? 1.0 : 0.0);  // |t| < 0.5 for a light with t > 0: rounds to the deficit 0
   if (a < 4503599627370496.0)
     e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) - 0x4330000000000000ull;
   else
