@@ -664,16 +664,18 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
       }
       uint32_t a = lo, b = k0 - lo;
       const uint32_t steps = min((uint32_t)PER, d - k0);
+      uint64_t va = s_v[a], vb = s_v[TOP - b];  // heads of the two sequences: only the one taken is read again
 #pragma unroll
       for (int s = 0; s < PER; ++s) {
         if ((uint32_t)s < steps) {
-          const uint64_t va = s_v[a], vb = s_v[TOP - b];
           if (vb <= va) {
             s_res[TOP - b] = a;
             ++b;
+            vb = s_v[TOP - b];
           } else {
             ++a;
             if (a < nl) s_res[a] = s_hs[min(b, nh - 1)];
+            va = s_v[a];
           }
         }
       }
