@@ -118,6 +118,20 @@ int sky_walk_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uin
                      uint64_t philox_seed, uint32_t* paths_device, uint32_t* lengths_device, uint64_t* sampled,
                      double* seconds);
 
+/* ---- sky_walk_offline for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses
+ *      that forbid hipMalloc).  No counterpart in the reference.  Same kernel, same paths and lengths; the
+ *      per-workgroup counts of sampled edges go to a static device array of the library (128 KiB per GPU, held
+ *      until the process ends) instead of an allocated counter, and their sum is written by a second kernel to
+ *      sampled_device, a device word of the caller (may be NULL).  The call allocates nothing, creates no event,
+ *      copies nothing to the host and does not wait: the kernels are enqueued on the graph's stream (the null
+ *      stream) and the caller synchronises (sky_device_synchronize) before reading the outputs.  At most
+ *      4,194,304 walkers per call (SKY_ERR_LIMIT beyond).  Every call on a GPU shares that GPU's array, so calls
+ *      that overlap on one GPU race. ---- */
+#define SKY_WALK_NOALLOC_MAX_WALKERS 4194304u
+int sky_walk_offline_noalloc(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uint32_t len, float stop_prob,
+                             uint64_t philox_seed, uint32_t* paths_device, uint32_t* lengths_device,
+                             uint64_t* sampled_device);
+
 /* ---- walk that rebuilds the table of the current vertex at every step: replaces OnlineWalkShMem(Walker&) /
  *      OnlineWalkGMem(Walker&) (src/online_walk.cu:245-327, online_walk_gmem.cu); bias SKY_BIAS_NODE2VEC applies
  *      the second-order factors of src/api/bias_node2vec.cu:15-27 with (p, q); SKY_BIAS_NODE2VEC_REJECT reaches

@@ -22,6 +22,7 @@ EXPORTS = [
     "sky_device_fill_u32", "sky_device_copy_u32", "sky_device_synchronize", "sky_device_name", "sky_graph_upload",
     "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
     "sky_alias_build_all", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
+    "sky_walk_offline_noalloc",
     "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_philox_selftest",
     "sky_last_build_profile", "sky_set_option",
 ]
@@ -200,6 +201,12 @@ class Graph:
     def walk_offline(self, seeds, length, stop_prob, seed, out=None):
         """OfflineWalk: returns (paths DeviceArray, lengths DeviceArray, sampled, seconds)."""
         return self._walk(lib().sky_walk_offline, (), seeds, length, stop_prob, seed, out)
+
+    def walk_offline_noalloc(self, seeds_d, length, stop_prob, seed, paths, lengths, sampled_d):
+        """sky_walk_offline_noalloc: every buffer is the caller's; enqueues and returns (synchronize() before reading)."""
+        _ck(lib().sky_walk_offline_noalloc(self.h, seeds_d.ptr, C.c_uint32(seeds_d.count), C.c_uint32(length),
+                                           C.c_float(stop_prob), C.c_uint64(seed), paths.ptr, lengths.ptr,
+                                           sampled_d.ptr if sampled_d is not None else None))
 
     def walk_online(self, bias_kind, p, q, seeds, length, stop_prob, seed, out=None):
         """OnlineWalkShMem."""

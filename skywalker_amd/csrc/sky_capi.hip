@@ -248,6 +248,15 @@ int sky_walk_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uin
   return walk_offline(g, seeds_device, N, len, stop_prob, philox_seed, paths_device, lengths_device, sampled, seconds);
 }
 
+int sky_walk_offline_noalloc(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uint32_t len, float stop_prob,
+                             uint64_t philox_seed, uint32_t* paths_device, uint32_t* lengths_device,
+                             uint64_t* sampled_device) {
+  SKY_TRY(check_walk_args("sky_walk_offline_noalloc", g, seeds_device, N, len, stop_prob, paths_device, lengths_device));
+  if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_walk_offline_noalloc: alias tables have not been built");
+  return walk_offline_noalloc(g, seeds_device, N, len, stop_prob, philox_seed, paths_device, lengths_device,
+                              sampled_device);
+}
+
 int sky_walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds_device, uint32_t N,
                     uint32_t len, float stop_prob, uint64_t philox_seed, uint32_t* paths_device,
                     uint32_t* lengths_device, uint64_t* sampled, double* seconds) {

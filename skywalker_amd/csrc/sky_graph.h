@@ -85,6 +85,8 @@ void set_online_full_build(int mode);
 uint32_t tiled_max_tiles();
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
                  uint32_t* paths, uint32_t* lengths, uint64_t* sampled, double* seconds);
+int walk_offline_noalloc(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
+                         uint32_t* paths, uint32_t* lengths, uint64_t* sampled_device);
 int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* seeds, uint32_t N, uint32_t len,
                 float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
                 double* seconds);

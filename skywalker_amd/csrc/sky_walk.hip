@@ -17,7 +17,8 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
     const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
     const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t V, uint32_t len,
     float stop_prob, uint64_t seed, uint32_t* __restrict__ paths, uint32_t* __restrict__ lengths,
-    unsigned long long* __restrict__ sampled) {
+    unsigned long long* __restrict__ sampled, unsigned long long* __restrict__ block_partials) {
+  __shared__ unsigned long long s_part[WALK_BLOCK / 64];
   const uint32_t i = blockIdx.x * WALK_BLOCK + threadIdx.x;
   uint32_t s = 0;
   if (i < N) {
@@ -42,7 +43,18 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
   unsigned long long t = s;
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) t += shfl_xor_u64(t, m);
-  if ((threadIdx.x & 63) == 0 && t) atomicAdd(sampled, t);
+  if (block_partials) {  // one sum per workgroup, added up by reduce_partials_kernel: no counter to clear
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = t;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long b = 0;
+#pragma unroll
+      for (int w = 0; w < WALK_BLOCK / 64; ++w) b += s_part[w];
+      block_partials[blockIdx.x] = b;
+    }
+  } else if ((threadIdx.x & 63) == 0 && t) {
+    atomicAdd(sampled, t);
+  }
 }
 
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
@@ -57,7 +69,8 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   SKY_HIP(hipEventRecord(e0, st));
   if (N)
     hipLaunchKernelGGL(walk_offline_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st, g->xadj,
-                       g->adjncy, g->table, seeds, N, g->V, len, stop_prob, seed, paths, lengths, d_sampled);
+                       g->adjncy, g->table, seeds, N, g->V, len, stop_prob, seed, paths, lengths, d_sampled,
+                       (unsigned long long*)nullptr);
   SKY_HIP(hipEventRecord(e1, st));
   SKY_HIP(hipStreamSynchronize(st));
   SKY_HIP(hipGetLastError());
@@ -70,6 +83,61 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   SKY_HIP(hipFree(d_sampled));
   if (sampled) *sampled = h;
   if (seconds) *seconds = ms * 1e-3;
+  return SKY_OK;
+}
+
+// ---------------------------------------------------------------- the same walk without any allocation
+// For callers that cannot allocate (HIP graph capture, serving loops): the per-workgroup counts of sampled
+// edges go to a file-scope device array instead of a counter from hipMalloc, a second kernel adds them up into
+// the caller's own device word, no event is created and nothing is copied to the host.  Every call on a GPU
+// shares that GPU's array: calls that overlap on one GPU race.  Nothing in it needs clearing (each workgroup of
+// a call writes its own element before the sum reads it).
+constexpr uint32_t NOALLOC_MAX_BLOCKS = 16384;  // 128 KiB of device memory per GPU, held until the process ends
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned long long scratch[NOALLOC_MAX_BLOCKS];
+static unsigned long long* g_scratch_ptr[NOALLOC_MAX_DEVICES];  // device address of `scratch` on each GPU
+
+__global__ __launch_bounds__(1024) void reduce_partials_kernel(const unsigned long long* __restrict__ partials,
+                                                               uint32_t n, unsigned long long* __restrict__ out) {
+  __shared__ unsigned long long s_w[16];
+  unsigned long long t = 0;
+  for (uint32_t k = threadIdx.x; k < n; k += 1024u) t += partials[k];
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) t += shfl_xor_u64(t, m);
+  if ((threadIdx.x & 63) == 0) s_w[threadIdx.x >> 6] = t;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long b = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) b += s_w[w];
+    *out = b;
+  }
+}
+
+int walk_offline_noalloc(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob,
+                         uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled_device) {
+  const uint64_t max_walkers = (uint64_t)NOALLOC_MAX_BLOCKS * WALK_BLOCK;
+  if (N > max_walkers)
+    return fail(SKY_ERR_LIMIT, "sky_walk_offline_noalloc: " + std::to_string(N) + " walkers, the static scratch holds " +
+                                   std::to_string(max_walkers) + " (split the batch)");
+  int dev = 0;
+  SKY_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return fail(SKY_ERR_LIMIT, "sky_walk_offline_noalloc: device index beyond 63");
+  if (!g_scratch_ptr[dev]) {  // once per device, with that device current: each GPU holds its own copy of the array
+    unsigned long long* p = nullptr;
+    SKY_HIP(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[dev] = p;
+  }
+  unsigned long long* const partials = g_scratch_ptr[dev];
+  hipStream_t st = g->stream;
+  const uint32_t blocks = (N + WALK_BLOCK - 1) / WALK_BLOCK;
+  if (blocks)
+    hipLaunchKernelGGL(walk_offline_kernel, dim3(blocks), dim3(WALK_BLOCK), 0, st, g->xadj, g->adjncy, g->table, seeds,
+                       N, g->V, len, stop_prob, seed, paths, lengths, (unsigned long long*)nullptr, partials);
+  if (sampled_device)
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, blocks,
+                       reinterpret_cast<unsigned long long*>(sampled_device));
+  SKY_HIP(hipGetLastError());
   return SKY_OK;
 }
 
