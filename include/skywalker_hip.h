@@ -102,7 +102,10 @@ int sky_graph_free(sky_graph* g);
 int sky_alias_build_all(sky_graph* g, double* seconds);
 /* Copies the table to host as two arrays (any destination may be NULL). */
 int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid);
-/* Installs caller-built tables (host arrays) instead of building: for tests and table persistence. */
+/* Installs caller-built tables (host arrays) instead of building: for tests and table persistence.  The arrays are
+ * checked before they are used: valid[v] is 0 or 1 (0 for a vertex without edges); every prob lies in [0, 1];
+ * in a valid row every alias is below the row's degree, in an invalid row every alias is SKY_INVALID.
+ * SKY_ERR_ARG otherwise, and the graph keeps the tables it had. */
 int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, const int8_t* valid);
 
 /* ---- start vertices uniform over [0,V): Philox(seed; i). seeds_device[N]. The reference uses 0..N-1
@@ -149,6 +152,11 @@ int sky_sample_layout(const uint32_t* fanout, uint32_t hops, uint64_t* length_pe
 int sky_sample_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
                        uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device,
                        uint64_t* sampled, double* seconds);
+/* sky_sample_online draws WITH replacement, like sky_sample_offline and the reference's offline kernel
+ * (src/offline_sample.cu:109-133): a parent of more than fanout neighbours yields exactly fanout children, which may
+ * repeat, and sample_lengths holds fanout.  The reference's OnlineGBSampleNew draws distinct neighbours by retrying
+ * against a selected[] set and may return fewer than fanout (src/online_sample_new.cu:83-105); that rule is not
+ * offered.  Online and offline results of this library are identical. */
 int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
                       uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device, uint64_t* sampled,
                       double* seconds);

@@ -210,8 +210,37 @@ int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t*
   return SKY_OK;
 }
 
+// A table from outside is data the walk and sample kernels index with: every alias must stay inside its row
+// (or be SKY_INVALID in a row flagged invalid), every prob must be a probability.
+static int check_tables(const uint32_t* xadj, uint32_t V, const float* prob, const uint32_t* alias,
+                        const int8_t* valid) {
+  for (uint32_t v = 0; v < V; ++v) {
+    const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
+    if (valid[v] != 0 && valid[v] != 1)
+      return fail(SKY_ERR_ARG, "sky_alias_upload: valid[" + std::to_string(v) + "] is neither 0 nor 1");
+    if (deg == 0 && valid[v])
+      return fail(SKY_ERR_ARG, "sky_alias_upload: vertex " + std::to_string(v) + " has no edge but is flagged valid");
+    for (uint32_t i = 0; i < deg; ++i) {
+      const float p = prob[off + i];
+      const uint32_t a = alias[off + i];
+      if (!(p >= 0.0f && p <= 1.0f))
+        return fail(SKY_ERR_ARG, "sky_alias_upload: prob of slot " + std::to_string(off + i) + " is not in [0, 1]");
+      if (valid[v] ? a >= deg : a != SKY_INVALID)
+        return fail(SKY_ERR_ARG, "sky_alias_upload: alias of slot " + std::to_string(off + i) + " (row of " +
+                                     std::to_string(deg) + " entries, valid " + std::to_string((int)valid[v]) +
+                                     ") is " + std::to_string(a));
+    }
+  }
+  return SKY_OK;
+}
+
 int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, const int8_t* valid) {
-  if (!g || !prob || !alias || !valid) return fail(SKY_ERR_ARG, "sky_alias_upload: null pointer");
+  if (!g || (g->E && (!prob || !alias)) || (g->V && !valid)) return fail(SKY_ERR_ARG, "sky_alias_upload: null pointer");
+  {
+    std::vector<uint32_t> xadj((size_t)g->V + 1);
+    SKY_HIP(hipMemcpy(xadj.data(), g->xadj, xadj.size() * 4, hipMemcpyDeviceToHost));
+    SKY_TRY(check_tables(xadj.data(), g->V, prob, alias, valid));
+  }
   if (!g->table) SKY_TRY(alloc_padded(&g->table, (size_t)g->E));
   if (!g->valid) SKY_TRY(alloc_padded(&g->valid, (size_t)g->V));
   if (g->E) {

@@ -97,6 +97,15 @@ int main(int argc, char* argv[]) {
     LOG("node2vec is second-order: switching to --ol=1\n");
     FLAGS_ol = true;
   }
+  // the reference takes these as they come (a negative depth indexes hops out of bounds, main.cu:177-186)
+  if (FLAGS_d < 1 || FLAGS_k < 1 || FLAGS_n < 0) {
+    fprintf(stderr, "skywalker: need --d >= 1, --k >= 1 and -n >= 0 (got d=%d k=%d n=%d)\n", FLAGS_d, FLAGS_k, FLAGS_n);
+    return 1;
+  }
+  if (!(FLAGS_tp >= 0.0 && FLAGS_tp <= 1.0) || !(FLAGS_p > 0.0) || !(FLAGS_q > 0.0)) {
+    fprintf(stderr, "skywalker: need 0 <= --tp <= 1, --p > 0 and --q > 0\n");
+    return 1;
+  }
   int sample_size = FLAGS_n;
   const int NeighborSize = FLAGS_k, Depth = FLAGS_d;
   std::vector<uint> hops(Depth + 1, (uint)NeighborSize);
@@ -107,6 +116,10 @@ int main(int argc, char* argv[]) {
   }
   Graph* ginst = new Graph();
   if (!ginst->ok) return 1;
+  if (ginst->numNode == 0) {  // start vertices are taken modulo the vertex count
+    fprintf(stderr, "skywalker: %s has no vertices\n", FLAGS_input.c_str());
+    return 1;
+  }
   if (FLAGS_full && !FLAGS_stream) {
     sample_size = (int)ginst->numNode;
     FLAGS_n = sample_size;

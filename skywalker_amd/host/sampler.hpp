@@ -212,36 +212,61 @@ inline float ConstructTable(Sampler& sampler, uint ngpu = 1, uint index = 0) {
   return (float)sec;
 }
 
-// Table persistence (the reference has none: every run rebuilds).  File: "SKYTBL01", V, E (u64 each), then
-// prob f32[E], alias u32[E], valid i8[V], little endian.
+// Table persistence (the reference has none: every run rebuilds).  File: "SKYTBL02", V, E, fingerprint (u64 each),
+// then prob f32[E], alias u32[E], valid i8[V], little endian.  The fingerprint is FNV-1a over the graph's row
+// offsets and edge weights: every R-MAT graph of one scale and edge factor has the same V and E, so those two
+// alone would let the tables of another graph in.  sky_alias_upload checks the arrays themselves.
+inline bool GraphFingerprint(const gpu_graph& g, uint64_t* out) {
+  std::vector<uint32_t> xadj((size_t)g.vtx_num + 1);
+  std::vector<float> w(g.edge_num);
+  if (sky_graph_download(g.handle, xadj.data(), nullptr, w.data()) != 0) return false;
+  uint64_t h = 1469598103934665603ull;
+  auto mix = [&](const void* p, size_t bytes) {
+    const unsigned char* b = static_cast<const unsigned char*>(p);
+    for (size_t i = 0; i < bytes; ++i) h = (h ^ b[i]) * 1099511628211ull;
+  };
+  mix(xadj.data(), xadj.size() * 4);
+  mix(w.data(), w.size() * 4);
+  *out = h;
+  return true;
+}
 inline bool SaveTable(Sampler& sampler, const std::string& path) {
   const uint64_t V = sampler.ggraph.vtx_num, E = sampler.ggraph.edge_num;
+  uint64_t fp = 0;
+  if (!GraphFingerprint(sampler.ggraph, &fp)) return false;
   std::vector<float> prob(E);
   std::vector<uint32_t> alias(E);
   std::vector<int8_t> valid(V);
   SKY_RT_CALL(sky_alias_download(sampler.ggraph.handle, prob.data(), alias.data(), valid.data()));
   FILE* f = fopen(path.c_str(), "wb");
   if (!f) return false;
-  bool ok = fwrite("SKYTBL01", 1, 8, f) == 8 && fwrite(&V, 8, 1, f) == 1 && fwrite(&E, 8, 1, f) == 1;
+  bool ok = fwrite("SKYTBL02", 1, 8, f) == 8 && fwrite(&V, 8, 1, f) == 1 && fwrite(&E, 8, 1, f) == 1 &&
+            fwrite(&fp, 8, 1, f) == 1;
   ok = ok && fwrite(prob.data(), 4, E, f) == E && fwrite(alias.data(), 4, E, f) == E;
   ok = ok && fwrite(valid.data(), 1, V, f) == V;
   return fclose(f) == 0 && ok;
 }
 inline bool LoadTable(Sampler& sampler, const std::string& path) {
   const uint64_t V = sampler.ggraph.vtx_num, E = sampler.ggraph.edge_num;
+  uint64_t fp = 0;
+  if (!GraphFingerprint(sampler.ggraph, &fp)) return false;
   FILE* f = fopen(path.c_str(), "rb");
   if (!f) return false;
   char magic[8];
-  uint64_t fv = 0, fe = 0;
-  bool ok = fread(magic, 1, 8, f) == 8 && !memcmp(magic, "SKYTBL01", 8) && fread(&fv, 8, 1, f) == 1 &&
-            fread(&fe, 8, 1, f) == 1 && fv == V && fe == E;
+  uint64_t fv = 0, fe = 0, ffp = 0;
+  bool ok = fread(magic, 1, 8, f) == 8 && !memcmp(magic, "SKYTBL02", 8) && fread(&fv, 8, 1, f) == 1 &&
+            fread(&fe, 8, 1, f) == 1 && fread(&ffp, 8, 1, f) == 1 && fv == V && fe == E && ffp == fp;
   std::vector<float> prob(ok ? E : 0);
   std::vector<uint32_t> alias(ok ? E : 0);
   std::vector<int8_t> valid(ok ? V : 0);
   ok = ok && fread(prob.data(), 4, E, f) == E && fread(alias.data(), 4, E, f) == E && fread(valid.data(), 1, V, f) == V;
+  ok = ok && fgetc(f) == EOF;  // nothing may follow
   fclose(f);
   if (!ok) return false;
-  SKY_RT_CALL(sky_alias_upload(sampler.ggraph.handle, prob.data(), alias.data(), valid.data()));
+  if (sky_alias_upload(sampler.ggraph.handle, prob.data(), alias.data(), valid.data()) != 0) {
+    fprintf(stderr, "%s\n", sky_last_error());
+    return false;  // a damaged table: an alias outside its row, a prob that is no probability
+  }
   sampler.ggraph.Refresh();
   sampler.alias_table = sampler.ggraph.alias_table;
   sampler.valid = sampler.ggraph.valid;

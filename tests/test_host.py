@@ -95,16 +95,58 @@ def test_cli_saved_tables_give_the_same_walks(tmp_path, orc):
     assert rc == 0, err
     raw = open(t, "rb").read()
     V, E = len(xadj) - 1, len(adjncy)
-    assert raw[:8] == b"SKYTBL01" and struct.unpack("<2Q", raw[8:24]) == (V, E) and len(raw) == 24 + 8 * E + V
+    assert raw[:8] == b"SKYTBL02" and struct.unpack("<2Q", raw[8:24]) == (V, E) and len(raw) == 32 + 8 * E + V
     prob, alias, valid = orc.alias_build(xadj, w.astype(np.float32))
-    assert np.array_equal(np.frombuffer(raw, np.float32, E, 24).view(np.uint32), prob.view(np.uint32))
-    assert np.array_equal(np.frombuffer(raw, np.uint32, E, 24 + 4 * E), alias)
+    assert np.array_equal(np.frombuffer(raw, np.float32, E, 32).view(np.uint32), prob.view(np.uint32))
+    assert np.array_equal(np.frombuffer(raw, np.uint32, E, 32 + 4 * E), alias)
     rc, out2, err = run(common + ["--loadtable", t])
     assert rc == 0, err
     keep = lambda o: [l for l in o.splitlines() if l.strip()][:-3]  # everything but the timing lines
     assert keep(out1)[1:] == keep(out2)[1:] and len(keep(out1)) >= 7
     rc, _, err = run(common + ["--loadtable", p])  # not a table file
     assert rc != 0 and "cannot use table file" in err
+    # a damaged file: one alias points outside its row.  The library refuses the arrays, nothing walks on them.
+    row = int(np.argmax(np.diff(xadj.astype(np.int64)) >= 3))
+    bad = bytearray(raw)
+    struct.pack_into("<I", bad, 32 + 4 * E + 4 * int(xadj[row]), 0x7FFFFFFF)
+    open(t + ".bad", "wb").write(bytes(bad))
+    rc, _, err = run(common + ["--loadtable", t + ".bad"])
+    assert rc != 0 and "cannot use table file" in err and "alias of slot %d" % xadj[row] in err
+    # the tables of another graph with the same V and E (every R-MAT graph of one scale and edge factor has them)
+    xadj2, adjncy2 = orc.rmat_csr(11, 8, 6)
+    p2 = str(tmp_path / "t2.w.gr")
+    write_gr(p2, xadj2, adjncy2, w)
+    rc, _, err = run([common[0], "--deepwalk", "--bias=1", "--ol=0", "--input", p2, "-n", "10", "--d", "3",
+                      "--loadtable", t])
+    assert rc != 0 and "cannot use table file" in err
+
+
+@pytest.mark.gpu
+def test_alias_upload_checks_the_arrays(orc):
+    from skywalker_amd import capi
+    xadj = np.array([0, 3, 3, 5], np.uint32)
+    adjncy = np.array([1, 2, 2, 0, 1], np.uint32)
+    w = np.array([1, 2, 3, 0, 0], np.float32)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    prob, alias, valid = orc.alias_build(xadj, w)
+    assert valid.tolist() == [1, 0, 0] and alias[3] == capi.INVALID
+    g.upload_tables(prob, alias, valid)  # the oracle's own table passes
+    cases = []
+    a = alias.copy(); a[1] = 3; cases.append((prob, a, valid, "alias of slot 1"))
+    a = alias.copy(); a[3] = 0; cases.append((prob, a, valid, "alias of slot 3"))      # invalid row must hold SKY_INVALID
+    a = alias.copy(); a[0] = capi.INVALID; cases.append((prob, a, valid, "alias of slot 0"))
+    p = prob.copy(); p[2] = np.nan; cases.append((p, alias, valid, "prob of slot 2"))
+    p = prob.copy(); p[0] = 1.5; cases.append((p, alias, valid, "prob of slot 0"))
+    p = prob.copy(); p[0] = -0.25; cases.append((p, alias, valid, "prob of slot 0"))
+    v = valid.copy(); v[1] = 1; cases.append((prob, alias, v, "no edge"))
+    v = valid.copy(); v[0] = 2; cases.append((prob, alias, v, "neither 0 nor 1"))
+    for pp, aa, vv, msg in cases:
+        with pytest.raises(capi.SkyError) as e:
+            g.upload_tables(pp, aa, vv)
+        assert e.value.code == -1 and msg in str(e.value), (msg, str(e.value))
+    got = g.tables()  # the graph still holds the last good tables
+    assert np.array_equal(got[0], prob) and np.array_equal(got[1], alias) and np.array_equal(got[2], valid)
+    g.free()
 
 
 @pytest.mark.gpu
@@ -170,6 +212,76 @@ def test_cli_online_sage_and_csv(tmp_path, orc):
     assert hop1 == data[0, 1:1 + sl[0, 0]].tolist()
     last = out.strip().splitlines()[-1]
     assert last.startswith("s.w.gr,") or re.match(r"^[\d.]+,\t[\d.]+,$", last)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("online", [0, 1])
+def test_cli_unbiased_two_hop_sampling(tmp_path, orc, online):
+    # --bias=0 --sage: the reference's unbiased k-hop sampler (src/unbiased_sample.cu:10-316) = unit weights here
+    xadj, adjncy = orc.rmat_csr(11, 8, 21)
+    w = (orc.gen_weights(orc.W_UNIFORM, 21, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "us.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--sage", "--bias=0", "--ol=%d" % online, "--input", p, "-n", "300",
+                        "--printresult", "--seed", "3"])
+    assert rc == 0, err
+    ones = np.ones(len(adjncy), np.float32)
+    data, sl, sampled = orc.sample_online(xadj, adjncy, ones, np.arange(300, dtype=np.uint32), [1, 25, 10], 3)
+    blocks = out.split("th sample src: ")[1:]
+    assert len(blocks) == 4
+    for j, blk in enumerate(blocks):
+        m = re.match(r"(\d+), 1-hop len: (\d+)", blk)
+        assert int(m.group(1)) == j and int(m.group(2)) == sl[j, 0]
+        hop1 = [int(x) for x in blk.split("1-hop : ")[1].splitlines()[0].split()]
+        assert hop1 == data[j, 1:1 + sl[j, 0]].tolist()
+        for i in range(sl[j, 0]):
+            line = blk.split("\t %d th 2-hop [%d]: " % (i, data[j, 1 + i]))[1].splitlines()[0]
+            assert [int(x) for x in line.split()] == data[j, 26 + 10 * i:26 + 10 * i + min(sl[j, 1 + i], 30)].tolist()
+    lines = [l for l in out.splitlines() if l.strip()]
+    sample_ms, mseps = float(lines[-2]), float(lines[-1])  # no table line for an unbiased run (main.cu:406)
+    assert abs(mseps - sampled / (sample_ms * 1e-3) / 1e6) <= 0.02 * mseps + 0.02
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("table", [False, True])
+def test_cli_unbiased_node2vec(tmp_path, orc, table):
+    # --bias=0 --node2vec: the reference's unbiased node2vec walker (src/unbiased_walk.cu:14-60) = unit weights here
+    xadj, adjncy = orc.rmat_csr(11, 8, 23)
+    w = (orc.gen_weights(orc.W_UNIFORM, 23, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "un.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--node2vec", "--bias=0", "--input", p, "-n", "400", "--d", "15",
+                        "--p", "0.5", "--q", "2", "--printresult", "--seed", "8"] + (["--n2v_table"] if table else []))
+    assert rc == 0, err
+    lines = out.splitlines()
+    ones = np.ones(len(adjncy), np.float32)
+    seeds = np.arange(400, dtype=np.uint32)
+    if table:
+        paths, lengths, sampled = orc.walk_online(xadj, adjncy, ones, 1, 0.5, 2.0, seeds, 15, 0.0, 8)
+    else:
+        prob, alias, valid = orc.alias_build(xadj, ones)
+        paths, lengths, sampled = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, 0.5, 2.0, seeds, 15, 0.0, 8)
+    for j in range(3):
+        i = lines.index("%drd path len %d " % (j, lengths[j]))
+        assert [int(x) for x in lines[i + 1].split()] == paths[j, :min(lengths[j], 16)].tolist()
+    sample_ms, mseps = (float(l.strip()) for l in lines[-2:])
+    assert abs(mseps - sampled / (sample_ms * 1e-3) / 1e6) <= 0.02 * mseps + 0.02
+
+
+@pytest.mark.parametrize("flags,msg", [(["--d", "-1"], "--d >= 1"), (["--d", "0"], "--d >= 1"), (["-n", "-5"], "-n >= 0"),
+                                       (["--k", "0"], "--k >= 1"), (["--tp", "1.5"], "--tp"), (["--p", "0"], "--p > 0")])
+def test_cli_rejects_bad_numbers(flags, msg):
+    # checked before any file is opened or any device is touched
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--input", "/nonexistent"] + flags)
+    assert rc == 1 and msg in err
+
+
+@pytest.mark.gpu
+def test_cli_rejects_a_graph_without_vertices(tmp_path):
+    p = str(tmp_path / "empty.gr")
+    write_gr(p, np.zeros(1, np.uint32), np.zeros(0, np.uint32))
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--input", p])
+    assert rc == 1 and "no vertices" in err
 
 
 @pytest.mark.gpu
