@@ -6,17 +6,19 @@
 // prefix exceeds the light's exclusive deficit prefix, and a heavy's residual probability belongs
 // to the one light whose deficit interval (SL - D, SL] contains the heavy's surplus prefix.  So
 //   pass A   exact sum of the weights -> ledger
-//   collect  the next ST_CAP heavies in slot order into LDS, {surplus prefix, slot}, 10 bytes each,
-//            and the slot of the heavy after them, if there is one; each takes the next heavy as
-//            alias, the row's last heavy keeps {1, itself}
+//   collect  the next ST_CAP heavies in slot order into LDS, {surplus prefix, slot, residual}, 14 bytes
+//            each, and the slot of the heavy after them, if there is one
 //   emit     classify every entry, running deficit prefix; a light whose alias lies in the window
-//            gets its entry, and every light finishes the window's heavies that fall into its
-//            deficit interval (usually none, sometimes one)
-// Rows with more heavies than one window holds repeat collect and emit: both move through the row
-// in slot order and only come back to the chunk in which the previous window ended, because the
-// alias ranks of the lights and the slots of the heavies both grow along the row.  Heavies no light
-// reaches keep {1, itself}.  A heavy's probability and alias are separate 4-byte stores by
-// different threads of the workgroup.  After the first pass the weights come from L2.
+//            gets its entry, and every light leaves the residual of the window's heavies that fall
+//            into its deficit interval (usually none, sometimes one) in the window; entries go out
+//            four at a time as two 16-byte stores, heavy slots among them carry a placeholder
+//   sweep    every heavy of the window gets its final entry from the window: {residual, next heavy}
+//            when a light reached it and it is not the row's last heavy, {1, itself} otherwise
+// Rows with more heavies than one window holds repeat collect, emit and sweep: all move through
+// the row in slot order and only come back to the chunk in which the previous window ended, because
+// the alias ranks of the lights and the slots of the heavies both grow along the row.  An emit pass
+// leaves alone what belongs to another window: lights whose alias lies outside this one, and heavies of
+// earlier windows, whose final entries are already written.  After the first pass the weights come from L2.
 #include "sky_build_common.h"
 #include "sky_graph.h"
 
@@ -26,7 +28,7 @@ constexpr int ST_T = 512;                 // threads per row
 constexpr int ST_PER = 8;                 // consecutive slots per thread and chunk
 constexpr int ST_CH = ST_T * ST_PER;      // slots per chunk
 constexpr int ST_NW = ST_T / 64;
-constexpr uint32_t ST_CAP = 8063;         // heavies per row kept in LDS (and one sentinel): two workgroups share a CU's 160 KB
+constexpr uint32_t ST_CAP = 5815;         // heavies per row kept in LDS (and one sentinel): two workgroups share a CU's 160 KB
 static_assert(STREAM_MAX_DEG + 3 <= 65536, "heavy slots are stored as 16-bit numbers");
 
 struct StreamRow {
@@ -103,6 +105,22 @@ __device__ __forceinline__ void stream_excl(uint64_t a, uint32_t c, uint64_t* s_
   tot_c = rc;
 }
 
+// The same for one u32 per thread alone.
+__device__ __forceinline__ void stream_excl_c(uint32_t c, uint32_t* s_c, uint32_t& ex_c, uint32_t& tot_c) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint32_t ic = group_scan_u32<64>(c);
+  if (lane == 63) s_c[wave] = ic;
+  __syncthreads();
+  uint32_t rc = 0;
+  ex_c = ic - c;
+#pragma unroll
+  for (int w = 0; w < ST_NW; ++w) {
+    if (w == wave) ex_c += rc;
+    rc += s_c[w];
+  }
+  tot_c = rc;
+}
+
 // For M keys at once: number of entries of the sorted LDS array a[0..n), n >= 1, that are <= key[m].
 // The M chains of dependent LDS reads advance in lockstep, so their latencies overlap.
 template <int M>
@@ -140,6 +158,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
                                                             AliasEntry* __restrict__ table,
                                                             int8_t* __restrict__ valid) {
   __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the window's h-th heavy, then a sentinel
+  __shared__ float s_prob[ST_CAP + 1];     // its residual probability, left by the light that reaches it
   __shared__ uint16_t s_slot[ST_CAP + 1];  // its span slot; after them the slot lights beyond the window take
   __shared__ WSum3 s_w[ST_NW];
   __shared__ uint64_t s_a[2][ST_NW];  // two sets of wavefront sums, used alternately
@@ -215,10 +234,10 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   float* s_w32 = reinterpret_cast<float*>(s_sh);  // weight of heavy h in the low half of s_sh[h], until its prefix replaces it
 
   // window state: collecting resumes at chunk cb (cnt_cb heavies lie before it), emitting at chunk cc
-  // (def_cc deficits lie before it)
+  // (def_cc deficits and hc_cc heavies lie before it)
   uint32_t hb = 0;     // rank of the window's first heavy
   uint64_t sh_lo = 0;  // surplus prefix of the heavies before the window
-  uint32_t cb = 0, cnt_cb = 0, cc = 0;
+  uint32_t cb = 0, cnt_cb = 0, cc = 0, hc_cc = 0;
   uint64_t def_cc = 0;
   for (;;) {
     // ---- collect: heavies of ranks [hb, hb + ST_CAP) and the slot of rank hb + ST_CAP
@@ -244,9 +263,8 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
             if (idx - r.lead < r.span - r.lead && hv) heavy |= 1u << (q * 4 + k);
           }
         }
-      uint64_t ex_u, tot_u;
       uint32_t ex_c, tot_c;
-      stream_excl(0ull, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_u, ex_c, tot_u, tot_c);
+      stream_excl_c((uint32_t)__popc(heavy), s_c[c & 1], ex_c, tot_c);
       uint32_t rank = cnt + ex_c;
 #pragma unroll
       for (int j = 0; j < ST_PER; ++j)
@@ -274,15 +292,19 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     const uint32_t next_slot = more ? uniform_u32(s_next) : NONE32;
     uint64_t sh_hi;  // surplus prefix of the window's last heavy
     {
-      // surplus prefix of the window: 16 consecutive heavies per thread
-      constexpr int HP = 16;
+      // surplus prefix of the window: HP consecutive heavies per thread; the surplus takes the weight's place
+      // in s_sh first, the prefix takes the surplus's place after the scan
+      constexpr int HP = 12;
       static_assert(ST_CAP < (uint32_t)ST_T * HP, "one round covers the window");
-      // (the amounts are computed twice rather than kept: 32 registers less at the kernel's widest point)
       uint64_t su = 0;
 #pragma unroll
       for (int k = 0; k < HP; ++k) {
         const uint32_t h = (uint32_t)HP * tid + k;
-        if (h < nw) su += classify_fast((double)s_w32[2 * h], true, L).amount;
+        if (h < nw) {
+          const uint64_t a = classify_fast((double)s_w32[2 * h], true, L).amount;
+          s_sh[h] = a;
+          su += a;
+        }
       }
       uint64_t ex_u, tot_u;
       uint32_t ex_c, tot_c;
@@ -292,7 +314,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       for (int k = 0; k < HP; ++k) {
         const uint32_t h = (uint32_t)HP * tid + k;
         if (h < nw) {
-          acc += classify_fast((double)s_w32[2 * h], true, L).amount;  // read before s_sh[h] takes its place
+          acc += s_sh[h];
           s_sh[h] = acc;
         }
       }
@@ -300,18 +322,6 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     }
     const bool any_heavy = hb + nw != 0;
     const bool whole_row = hb == 0 && !more;  // the usual case: one window holds every heavy of the row
-    // every heavy takes the next heavy as alias; the row's last heavy keeps its bucket.  When the window holds
-    // the whole row the emit pass meets every heavy and writes this beside the entries of its neighbours
-    // (a store of its own here costs a second write of the line); otherwise it is written from the list.
-    for (uint32_t h = tid; h < nw && !whole_row; h += ST_T) {
-      const uint32_t slot = s_slot[h];
-      const uint32_t nxt = h + 1 < nw ? (uint32_t)s_slot[h + 1] : next_slot;
-      if (nxt != NONE32) {
-        table[r.base + slot].alias = nxt - r.lead;
-      } else {
-        table[r.base + slot] = AliasEntry{1.0f, slot - r.lead};
-      }
-    }
     if (tid == 0) {  // after the list: a sentinel, and the slot that lights beyond the window's last heavy take
       s_sh[nw] = ~0ull;
       s_slot[nw] = more ? (uint16_t)next_slot : (nw ? s_slot[nw - 1] : (uint16_t)0);
@@ -320,18 +330,16 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
 
     // ---- emit: chunks from cc on, until the deficits before a chunk reach the window's last surplus prefix
     uint64_t carry_d = def_cc;
-    uint32_t carry_c = 0;        // heavies before the chunk (kept for whole_row only, where cc = 0)
+    uint32_t carry_c = hc_cc;    // heavies before the chunk
     uint32_t last_c = cc;        // the last chunk worked on, where the next window starts again
     uint64_t last_def = def_cc;  // deficits before it
-    bool reached_end = true;
+    uint32_t last_hc = hc_cc;    // heavies before it
     nx = fetch_chunk(wgt, r, cc, tid);
     for (uint32_t c = cc; c < nch; ++c) {
-      if (more && carry_d >= sh_hi) {  // uniform: the lights from here on belong to later windows
-        reached_end = false;
-        break;
-      }
+      if (more && carry_d >= sh_hi) break;  // uniform: the lights from here on belong to later windows
       last_c = c;
       last_def = carry_d;
+      last_hc = carry_c;
       const RawChunk cur = nx;
       if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
       const bool on = wave_in_row(r, c, wave);  // a wavefront past the row's end only takes part in the scan
@@ -345,9 +353,11 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
         live = unpack_chunk(cur, r, c, tid, wd);
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
-          const Entry e = classify_fast(wd[j], (live >> j) & 1, L);
+          // only the lights' amounts are used here, and a deficit stays below 2^F: the short rounding will do
+          const Entry e = classify_small_unmasked(wd[j], L);
+          const bool in = (live >> j) & 1;
           op[j] = (float)e.p;
-          dl[j] = e.heavy ? 0 : e.amount;
+          dl[j] = (e.heavy || !in) ? 0 : e.amount;
           run += dl[j];
           if (e.heavy) heavy |= 1u << j;
         }
@@ -369,45 +379,59 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
         uint64_t hv = s_sh[b];       // ~0 once the window is exhausted
         uint32_t hslot = s_slot[b];  // then: the first heavy after the window, or the row's last heavy
         const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
+        uint32_t oa[ST_PER];
+        uint32_t wr = 0;  // entries this window writes: its lights, and heavies as placeholders unless an earlier window owns them
+        uint32_t hrank = carry_c + ex_c;
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
-          if (!((live >> j) & 1)) continue;
           const uint32_t idx = pos0 + j;
+          oa[j] = idx - r.lead;
+          if (!((live >> j) & 1)) continue;
           if ((heavy >> j) & 1) {
-            if (whole_row) {
-              const uint32_t hr = carry_c + ex_c + (uint32_t)__popc(heavy & ((1u << j) - 1));
-              if (hr + 1 < nw) {
-                table[r.base + idx].alias = (uint32_t)s_slot[hr + 1] - r.lead;
-              } else {
-                table[r.base + idx] = AliasEntry{1.0f, idx - r.lead};
-              }
-            }
+            op[j] = 1.0f;
+            if (hrank >= hb) wr |= 1u << j;
+            ++hrank;
             continue;
           }
           // the light's alias is the first heavy whose surplus prefix exceeds sl: in this window iff
           // sh_lo <= sl < sh_hi, or beyond every heavy of the row
-          if (whole_row || (sl >= sh_lo && (sl < sh_hi || !more)))
-            table[r.base + idx] = AliasEntry{op[j], (any_heavy ? hslot : idx) - r.lead};
+          if (whole_row || (sl >= sh_lo && (sl < sh_hi || !more))) wr |= 1u << j;
+          if (any_heavy) oa[j] = hslot - r.lead;
           // heavies of the window whose surplus prefix lies in (sl, sl + D]: this light finishes them
           sl += dl[j];
           while (hv <= sl) {
-            if (b + 1 < nw || more) table[r.base + hslot].prob = residual_prob(L.one + hv - sl, L);
+            s_prob[b] = residual_prob(L.one + hv - sl, L);
             ++b;
             hv = s_sh[b];
             hslot = s_slot[b];
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < ST_PER / 4; ++q) {
+          const uint32_t m = (wr >> (4 * q)) & 15u;
+          AliasEntry* t = table + r.base + pos0 + 4 * q;
+          if (m == 15u) {
+            const float p4[4] = {op[4 * q], op[4 * q + 1], op[4 * q + 2], op[4 * q + 3]};
+            const uint32_t a4[4] = {oa[4 * q], oa[4 * q + 1], oa[4 * q + 2], oa[4 * q + 3]};
+            store_entries4(t, p4, a4);
+          } else if (m) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              if ((m >> k) & 1) t[k] = AliasEntry{op[4 * q + k], oa[4 * q + k]};
           }
         }
       }
       carry_d += uniform_u64(tot_d);
       carry_c += uniform_u32(tot_c);
     }
-    if (reached_end) {  // carry_d is the row's total deficit: heavies beyond it are reached by no light
-      __syncthreads();
-      for (uint32_t h = tid; h < nw; h += ST_T)
-        if (s_sh[h] > carry_d && (h + 1 < nw || more)) {
-          const uint32_t slot = s_slot[h];
-          table[r.base + slot] = AliasEntry{1.0f, slot - r.lead};
-        }
+    // ---- sweep: the final entry of every heavy of the window.  A light reached it iff its surplus prefix is
+    // within the deficits seen (all of them when the pass stopped early: it stops once they cover the window).
+    __syncthreads();  // also orders the placeholders before the entries that replace them: the barrier's release waits for this wavefront's stores
+    for (uint32_t h = tid; h < nw; h += ST_T) {
+      const uint32_t slot = s_slot[h];
+      const uint32_t nxt = h + 1 < nw ? (uint32_t)s_slot[h + 1] : next_slot;
+      const bool fin = nxt != NONE32 && s_sh[h] <= carry_d;
+      table[r.base + slot] = fin ? AliasEntry{s_prob[h], nxt - r.lead} : AliasEntry{1.0f, slot - r.lead};
     }
     if (!more) break;
     hb += nw;
@@ -416,7 +440,8 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     cnt_cb = next_cnt_cb;
     cc = last_c;
     def_cc = last_def;
-    __syncthreads();  // the lists are rewritten by the next window
+    hc_cc = last_hc;
+    __syncthreads();  // the lists are rewritten by the next window, whose stores must not overtake this sweep's
   }
 }
 
