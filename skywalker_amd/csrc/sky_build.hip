@@ -33,19 +33,184 @@ namespace sky {
 __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d == 0) return CLS_EMPTY;
   if (d <= 2) return CLS_TINY;
-  // 6-slot variants of the narrower groups cost more per edge than they gain in fill
-  if (d <= 5) return CLS_G2;
-  if (d <= 13) return CLS_G4;
-  if (d <= 29) return CLS_G8;
-  if (d <= 61) return CLS_G16;
-  if (d <= 125) return CLS_G32;
-  if (d <= 191) return CLS_G32X;
+  // rows of the group kernels start at any slot (their vector loads and stores only need 4-byte alignment)
+  if (d <= 8) return CLS_G2;
+  if (d <= 16) return CLS_G4;
+  if (d <= 32) return CLS_G8;
+  if (d <= 64) return CLS_G16;
+  if (d <= 128) return CLS_G32;
+  if (d <= 192) return CLS_G32X;
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
   if (nw <= 16) return CLS_MW2 + (int)nw - 2;
   if (d > STREAM_MAX_DEG) return CLS_HUGE;
   return d > 24576u ? CLS_STREAM : CLS_STREAM_LAST;
+}
+
+// Vectors that are only 4-byte aligned: global loads and stores of 8 and 16 bytes need no more on gfx950.
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef float float2u __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint32_t uint4u __attribute__((ext_vector_type(4), aligned(4)));
+
+// ---------------------------------------------------------------- 2..32 lanes per row
+// G lanes share one row of at most PER * G slots; every lane holds PER consecutive weights, so a
+// wavefront carries 64 / G rows and the per-row steps that do not depend on the row length (exact
+// sum, ledger, scans) are paid once per 64 / G rows.  Prefix sums run over the group by DPP; SL and
+// SH of every slot go to a per-group LDS strip padded to PER * G slots (slots outside the row add
+// nothing), which each entry then searches once with a fixed number of probes; the heavies' slots,
+// compacted by rank, give "next heavy" and "last heavy".  The rank rides in bits 52..63 of the SH scan.
+// Every lane of the wavefront must call this together (DPP); a group without a row passes d = 0.
+// s_pre: [2 * 256 * PER] u64 ([0, BLK): SL of every slot of the block; [BLK, 2 * BLK): SH), s_hs: [256 * PER]
+// (per group: row-local slot of its h-th heavy).  Returns false for a row whose weights sum to zero.
+constexpr uint64_t GROUP_CNT = 1ull << 52;
+
+template <int G, int PER>
+__device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const float* __restrict__ wgt,
+                                                AliasEntry* __restrict__ table, uint64_t* __restrict__ s_pre,
+                                                uint8_t* __restrict__ s_hs) {
+  static_assert(PER == 4 || PER == 6, "a lane loads one float4 or three float2");
+  constexpr uint32_t SLOTS = PER * G;
+  constexpr uint32_t HB = PER == 4 ? SLOTS : SLOTS / 3 * 2;  // largest power of two <= SLOTS
+  constexpr uint32_t BLK = 256 * PER;                        // slots of one block's strips
+  const int gl = threadIdx.x & (G - 1);
+  const int lane = lane_id();
+  const uint32_t gbase = (uint32_t)PER * (threadIdx.x - gl);  // first LDS slot of the group
+  const uint32_t pos = (uint32_t)PER * gl;
+
+  float xs[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) xs[k] = 0.0f;
+  if (PER == 4) {
+    if (pos < d) {
+      const float4u x = *reinterpret_cast<const float4u*>(wgt + off + pos);
+      xs[0] = x.x; xs[1] = x.y; xs[2] = x.z; xs[3] = x.w;
+    }
+  } else {
+#pragma unroll
+    for (int h = 0; h < PER / 2; ++h)
+      if (pos + 2 * h < d) {
+        const float2u x = *reinterpret_cast<const float2u*>(wgt + off + pos + 2 * h);
+        xs[2 * h] = x.x;
+        xs[2 * h + 1] = x.y;
+      }
+  }
+  double wd[PER];
+  uint32_t live = 0;
+  WSum3 S{0.0, 0.0, 0.0};
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const bool in = pos + k < d;
+    if (in) live |= 1u << k;
+    wd[k] = (double)masked_weight(xs[k], in);
+    wsum3_add(S, wd[k]);
+  }
+  S = group_sum_wsum3<G>(S);
+  const bool row_ok = S.top + S.mid + S.low != 0.0;
+  Ledger L = make_ledger_small(d, wsum3_to_double(S));
+  if (!row_ok) L.scale = 0.0;
+
+  uint64_t dl[PER], sl[PER], sh[PER];
+  float op[PER];
+  uint32_t heavy = 0;
+  uint64_t ra = 0, rb = 0;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const Entry e = classify_small_unmasked(wd[k], L);
+    dl[k] = (e.heavy || !((live >> k) & 1)) ? 0 : e.amount;
+    ra += dl[k];
+    rb += e.heavy ? (e.amount | GROUP_CNT) : 0;
+    sl[k] = ra;
+    sh[k] = rb;
+    op[k] = (float)e.p;
+    if (e.heavy) heavy |= 1u << k;
+  }
+  const uint64_t ia = group_scan_u64<G>(ra), ib = group_scan_u64<G>(rb);
+  const uint32_t nh = (uint32_t)(shfl_u64(ib, (lane - gl) + G - 1) >> 52);
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    sl[k] += ia - ra;
+    sh[k] += ib - rb;
+    s_pre[gbase + pos + k] = sl[k];
+    s_pre[BLK + gbase + pos + k] = sh[k] & (GROUP_CNT - 1);
+    if ((heavy >> k) & 1) s_hs[gbase + (uint32_t)(sh[k] >> 52) - 1] = (uint8_t)(pos + k);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // light: first slot with SH > SL - D.  heavy: first slot with SL >= SH, i.e. SL > SH - 1.
+  // The first probe narrows the answer to a window of HB slots that ends inside the strip.
+  uint32_t arr[PER], at[PER];
+  uint64_t key[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const bool hv = (heavy >> k) & 1;
+    arr[k] = gbase + (hv ? 0u : BLK);
+    key[k] = hv ? (sh[k] & (GROUP_CNT - 1)) - 1 : sl[k] - dl[k];
+    at[k] = HB == SLOTS ? 0u : (s_pre[arr[k] + HB - 1] <= key[k] ? SLOTS - HB : 0u);
+  }
+#pragma unroll
+  for (uint32_t step = HB / 2; step >= 1; step >>= 1) {
+    uint64_t v[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) v[k] = s_pre[arr[k] + at[k] + step - 1];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) at[k] += v[k] <= key[k] ? step : 0u;
+  }
+  uint32_t oa[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const uint64_t v = s_pre[arr[k] + at[k]];
+    const bool found = v > key[k];
+    const uint32_t self = pos + k;
+    if (!((heavy >> k) & 1)) {
+      oa[k] = found ? at[k] : (nh ? (uint32_t)s_hs[gbase + nh - 1] : self);
+    } else {
+      const uint32_t hc = (uint32_t)(sh[k] >> 52);
+      if (hc < nh && found) {
+        op[k] = residual_prob(L.one + key[k] + 1 - v, L);
+        oa[k] = s_hs[gbase + hc];
+      } else {
+        op[k] = 1.0f;
+        oa[k] = self;
+      }
+    }
+    if (!row_ok) {
+      op[k] = 0.0f;
+      oa[k] = SKY_INVALID;
+    }
+  }
+  // the next row of this group reuses the strips: its writes must stay behind these reads
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int h = 0; h < PER / 2; ++h) {
+    const uint32_t m = (live >> (2 * h)) & 3u;
+    AliasEntry* t = table + off + pos + 2 * h;
+    if (m == 3u) {
+      uint4u o;
+      o.x = __float_as_uint(op[2 * h]); o.y = oa[2 * h]; o.z = __float_as_uint(op[2 * h + 1]); o.w = oa[2 * h + 1];
+      *reinterpret_cast<uint4u*>(t) = o;
+    } else if (m == 1u) {
+      t[0] = AliasEntry{op[2 * h], oa[2 * h]};
+    }
+  }
+  return row_ok || d == 0;
+}
+
+template <int G, int PER>
+__global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restrict__ vlist, uint32_t count,
+                                                          const float* __restrict__ wgt,
+                                                          AliasEntry* __restrict__ table,
+                                                          int8_t* __restrict__ valid) {
+  __shared__ uint64_t s_pre[2 * 256 * PER];
+  __shared__ uint8_t s_hs[256 * PER];
+  const uint32_t grp = (blockIdx.x * 256u + threadIdx.x) / G;
+  RowRef rr{0, 0, 0, 0};
+  if (grp < count) rr = vlist[grp];
+  const bool ok = group_build_row<G, PER>(rr.off, rr.d, wgt, table, s_pre, s_hs);
+  if ((threadIdx.x & (G - 1)) == 0 && !ok) valid[rr.v] = 0;  // the binning pass has set it
 }
 
 // ---------------------------------------------------------------- binning
@@ -106,8 +271,41 @@ __global__ __launch_bounds__(64) void bin_offsets_kernel(uint32_t* __restrict__ 
   if (lane == 0) counts[c] = run;
 }
 
+// A row of one or two entries in closed form.
+__device__ __forceinline__ bool tiny_row(uint32_t off, uint32_t d, const float* __restrict__ wgt,
+                                         AliasEntry* __restrict__ table) {
+  // a weight adds to the exact sum iff it is at least 2^-64
+  constexpr float UNIT = 5.421010862427522170037e-20f;  // 2^-64
+  const float w0 = clamp_weight(wgt[off]);
+  if (d == 1) {
+    const bool ok = w0 >= UNIT;
+    table[off] = AliasEntry{ok ? 1.0f : 0.0f, ok ? 0u : SKY_INVALID};
+    return ok;
+  }
+  const float w1 = clamp_weight(wgt[off + 1]);
+  const bool ok = w0 >= UNIT || w1 >= UNIT;
+  AliasEntry a{0.0f, SKY_INVALID}, b{0.0f, SKY_INVALID};
+  if (ok) {
+    WSum3 S{0.0, 0.0, 0.0};
+    wsum3_add(S, (double)w0);
+    wsum3_add(S, (double)w1);
+    const Ledger L = make_ledger_small(2, wsum3_to_double(S));
+    const Entry e0 = classify_small((double)w0, true, L), e1 = classify_small((double)w1, true, L);
+    // a lone heavy is the last heavy: it keeps its bucket and tops up the light
+    a = AliasEntry{e0.heavy ? 1.0f : (float)e0.p, (!e0.heavy && e1.heavy) ? 1u : 0u};
+    b = AliasEntry{e1.heavy ? 1.0f : (float)e1.p, (!e1.heavy && e0.heavy) ? 0u : 1u};
+  }
+  uint4u o;
+  o.x = __float_as_uint(a.prob); o.y = a.alias; o.z = __float_as_uint(b.prob); o.w = b.alias;
+  *reinterpret_cast<uint4u*>(table + off) = o;
+  return ok;
+}
+
 // Writes each row of class >= CLS_G2 into its class segment of vlist, and finishes
-// the classes that need no cooperation: deg 0 (valid = 0) and deg 1..2 (closed form).
+// the classes that need no cooperation: deg 0 (valid = 0) and deg 1..2 (closed form).  The rows of one
+// or two entries that a wavefront meets in a step go to a list of its own in LDS first and are then
+// built with its lanes side by side (they are a fifth of the vertices of a power-law graph: built where
+// they are met, every step would pay for them with most lanes idle).
 __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __restrict__ xadj,
                                                           const float* __restrict__ wgt,
                                                           const uint32_t* __restrict__ src, uint32_t n,
@@ -118,204 +316,47 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
                                                           AliasEntry* __restrict__ table,
                                                           int8_t* __restrict__ valid) {
   __shared__ uint32_t s_cur[CLS_COUNT];
+  __shared__ uint2 s_tiny[4][64 * BIN_ITEMS];  // per wavefront: {offset, vertex} of its rows of 1..2 entries
+  __shared__ uint8_t s_tiny_d[4][64 * BIN_ITEMS];
   if (threadIdx.x < CLS_COUNT)
     s_cur[threadIdx.x] = class_start[threadIdx.x] + blk_off[blockIdx.x * CLS_COUNT + threadIdx.x];
   __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
   for (uint32_t chunk = lo; chunk < hi; chunk += 256u * BIN_ITEMS) {
+    uint32_t nt = 0;  // wave-uniform: rows in this wavefront's list
 #pragma unroll
     for (int i = 0; i < BIN_ITEMS; ++i) {
       const uint32_t item = chunk + i * 256u + threadIdx.x;
-      if (item >= hi) continue;
-      const uint32_t v = src ? src[item] : item;
-      const uint32_t off = xadj[v], d = xadj[v + 1] - off;
-      const int c = degree_class(d);
-      if (c == CLS_EMPTY) {
-        valid[v] = 0;
-      } else if (c == CLS_TINY) {
-        // a weight adds to the exact sum iff it is at least 2^-64
-        constexpr float UNIT = 5.421010862427522170037e-20f;  // 2^-64
-        const float w0 = clamp_weight(wgt[off]);
-        if (d == 1) {
-          const bool ok = w0 >= UNIT;
-          table[off] = AliasEntry{ok ? 1.0f : 0.0f, ok ? 0u : SKY_INVALID};
-          valid[v] = ok;
-        } else {
-          const float w1 = clamp_weight(wgt[off + 1]);
-          if (!(w0 >= UNIT || w1 >= UNIT)) {
-            table[off] = table[off + 1] = AliasEntry{0.0f, SKY_INVALID};
-            valid[v] = 0;
-          } else {
-            WSum3 S{0.0, 0.0, 0.0};
-            wsum3_add(S, (double)w0);
-            wsum3_add(S, (double)w1);
-            const Ledger L = make_ledger_small(2, wsum3_to_double(S));
-            const Entry e0 = classify_small((double)w0, true, L), e1 = classify_small((double)w1, true, L);
-            // a lone heavy is the last heavy: it keeps its bucket and tops up the light
-            table[off] = AliasEntry{e0.heavy ? 1.0f : (float)e0.p, (!e0.heavy && e1.heavy) ? 1u : 0u};
-            table[off + 1] = AliasEntry{e1.heavy ? 1.0f : (float)e1.p, (!e1.heavy && e0.heavy) ? 0u : 1u};
-            valid[v] = 1;
-          }
-        }
-      } else {
+      int c = -1;
+      uint32_t v = 0, off = 0, d = 0;
+      if (item < hi) {
+        v = src ? src[item] : item;
+        off = xadj[v];
+        d = xadj[v + 1] - off;
+        c = degree_class(d);
+      }
+      const unsigned long long m = __ballot(c == CLS_TINY);
+      if (c == CLS_TINY) {
+        const uint32_t p = nt + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+        s_tiny[wave][p] = make_uint2(off, v);
+        s_tiny_d[wave][p] = (uint8_t)d;
+      } else if (c >= CLS_G2) {
         vlist[atomicAdd(&s_cur[c], 1u)] = RowRef{v, off, d, 0};
-        valid[v] = 1;  // written here, next to its neighbours' flags; the row's kernel clears it if the row has no weight
       }
+      nt += (uint32_t)__popcll(m);
+      if (c >= 0) valid[v] = c != CLS_EMPTY;  // written here, next to its neighbours' flags; a row without weight clears it later
     }
-  }
-}
-
-// ---------------------------------------------------------------- 2..32 lanes per row
-// G lanes share one row of at most PER * G slots, counted from the row's aligned start (16 bytes for
-// PER = 4, 8 bytes for PER = 6); every lane holds PER consecutive weights, so a wavefront carries
-// 64 / G rows and the per-row steps that do not depend on the row length (exact sum, ledger, scans)
-// are paid once per 64 / G rows.  Prefix sums run over the group by DPP; SL and SH of every slot go
-// to a per-group LDS strip padded to PER * G slots (slots outside the row add nothing), which each
-// entry then searches once with a fixed number of probes; the heavies' slots, compacted by rank,
-// give "next heavy" and "last heavy".  The rank rides in bits 52..63 of the SH scan.
-constexpr uint64_t GROUP_CNT = 1ull << 52;
-
-template <int G, int PER>
-__global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restrict__ vlist, uint32_t count,
-                                                          const float* __restrict__ wgt,
-                                                          AliasEntry* __restrict__ table,
-                                                          int8_t* __restrict__ valid) {
-  static_assert(PER == 4 || PER == 6, "a lane loads one float4 or three float2");
-  constexpr uint32_t SLOTS = PER * G;
-  constexpr uint32_t HB = PER == 4 ? SLOTS : SLOTS / 3 * 2;  // largest power of two <= SLOTS
-  constexpr uint32_t ALIGN = PER == 4 ? 4 : 2;               // the row's slots start at a multiple of this
-  constexpr uint32_t BLK = 256 * PER;                        // slots of one block's strips
-  __shared__ uint64_t s_pre[2 * BLK];  // [0, BLK): SL of every slot of the block; [BLK, 2 * BLK): SH
-  __shared__ uint8_t s_hs[BLK];        // per group: row-local slot of its h-th heavy
-  const uint32_t grp = (blockIdx.x * 256u + threadIdx.x) / G;
-  const int gl = threadIdx.x & (G - 1);
-  const int lane = lane_id();
-  const uint32_t gbase = (uint32_t)PER * (threadIdx.x - gl);  // first LDS slot of the group
-  RowRef rr{0, 0, 0, 0};
-  if (grp < count) rr = vlist[grp];
-  const uint32_t off = rr.off, d = rr.d;
-  const uint32_t base = off & ~(ALIGN - 1), lead = off - base, span = d ? lead + d : 0;
-  const uint32_t pos = (uint32_t)PER * gl;
-
-  float xs[PER];
-#pragma unroll
-  for (int k = 0; k < PER; ++k) xs[k] = 0.0f;
-  if (PER == 4) {
-    if (pos < span) {
-      const float4 x = *reinterpret_cast<const float4*>(wgt + base + pos);
-      xs[0] = x.x; xs[1] = x.y; xs[2] = x.z; xs[3] = x.w;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (uint32_t t = lane; t < nt; t += 64u) {
+      const uint2 rec = s_tiny[wave][t];
+      if (!tiny_row(rec.x, s_tiny_d[wave][t], wgt, table)) valid[rec.y] = 0;
     }
-  } else {
-#pragma unroll
-    for (int h = 0; h < PER / 2; ++h)
-      if (pos + 2 * h < span) {
-        const float2 x = *reinterpret_cast<const float2*>(wgt + base + pos + 2 * h);
-        xs[2 * h] = x.x;
-        xs[2 * h + 1] = x.y;
-      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the next step's list entries stay behind these reads
+    __builtin_amdgcn_wave_barrier();
   }
-  double wd[PER];
-  uint32_t live = 0;
-  WSum3 S{0.0, 0.0, 0.0};
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    const uint32_t idx = pos + k;
-    const bool in = idx - lead < d;  // one unsigned compare: slots before the row wrap around
-    if (in) live |= 1u << k;
-    wd[k] = (double)masked_weight(xs[k], in);
-    wsum3_add(S, wd[k]);
-  }
-  S = group_sum_wsum3<G>(S);
-  const bool row_ok = S.top + S.mid + S.low != 0.0;
-  Ledger L = make_ledger_small(d, wsum3_to_double(S));
-  if (!row_ok) L.scale = 0.0;
-
-  uint64_t dl[PER], sl[PER], sh[PER];
-  float op[PER];
-  uint32_t heavy = 0;
-  uint64_t ra = 0, rb = 0;
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    const Entry e = classify_small_unmasked(wd[k], L);
-    dl[k] = (e.heavy || !((live >> k) & 1)) ? 0 : e.amount;
-    ra += dl[k];
-    rb += e.heavy ? (e.amount | GROUP_CNT) : 0;
-    sl[k] = ra;
-    sh[k] = rb;
-    op[k] = (float)e.p;
-    if (e.heavy) heavy |= 1u << k;
-  }
-  const uint64_t ia = group_scan_u64<G>(ra), ib = group_scan_u64<G>(rb);
-  const uint32_t nh = (uint32_t)(shfl_u64(ib, (lane - gl) + G - 1) >> 52);
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    sl[k] += ia - ra;
-    sh[k] += ib - rb;
-    s_pre[gbase + pos + k] = sl[k];
-    s_pre[BLK + gbase + pos + k] = sh[k] & (GROUP_CNT - 1);
-    if ((heavy >> k) & 1) s_hs[gbase + (uint32_t)(sh[k] >> 52) - 1] = (uint8_t)(pos + k - lead);
-  }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-  // light: first slot with SH > SL - D.  heavy: first slot with SL >= SH, i.e. SL > SH - 1.
-  // The first probe narrows the answer to a window of HB slots that ends inside the strip.
-  uint32_t arr[PER], at[PER];
-  uint64_t key[PER];
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    const bool hv = (heavy >> k) & 1;
-    arr[k] = gbase + (hv ? 0u : BLK);
-    key[k] = hv ? (sh[k] & (GROUP_CNT - 1)) - 1 : sl[k] - dl[k];
-    at[k] = HB == SLOTS ? 0u : (s_pre[arr[k] + HB - 1] <= key[k] ? SLOTS - HB : 0u);
-  }
-#pragma unroll
-  for (uint32_t step = HB / 2; step >= 1; step >>= 1) {
-    uint64_t v[PER];
-#pragma unroll
-    for (int k = 0; k < PER; ++k) v[k] = s_pre[arr[k] + at[k] + step - 1];
-#pragma unroll
-    for (int k = 0; k < PER; ++k) at[k] += v[k] <= key[k] ? step : 0u;
-  }
-  uint32_t oa[PER];
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    const uint64_t v = s_pre[arr[k] + at[k]];
-    const bool found = v > key[k];
-    const uint32_t self = pos + k - lead;
-    if (!((heavy >> k) & 1)) {
-      oa[k] = found ? at[k] - lead : (nh ? (uint32_t)s_hs[gbase + nh - 1] : self);
-    } else {
-      const uint32_t hc = (uint32_t)(sh[k] >> 52);
-      if (hc < nh && found) {
-        op[k] = residual_prob(L.one + key[k] + 1 - v, L);
-        oa[k] = s_hs[gbase + hc];
-      } else {
-        op[k] = 1.0f;
-        oa[k] = self;
-      }
-    }
-    if (!row_ok) {
-      op[k] = 0.0f;
-      oa[k] = SKY_INVALID;
-    }
-  }
-  // pairs of entries start at multiples of 16 bytes
-#pragma unroll
-  for (int h = 0; h < PER / 2; ++h) {
-    const uint32_t m = (live >> (2 * h)) & 3u;
-    AliasEntry* t = table + base + pos + 2 * h;
-    if (m == 3u) {
-      *reinterpret_cast<uint4*>(t) =
-          make_uint4(__float_as_uint(op[2 * h]), oa[2 * h], __float_as_uint(op[2 * h + 1]), oa[2 * h + 1]);
-    } else if (m == 1u) {
-      t[0] = AliasEntry{op[2 * h], oa[2 * h]};
-    } else if (m == 2u) {
-      t[1] = AliasEntry{op[2 * h + 1], oa[2 * h + 1]};
-    }
-  }
-  if (gl == 0 && d && !row_ok) valid[rr.v] = 0;  // the binning pass has set it
 }
 
 // ---------------------------------------------------------------- one row per workgroup, prefix arrays in LDS

@@ -31,12 +31,12 @@ namespace sky {
 enum BuildClass : int {
   CLS_EMPTY = 0,    // deg 0            handled while binning
   CLS_TINY = 1,     // deg 1..2         one lane per vertex, handled while binning
-  CLS_G2 = 2,       // deg 3..5         2 lanes per row, 4 slots per lane
-  CLS_G4 = 3,       // deg <= 13        4 lanes
-  CLS_G8 = 4,       // deg <= 29        8 lanes
-  CLS_G16 = 5,      // deg <= 61        16 lanes
-  CLS_G32 = 6,      // deg <= 125       32 lanes
-  CLS_G32X = 7,     // deg <= 191       32 lanes, 6 slots per lane
+  CLS_G2 = 2,       // deg 3..8         2 lanes per row, 4 slots per lane
+  CLS_G4 = 3,       // deg <= 16        4 lanes
+  CLS_G8 = 4,       // deg <= 32        8 lanes
+  CLS_G16 = 5,      // deg <= 64        16 lanes
+  CLS_G32 = 6,      // deg <= 128       32 lanes
+  CLS_G32X = 7,     // deg <= 192       32 lanes, 6 slots per lane
   CLS_LDS_W1 = 8,   // deg <= 253       one wavefront per row, 4 slots per lane
   CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
   CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..16 (class CLS_MW2 + nw - 2): one workgroup per row whose
