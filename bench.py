@@ -2,9 +2,12 @@
 """Benchmark of the alias-method hot path on one MI355X.
 
 A step = one pass of the hot path over one batch of synthetic input that is already resident in HBM:
-offline alias tables for every vertex (sky_alias_build_all), then a biased DeepWalk of length 80 from the
-batch of start vertices (sky_walk_offline), and for the large configuration also PPR (stop 0.15, max 100).
-Prints ONE JSON line.  Only one GPU is ever used.
+  c1, c2, c5  offline alias tables for every vertex (sky_alias_build_all), then a biased DeepWalk of length 80
+              from the batch of start vertices (sky_walk_offline), and for c5 also PPR (stop 0.15, at most 100 steps)
+  c3          online biased 2-hop sampling (sky_sample_online): tables built on the fly for the frontier
+  c4          online node2vec (sky_walk_online): first-order tables of every row rebuilt, then rejection sampling
+The timed steps run without any per-kernel event; the per-kernel figures of the roofline come from extra, untimed
+steps with the library's build profile switched on.  Prints ONE JSON line.  Only one GPU is ever used.
 """
 import argparse
 import json
@@ -30,13 +33,8 @@ CONFIGS = {
 }
 # algorithmic bytes per edge of one launch: read w (4) and write prob + alias (8); the two tiled passes that only
 # read the weights count 4; xadj / valid are per vertex and small
-BYTES_PER_EDGE = {"tiled_sum": 4, "tiled_totals": 4, "bin": 12}
-# HBM bytes per edge measured with rocprofv3 --pmc FETCH_SIZE (x2.0, calibrated on copy_u32_kernel) and WRITE_SIZE
-# (x1.0); see profiles/c5_build_traffic.md
-TRAFFIC_PER_EDGE = {"stream": 19.2, "mw10": 12.1, "mw9": 12.1, "mw4": 12.2, "mw3": 12.2, "mw2": 12.6, "lds_w2": 12.6,
-                    "lds_w1": 14.6, "g32x": 13.0, "g32": 13.8, "g16": 14.8, "g8": 19.2, "g4": 24.1, "g2": 34.5,
-                    "tiled_emit": 24.4, "tiled_sum": 4.3, "tiled_totals": 4.3}
-WALK_TRAFFIC_PER_STEP = 398.5  # walk_offline_kernel, same source
+BYTES_PER_EDGE = {"tiled_sum": 4, "tiled_totals": 4}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "c5_kernel_traffic.txt")
 METRIC = "sampled edges/sec (SEPS) + alias-table build edges/sec on 1 MI355X; % HBM peak"
 ARITHMETIC = "f64 classification and exact three-limb sums, u64 fixed-point ledger, f32 tables, u32 indices"
 KERNEL_OF = {  # build_profile entry -> kernel symbol
@@ -53,7 +51,48 @@ KERNEL_OF.update({"mw3": "build_merge_kernel<256,6>", "mw5": "build_merge_kernel
                   "mw7": "build_merge_kernel<256,14>", "mw9": "build_merge_kernel<768,6>", "mw10": "build_merge_kernel<512,10>"})
 
 
-def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sample=1_000_000):
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def oracle_flags():
+    """Compiler flags of the CPU oracle, as its Makefile states them."""
+    try:
+        for line in open(os.path.join(ROOT, "oracle", "Makefile")):
+            if line.startswith("CXXFLAGS"):
+                return line.split("=", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def load_traffic():
+    """profiles/c5_kernel_traffic.txt: measured HBM bytes per edge (per step for the walk) of every kernel, with the
+    commit and the commands they come from.  Returns (dict kernel -> bytes, header dict) or (None, None)."""
+    try:
+        table, head = {}, {}
+        for line in open(TRAFFIC_FILE):
+            line = line.rstrip("\n")
+            if line.startswith("#"):
+                if ":" in line:
+                    k, v = line[1:].split(":", 1)
+                    head[k.strip()] = v.strip()
+                continue
+            if line.strip():
+                k, v = line.split("\t")
+                table[k] = float(v)
+        return table, head
+    except (OSError, ValueError):
+        return None, None
+
+
+def cpu_baseline_offline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sample=1_000_000):
     """Oracle timed on the host cores, on a bounded sample of the same workload."""
     import numpy as np
     V, E = g.V, g.E
@@ -72,7 +111,8 @@ def cpu_baseline(capi, orc, g, cfg, seeds_d, budget_edges=2_000_000_000, walk_sa
     t_walk = time.perf_counter() - t0
     value = (es + sampled) / (t_build + t_walk)
     return {
-        "value": value, "unit": "edges/s", "cores": orc.num_threads(), "kind": "port",
+        "value": value, "unit": "edges/s", "cores": orc.num_threads(), "cpu": cpu_model(), "kind": "port",
+        "compiler_flags": oracle_flags(),
         "sample": "oracle (C++/OpenMP) on the same graph: alias build of vertices [0,%d) = %d edges in %.3f s "
                   "(%.3e edges/s); DeepWalk L=%d of the first %d walkers = %d steps in %.3f s (%.3e steps/s)" %
                   (vs, es, t_build, es / t_build, cfg["length"], len(seeds), sampled, t_walk, sampled / t_walk),
@@ -113,6 +153,84 @@ def online_bench(args, cfg, capi, g, seeds, name, cus, t_gen, torch):
     capi.synchronize()
     wall = (time.perf_counter() - t0) / args.steps
     sampled, ksec = rec[-1][2], sum(r[3] for r in rec) / len(rec)
+
+    # algorithmic bytes of one batch, from the batch's own output
+    xadj = g.download_xadj()
+    deg = np.diff(xadj.astype(np.int64))
+    if cfg["mode"] == "sage":
+        data = out[0].to_host((N, lps))
+        fan = cfg["fanout"]
+        offs, width, o = [], [], 0
+        wd = 1
+        for f in fan:
+            wd *= f
+            offs.append(o)
+            width.append(wd)
+            o += wd
+        per_slot, rows = 0, []
+        for h in range(len(fan) - 1):
+            front = data[:, offs[h]:offs[h] + width[h]].ravel()
+            front = front[front < g.V]
+            d = deg[front]
+            k = fan[h + 1]
+            # per frontier vertex of degree d > 0: row bounds 8, weights 4 d, min(k, d) neighbour ids read and written
+            per_slot += int((8 + 4 * d[d > 0] + 8 * np.minimum(d[d > 0], k)).sum())
+            rows.append(np.unique(front))
+        distinct = np.unique(np.concatenate(rows)) if rows else np.zeros(0, np.int64)
+        alg_bytes = per_slot
+        # what one batch must move at least when every distinct frontier row is built once (as this library does):
+        # 12 bytes per entry of those rows + 8 per row, + 8 per sampled edge
+        distinct_bytes = int(12 * deg[distinct].sum() + 8 * len(distinct)) + 8 * int(sampled)
+        detail = {"formula": "sum over frontier vertices of 8 + 4 d + 8 min(k, d)",
+                  "distinct_rows_built": int(len(distinct)), "distinct_row_edges": int(deg[distinct].sum()),
+                  "bytes_with_each_distinct_row_built_once": distinct_bytes,
+                  "frac_with_each_distinct_row_built_once": distinct_bytes / ksec / HBM_PEAK}
+        kernel = "one batch: frontier_collect_kernel, the build kernels of the frontier rows, sample_hop_kernel (per hop)"
+    else:
+        steps = sampled
+        if args.n2v_table:
+            paths = out[0].to_host((N, L + 1))
+            lens = out[1].to_host()
+            cur = paths[:, :-1]
+            prev = np.concatenate([paths[:, :1], paths[:, :-2]], axis=1)
+            mask = np.arange(L)[None, :] < lens[:, None]
+            dc = deg[np.where(mask, cur, 0)]
+            dp = deg[np.where(mask, prev, 0)]
+            dp[:, 0] = 0
+            alg_bytes = int(((12 + 8 * dc + 4 * dp) * mask).sum())
+            detail = {"formula": "sum over steps of 12 + 8 d + 4 d_prev"}
+            kernel = "n2v_step_kernel (one launch per step)"
+        else:
+            alg_bytes = 12 * g.E + 5 * g.V + 24 * steps
+            detail = {"formula": "12 E + 5 V (first-order tables) + 24 per step; the rejection trials' reads "
+                                 "(12 + 4 log2 d_prev each) are not counted: a lower bound"}
+            kernel = "one batch: the offline build kernels, walk_n2v_reject_kernel"
+    roofline = {"bound": "hbm", "kernel": kernel, "achieved": alg_bytes / ksec / 1e9, "peak": HBM_PEAK / 1e9,
+                "unit": "GB/s", "frac": alg_bytes / ksec / HBM_PEAK, "traffic": None,
+                "launch_ms": ksec * 1e3, "algorithmic_bytes_per_launch": alg_bytes, "detail": detail}
+
+    cpu = None
+    if not args.no_cpu:
+        from oracle import orc
+        hx, hadj, hw = g.download()
+        hseeds = seeds.to_host()
+        t0 = time.perf_counter()
+        if cfg["mode"] == "sage":
+            _, _, osampled = orc.sample_online(hx, hadj, hw, hseeds, cfg["fanout"], cfg["seed"])
+            what_cpu = "oracle sample_online of the whole batch (%d seeds)" % N
+        elif args.n2v_table:
+            few = 2000
+            _, _, osampled = orc.walk_online(hx, hadj, hw, 1, cfg["p"], cfg["q"], hseeds[:few], cfg["length"], 0.0, cfg["seed"])
+            what_cpu = "oracle walk_online (table per step) of the first %d walkers" % few
+        else:
+            prob, alias, _ = orc.alias_build(hx, hw)
+            _, _, osampled = orc.walk_node2vec_reject(hx, hadj, prob, alias, cfg["p"], cfg["q"], hseeds, cfg["length"], 0.0,
+                                                      cfg["seed"])
+            what_cpu = "oracle alias_build of all rows + walk_node2vec_reject of the whole batch"
+        dt = time.perf_counter() - t0
+        cpu = {"value": osampled / dt, "unit": "edges/s", "cores": orc.num_threads(), "cpu": cpu_model(), "kind": "port",
+               "compiler_flags": oracle_flags(),
+               "sample": "%s: %d sampled edges in %.3f s" % (what_cpu, osampled, dt)}
     print(json.dumps({
         "metric": METRIC, "metric_detail": "value = sampled edges per second of one whole batch (tables built on the way)",
         "value": sampled / wall, "unit": "edges/s", "n_gpus": 1,
@@ -123,7 +241,7 @@ def online_bench(args, cfg, capi, g, seeds, name, cus, t_gen, torch):
                                (args.config, cfg["scale"], cfg["ef"], g.V, g.E, cfg["wkind"], what, N),
                    "device": name, "compute_units": cus, "graph_generation_s": t_gen},
         "sampled_edges": sampled, "kernel_region_ms": ksec * 1e3, "seps_kernel_region": sampled / ksec,
-        "roofline": None, "cpu_baseline": None}))
+        "roofline": roofline, "cpu_baseline": cpu}))
 
 
 def main():
@@ -133,6 +251,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--config", default="c5", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--profile-steps", type=int, default=3,
+                    help="untimed steps after the timed ones, run with per-kernel HIP events for the roofline")
     ap.add_argument("--n2v-table", action="store_true",
                     help="config c4: build the second-order table of every (walker, step) instead of rejection sampling")
     ap.add_argument("--calibrate", action="store_true",
@@ -148,7 +268,6 @@ def main():
     import numpy as np
 
     cfg = CONFIGS[args.config]
-    capi.set_option("build_profile", 1)  # HIP events between the build kernels: the roofline needs each one's duration
     if args.calibrate:
         words = 1 << 28
         a = capi.DeviceArray(words, np.uint32, fill=1)
@@ -175,12 +294,9 @@ def main():
         torch.cuda.synchronize()
         capi.synchronize()
 
-    rec = []
-
     def step():
         r = {}
         r["build_s"] = g.build_tables()
-        r["profile"] = g.build_profile()
         _, _, r["walk_edges"], r["walk_s"] = g.walk_offline(seeds, L, 0.0, cfg["seed"], out=(paths, lengths))
         if cfg["ppr"]:
             _, _, r["ppr_edges"], r["ppr_s"] = g.walk_offline(seeds, 100, 0.15, cfg["seed"] + 1,
@@ -190,6 +306,7 @@ def main():
     for _ in range(args.warmup):
         step()
     sync()
+    rec = []
     t0 = time.perf_counter()
     for _ in range(args.steps):
         rec.append(step())
@@ -197,19 +314,37 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
 
+    # per-kernel brackets of the build: extra steps, outside the timed region
+    prof = {}
+    psteps = max(1, args.profile_steps)
+    capi.set_option("build_profile", 1)
+    for _ in range(psteps):
+        g.build_tables()
+        for nm, ms, edges in g.build_profile():
+            p = prof.setdefault(nm, [0.0, edges])
+            p[0] += ms / psteps
+    capi.set_option("build_profile", 0)
+
     mean = lambda k: sum(r[k] for r in rec) / len(rec)
     build_s, walk_s, walk_edges = mean("build_s"), mean("walk_s"), rec[-1]["walk_edges"]
     work = E + walk_edges + (rec[-1]["ppr_edges"] if cfg["ppr"] else 0)
     build_bytes = 12 * E + 5 * V
-    # dominant kernel of the step, from the per-kernel HIP-event brackets of the build
-    prof = {}
-    for r in rec:
-        for nm, ms, edges in r["profile"]:
-            p = prof.setdefault(nm, [0.0, edges])
-            p[0] += ms / len(rec)
     dom = max((k for k in prof if prof[k][1] > 0), key=lambda k: prof[k][0])  # brackets without edges are host round trips
     dom_ms, dom_edges = prof[dom]
-    dom_bytes = BYTES_PER_EDGE.get(dom, 12) * dom_edges
+    # the binning pass reads xadj twice (8 bytes per vertex) and builds the rows of one or two entries
+    dom_bytes = BYTES_PER_EDGE.get(dom, 12) * dom_edges + (8 * V if dom == "bin" else 0)
+    # measured HBM traffic: only when the tracked table was made for the kernels that ran here
+    traffic_tab, traffic_head = load_traffic()
+    ran = sorted(KERNEL_OF.get(k, k) for k in prof)
+    traffic, walk_traffic, traffic_src = None, None, None
+    if traffic_tab is not None and args.config == "c5":
+        listed = sorted(k for k in traffic_tab if k != "walk_offline_kernel")
+        if listed == ran:
+            traffic = traffic_tab[KERNEL_OF.get(dom, dom)] * dom_edges
+            walk_traffic = traffic_tab.get("walk_offline_kernel")
+            traffic_src = "profiles/c5_kernel_traffic.txt (commit %s)" % traffic_head.get("commit", "?")
+        else:
+            traffic_src = "profiles/c5_kernel_traffic.txt lists other kernels than ran: not used"
     out = {
         "metric": METRIC,
         "metric_detail": "value = (alias-table entries built + walk steps sampled) per second of one whole step "
@@ -224,17 +359,17 @@ def main():
                    "device": name, "compute_units": cus, "graph_generation_s": t_gen},
         "build": {"edges_per_s": E / build_s, "ms": build_s * 1e3, "algorithmic_bytes": build_bytes,
                   "hbm_frac": build_bytes / build_s / HBM_PEAK,
+                  "kernels_from": "%d untimed steps with per-kernel HIP events after the timed steps" % psteps,
                   "kernels": {KERNEL_OF.get(k, k): {"ms": round(v[0], 4), "edges": v[1],
                                                     "GBps": round(BYTES_PER_EDGE.get(k, 12) * v[1] / (v[0] * 1e-3) / 1e9, 1) if v[0] > 0 else 0}
                               for k, v in prof.items()}},
         "walk": {"seps": walk_edges / walk_s, "ms": walk_s * 1e3, "steps": walk_edges,
                  "algorithmic_bytes": 24 * walk_edges, "hbm_frac": 24 * walk_edges / walk_s / HBM_PEAK,
-                 # every step gathers three 128-byte lines (xadj, table entry, adjncy): measured 399 B/step
-                 "measured_traffic_bytes_per_step": WALK_TRAFFIC_PER_STEP,
-                 "hbm_frac_measured_traffic": WALK_TRAFFIC_PER_STEP * walk_edges / walk_s / HBM_PEAK},
+                 "measured_traffic_bytes_per_step": walk_traffic,
+                 "hbm_frac_measured_traffic": (walk_traffic * walk_edges / walk_s / HBM_PEAK) if walk_traffic else None},
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF.get(dom, dom), "achieved": dom_bytes / (dom_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK,
-                     "traffic": TRAFFIC_PER_EDGE[dom] * dom_edges if dom in TRAFFIC_PER_EDGE else None,
+                     "traffic": traffic, "traffic_source": traffic_src,
                      "launch_ms": dom_ms, "algorithmic_bytes_per_launch": dom_bytes},
     }
     if cfg["ppr"]:
@@ -242,7 +377,7 @@ def main():
         out["ppr"] = {"seps": ppr_edges / ppr_s, "ms": ppr_s * 1e3, "steps": ppr_edges}
     if not args.no_cpu:
         from oracle import orc
-        out["cpu_baseline"] = cpu_baseline(capi, orc, g, cfg, seeds)
+        out["cpu_baseline"] = cpu_baseline_offline(capi, orc, g, cfg, seeds)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -154,6 +154,11 @@ class Graph:
         _ck(lib().sky_graph_download(self.h, _p(xadj), _p(adjncy), _p(w)))
         return xadj, adjncy, w
 
+    def download_xadj(self):
+        xadj = np.empty(self.V + 1, np.uint32)
+        _ck(lib().sky_graph_download(self.h, _p(xadj), None, None))
+        return xadj
+
     def build_tables(self):
         """ConstructTable: returns the kernel-region seconds."""
         sec = C.c_double(0)

@@ -310,7 +310,7 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
                                                           const float* __restrict__ wgt,
                                                           const uint32_t* __restrict__ src, uint32_t n,
                                                           uint32_t per_block,
-                                                          const uint32_t* __restrict__ class_start,
+                                                          const uint32_t* __restrict__ counts,
                                                           const uint32_t* __restrict__ blk_off,
                                                           RowRef* __restrict__ vlist,
                                                           AliasEntry* __restrict__ table,
@@ -318,8 +318,11 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
   __shared__ uint32_t s_cur[CLS_COUNT];
   __shared__ uint2 s_tiny[4][64 * BIN_ITEMS];  // per wavefront: {offset, vertex} of its rows of 1..2 entries
   __shared__ uint8_t s_tiny_d[4][64 * BIN_ITEMS];
-  if (threadIdx.x < CLS_COUNT)
-    s_cur[threadIdx.x] = class_start[threadIdx.x] + blk_off[blockIdx.x * CLS_COUNT + threadIdx.x];
+  if (threadIdx.x < CLS_COUNT) {  // the class lists lie back to back in class order
+    uint32_t start = 0;
+    for (uint32_t c = 0; c < threadIdx.x; ++c) start += counts[c];
+    s_cur[threadIdx.x] = start + blk_off[blockIdx.x * CLS_COUNT + threadIdx.x];
+  }
   __syncthreads();
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
@@ -919,7 +922,7 @@ constexpr size_t COUNTER_BYTES = 2 * CLS_COUNT * 4 + CLS_COUNT * 8;
 
 struct BuildScratch {
   RowRef* vlist = nullptr;       // [vcap]
-  uint32_t* counters = nullptr;  // [2*CLS_COUNT] counts then class starts, then CLS_COUNT 64-bit edge totals
+  uint32_t* counters = nullptr;  // [2*CLS_COUNT] class counts (the second half is unused), then CLS_COUNT 64-bit edge totals
   uint32_t* blk_cnt = nullptr;   // [BIN_BLOCKS * CLS_COUNT] class counts of every binning block, then their prefixes
   uint64_t* huge_off = nullptr;  // [huge_cap + 1], last = total
   uint64_t* huge_scratch = nullptr;
@@ -944,9 +947,40 @@ void set_build_profile(bool on) { g_build_profile = on; }
 void set_stream_min_edges(uint64_t n) { g_stream_min_edges = n; }
 void set_row_merge(bool on) { g_row_merge = on; }
 
+EventTimer::EventTimer(sky_graph* g) : stream(g->stream), pooled(g->ev), npooled(2) {}
+
+int pool_get(sky_graph* g, int slot, size_t bytes, void** out) {
+  sky_graph::PoolBuf& b = g->pool[slot];
+  if (b.cap < bytes) {
+    if (b.p) SKY_HIP(hipFree(b.p));
+    b.p = nullptr;
+    b.cap = 0;
+    SKY_HIP(hipMalloc(&b.p, bytes + 16));
+    b.cap = bytes;
+  }
+  *out = b.p;
+  return SKY_OK;
+}
+void pool_release(sky_graph* g) {
+  for (auto& b : g->pool) {
+    if (b.p) (void)hipFree(b.p);
+    b.p = nullptr;
+    b.cap = 0;
+  }
+  for (hipEvent_t& e : g->ev) {
+    if (e) (void)hipEventDestroy(e);
+    e = nullptr;
+  }
+}
+
 int EventTimer::mark(const char* name, uint64_t e) {
   hipEvent_t x;
-  SKY_HIP(hipEventCreate(&x));
+  if (ev.size() < npooled) {
+    if (!pooled[ev.size()]) SKY_HIP(hipEventCreate(&pooled[ev.size()]));
+    x = pooled[ev.size()];
+  } else {
+    SKY_HIP(hipEventCreate(&x));
+  }
   SKY_HIP(hipEventRecord(x, stream));
   ev.push_back(x);
   names.push_back(name);
@@ -968,7 +1002,7 @@ int EventTimer::finish(std::vector<sky_graph::ProfileEntry>* profile, double* se
   return SKY_OK;
 }
 EventTimer::~EventTimer() {
-  for (hipEvent_t e : ev) (void)hipEventDestroy(e);
+  for (size_t i = npooled; i < ev.size(); ++i) (void)hipEventDestroy(ev[i]);
 }
 
 int ensure_table_storage(sky_graph* g) {
@@ -1020,17 +1054,33 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n, per_block, sc.blk_cnt,
                        reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
     hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(64), 0, st, sc.blk_cnt, blocks, sc.counters);
-    SKY_HIP(hipMemcpyAsync(&host, sc.counters, COUNTER_BYTES, hipMemcpyDeviceToHost, st));
-    SKY_HIP(hipStreamSynchronize(st));
+    hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n, per_block,
+                       sc.counters, sc.blk_cnt, sc.vlist, g->table, g->valid);
+    // The class sizes decide the launches that follow.  Those of all vertices depend on xadj alone and are kept
+    // with the graph after the first time; any other list of rows is waited for.
+    const bool all_rows = src == nullptr && n == g->V;
+    if (all_rows && g->bin_known) {
+      for (int c = 0; c < CLS_COUNT; ++c) {
+        host.counts[c] = g->bin_counts[c];
+        host.edges[c] = g->bin_edges[c];
+      }
+    } else {
+      SKY_HIP(hipMemcpyAsync(&host, sc.counters, COUNTER_BYTES, hipMemcpyDeviceToHost, st));
+      SKY_HIP(hipStreamSynchronize(st));
+      if (all_rows) {
+        for (int c = 0; c < CLS_COUNT; ++c) {
+          g->bin_counts[c] = host.counts[c];
+          g->bin_edges[c] = host.edges[c];
+        }
+        g->bin_known = true;
+      }
+    }
     for (int c = 0; c < CLS_COUNT; ++c) counts[c] = host.counts[c];
     uint32_t acc = 0;
     for (int c = 0; c < CLS_COUNT; ++c) {
       starts[c] = acc;
       acc += counts[c];
     }
-    SKY_HIP(hipMemcpyAsync(sc.counters + CLS_COUNT, starts, sizeof(starts), hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n, per_block,
-                       sc.counters + CLS_COUNT, sc.blk_cnt, sc.vlist, g->table, g->valid);
   }
   if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
   RowRef* const vlist = sc.vlist;
@@ -1163,7 +1213,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
 int build_all_tables(sky_graph* g, double* seconds) {
   SKY_TRY(ensure_table_storage(g));
   SKY_TRY(prepare_build_scratch(g->V));
-  EventTimer tm(g->stream);
+  EventTimer tm(g);
   SKY_TRY(tm.mark("start", 0));
   if (g_build_profile) {
     SKY_TRY(build_rows(g, nullptr, g->V, &tm));

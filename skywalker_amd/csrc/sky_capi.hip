@@ -185,6 +185,7 @@ int sky_graph_free(sky_graph* g) {
   void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->table, g->valid};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
+  pool_release(g);
   delete g;
   return SKY_OK;
 }

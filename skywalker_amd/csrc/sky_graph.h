@@ -23,6 +23,22 @@ struct sky_graph {
     uint64_t edges;
   };
   std::vector<ProfileEntry> build_profile;
+
+  // Device buffers that calls on this graph reuse instead of allocating each time (they only grow), and the two
+  // events that bracket a call's kernel region.
+  enum PoolSlot { POOL_COUNTERS = 0, POOL_BITMAP, POOL_LIST, POOL_SLOTS };
+  struct PoolBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+  };
+  PoolBuf pool[POOL_SLOTS];
+  hipEvent_t ev[2] = {nullptr, nullptr};
+
+  // Class sizes of the last binning of all vertices.  They depend on xadj alone, which never changes, so a
+  // later build of all vertices sizes its launches from them without waiting for the device.
+  bool bin_known = false;
+  uint32_t bin_counts[32] = {0};
+  unsigned long long bin_edges[32] = {0};
 };
 
 namespace sky {
@@ -60,13 +76,19 @@ struct EventTimer {
   std::vector<hipEvent_t> ev;
   std::vector<const char*> names;
   std::vector<uint64_t> edges;
+  hipEvent_t* pooled = nullptr;  // events that exist already are used first and are not destroyed
+  size_t npooled = 0;
   explicit EventTimer(hipStream_t s) : stream(s) {}
+  EventTimer(sky_graph* g);  // on the graph's stream, with the graph's two events for the first two marks
   ~EventTimer();
   int mark(const char* name, uint64_t edges);
   // synchronises, then fills `profile` (may be null) and the time from first to last mark
   int finish(std::vector<sky_graph::ProfileEntry>* profile, double* seconds);
 };
 
+// A device buffer of at least `bytes` bytes that belongs to the graph; its contents do not survive a larger request.
+int pool_get(sky_graph* g, int slot, size_t bytes, void** out);
+void pool_release(sky_graph* g);
 int ensure_table_storage(sky_graph* g);
 int prepare_build_scratch(uint32_t max_rows);
 int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm);

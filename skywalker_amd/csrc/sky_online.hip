@@ -115,21 +115,15 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
   unsigned long long* d_sampled = nullptr;
   uint32_t *bitmap = nullptr, *list = nullptr, *d_cnt = nullptr;
   const uint32_t words = (g->V + 31) / 32;
-  auto cleanup = [&]() {
-    if (d_sampled) (void)hipFree(d_sampled);
-    if (bitmap) (void)hipFree(bitmap);
-    if (list) (void)hipFree(list);
-    if (d_cnt) (void)hipFree(d_cnt);
-  };
   auto body = [&]() -> int {
     SKY_TRY(ensure_table_storage(g));
     SKY_TRY(prepare_build_scratch(std::min(N, g->V)));
-    SKY_HIP(hipMalloc((void**)&d_sampled, 8));
-    SKY_HIP(hipMalloc((void**)&bitmap, (size_t)words * 4 + 16));
-    SKY_HIP(hipMalloc((void**)&list, (size_t)std::min(N, g->V) * 4 + 16));
-    SKY_HIP(hipMalloc((void**)&d_cnt, 8));
+    SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
+    d_cnt = reinterpret_cast<uint32_t*>(d_sampled + 1);
+    SKY_TRY(pool_get(g, sky_graph::POOL_BITMAP, (size_t)words * 4, (void**)&bitmap));
+    SKY_TRY(pool_get(g, sky_graph::POOL_LIST, (size_t)std::min(N, g->V) * 4, (void**)&list));
     SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
-    EventTimer tm(st);
+    EventTimer tm(g);
     SKY_TRY(tm.mark("start", 0));
     const uint32_t blocks = (N + 255) / 256;
     if (N) {
@@ -157,9 +151,7 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
     if (sampled) *sampled = h;
     return SKY_OK;
   };
-  const int rc = body();
-  cleanup();
-  return rc;
+  return body();
 }
 
 // ---------------------------------------------------------------- node2vec
@@ -392,9 +384,9 @@ int walk_online_node2vec(sky_graph* g, float p, float q, const uint32_t* seeds, 
   hipStream_t st = g->stream;
   unsigned long long* d_sampled = nullptr;
   auto body = [&]() -> int {
-    SKY_HIP(hipMalloc((void**)&d_sampled, 8));
+    SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
     SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
-    EventTimer tm(st);
+    EventTimer tm(g);
     SKY_TRY(tm.mark("start", 0));
     if (N) {
       const uint32_t blocks = (N + 255) / 256;
@@ -412,9 +404,7 @@ int walk_online_node2vec(sky_graph* g, float p, float q, const uint32_t* seeds, 
     if (sampled) *sampled = h;
     return SKY_OK;
   };
-  const int rc = body();
-  if (d_sampled) (void)hipFree(d_sampled);
-  return rc;
+  return body();
 }
 
 }  // namespace sky

@@ -120,24 +120,18 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
   unsigned long long* d_sampled = nullptr;
   uint32_t *bitmap = nullptr, *list = nullptr, *d_count = nullptr;
   const uint32_t words = (g->V + 31) / 32;
-  auto cleanup = [&]() {
-    if (d_sampled) (void)hipFree(d_sampled);
-    if (bitmap) (void)hipFree(bitmap);
-    if (list) (void)hipFree(list);
-    if (d_count) (void)hipFree(d_count);
-  };
   auto body = [&]() -> int {
-    SKY_HIP(hipMalloc((void**)&d_sampled, 8));
+    SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
+    d_count = reinterpret_cast<uint32_t*>(d_sampled + 1);
     SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
     if (N && slen) SKY_HIP(hipMemsetAsync(sample_lengths, 0, (size_t)N * slen * 4, st));
     if (online) {
       SKY_TRY(ensure_table_storage(g));
       SKY_TRY(prepare_build_scratch(g->V));
-      SKY_HIP(hipMalloc((void**)&bitmap, (size_t)words * 4 + 16));
-      SKY_HIP(hipMalloc((void**)&list, (size_t)g->V * 4 + 16));
-      SKY_HIP(hipMalloc((void**)&d_count, 4));
+      SKY_TRY(pool_get(g, sky_graph::POOL_BITMAP, (size_t)words * 4, (void**)&bitmap));
+      SKY_TRY(pool_get(g, sky_graph::POOL_LIST, (size_t)g->V * 4, (void**)&list));
     }
-    EventTimer tm(st);
+    EventTimer tm(g);
     SKY_TRY(tm.mark("start", 0));
     if (online) SKY_HIP(hipMemsetAsync(bitmap, 0, (size_t)words * 4, st));
     if (N) hipLaunchKernelGGL(sample_init_kernel, dim3((N + 255) / 256), dim3(256), 0, st, seeds, N, lps, data);
@@ -175,9 +169,7 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
     if (sampled) *sampled = hcount;
     return SKY_OK;
   };
-  const int rc = body();
-  cleanup();
-  return rc;
+  return body();
 }
 
 }  // namespace sky

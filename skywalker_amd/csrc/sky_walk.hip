@@ -61,28 +61,19 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
                  uint32_t* paths, uint32_t* lengths, uint64_t* sampled, double* seconds) {
   hipStream_t st = g->stream;
   unsigned long long* d_sampled = nullptr;
-  SKY_HIP(hipMalloc((void**)&d_sampled, 8));
+  SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
   SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
-  hipEvent_t e0, e1;
-  SKY_HIP(hipEventCreate(&e0));
-  SKY_HIP(hipEventCreate(&e1));
-  SKY_HIP(hipEventRecord(e0, st));
+  EventTimer tm(g);
+  SKY_TRY(tm.mark("start", 0));
   if (N)
     hipLaunchKernelGGL(walk_offline_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st, g->xadj,
                        g->adjncy, g->table, seeds, N, g->V, len, stop_prob, seed, paths, lengths, d_sampled,
                        (unsigned long long*)nullptr);
-  SKY_HIP(hipEventRecord(e1, st));
-  SKY_HIP(hipStreamSynchronize(st));
-  SKY_HIP(hipGetLastError());
-  float ms = 0;
-  SKY_HIP(hipEventElapsedTime(&ms, e0, e1));
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
+  SKY_TRY(tm.mark("walk", 0));
+  SKY_TRY(tm.finish(nullptr, seconds));
   unsigned long long h = 0;
   SKY_HIP(hipMemcpy(&h, d_sampled, 8, hipMemcpyDeviceToHost));
-  SKY_HIP(hipFree(d_sampled));
   if (sampled) *sampled = h;
-  if (seconds) *seconds = ms * 1e-3;
   return SKY_OK;
 }
 
@@ -217,9 +208,9 @@ int walk_node2vec_reject(sky_graph* g, float p, float q, const uint32_t* seeds, 
   const float fmax = fmaxf(1.0f, fmaxf(fp, fq));
   unsigned long long* d_sampled = nullptr;
   auto body = [&]() -> int {
-    SKY_HIP(hipMalloc((void**)&d_sampled, 8));
+    SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
     SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
-    EventTimer tm(st);
+    EventTimer tm(g);
     SKY_TRY(tm.mark("start", 0));
     if (N)
       hipLaunchKernelGGL(walk_n2v_reject_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st,
@@ -235,9 +226,7 @@ int walk_node2vec_reject(sky_graph* g, float p, float q, const uint32_t* seeds, 
     if (seconds) *seconds = sec + build_sec;
     return SKY_OK;
   };
-  const int rc = body();
-  if (d_sampled) (void)hipFree(d_sampled);
-  return rc;
+  return body();
 }
 
 }  // namespace sky
