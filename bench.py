@@ -253,6 +253,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--profile-steps", type=int, default=3,
                     help="untimed steps after the timed ones, run with per-kernel HIP events for the roofline")
+    ap.add_argument("--no-walk-variants", action="store_true",
+                    help="skip the untimed runs of the walk with the walk index and with walker lists")
     ap.add_argument("--n2v-table", action="store_true",
                     help="config c4: build the second-order table of every (walker, step) instead of rejection sampling")
     ap.add_argument("--calibrate", action="store_true",
@@ -325,6 +327,26 @@ def main():
             p[0] += ms / psteps
     capi.set_option("build_profile", 0)
 
+    # the same walks with the optional 16-byte walk index, and with live walkers handed from launch to launch:
+    # outside the timed region, reported beside the default path
+    extras = {}
+    if not args.no_walk_variants:
+        def walk_ms(reps=3):
+            return min(g.walk_offline(seeds, L, 0.0, cfg["seed"], out=(paths, lengths))[3] for _ in range(reps)) * 1e3
+        g.build_tables()
+        base_ms = walk_ms()
+        capi.set_option("walk_compact_every", 16)
+        compact_ms = walk_ms()
+        capi.set_option("walk_compact_every", 0)
+        idx_ms = g.build_walk_index() * 1e3
+        indexed_ms = walk_ms()
+        steps_n = rec[-1]["walk_edges"]
+        extras = {"default_ms": base_ms, "walker_lists_every_16_steps_ms": compact_ms,
+                  "walk_index": {"build_ms": idx_ms, "bytes_per_edge": 16, "walk_ms": indexed_ms,
+                                 "seps": steps_n / (indexed_ms * 1e-3),
+                                 "batches_to_pay_for_the_index": idx_ms / max(base_ms - indexed_ms, 1e-9)}}
+        g.build_tables()  # leaves the graph without a current index, as the timed steps saw it
+
     mean = lambda k: sum(r[k] for r in rec) / len(rec)
     build_s, walk_s, walk_edges = mean("build_s"), mean("walk_s"), rec[-1]["walk_edges"]
     work = E + walk_edges + (rec[-1]["ppr_edges"] if cfg["ppr"] else 0)
@@ -366,7 +388,8 @@ def main():
         "walk": {"seps": walk_edges / walk_s, "ms": walk_s * 1e3, "steps": walk_edges,
                  "algorithmic_bytes": 24 * walk_edges, "hbm_frac": 24 * walk_edges / walk_s / HBM_PEAK,
                  "measured_traffic_bytes_per_step": walk_traffic,
-                 "hbm_frac_measured_traffic": (walk_traffic * walk_edges / walk_s / HBM_PEAK) if walk_traffic else None},
+                 "hbm_frac_measured_traffic": (walk_traffic * walk_edges / walk_s / HBM_PEAK) if walk_traffic else None,
+                 "variants": extras},
         "roofline": {"bound": "hbm", "kernel": KERNEL_OF.get(dom, dom), "achieved": dom_bytes / (dom_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK,
                      "traffic": traffic, "traffic_source": traffic_src,

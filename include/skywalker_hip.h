@@ -121,6 +121,15 @@ int sky_walk_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uin
                      uint64_t philox_seed, uint32_t* paths_device, uint32_t* lengths_device, uint64_t* sampled,
                      double* seconds);
 
+/* ---- optional index for the walks on prebuilt tables (no counterpart in the reference, whose walk kernels gather
+ *      prob_array, alias_array and adjncy separately, src/offline_walk.cu:100-120): one 16-byte entry per CSR slot,
+ *      {prob, alias, neighbour of the slot, neighbour of its alias slot}, so that a step reads two cache lines
+ *      (xadj, entry) instead of three.  Costs 16 bytes per edge of device memory and one pass over the tables;
+ *      sky_walk_offline, sky_walk_offline_noalloc and the walks that end in them use it while it is current.  Any
+ *      call that rewrites table entries (sky_alias_build_all, sky_alias_upload, the online modes) makes it stale:
+ *      it is then ignored until it is built again.  Paths are the same with and without it. ---- */
+int sky_walk_index_build(sky_graph* g, double* seconds);
+
 /* ---- sky_walk_offline for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses
  *      that forbid hipMalloc).  No counterpart in the reference.  Same kernel, same paths and lengths; the
  *      per-workgroup counts of sampled edges go to a static device array of the library (128 KiB per GPU, held
@@ -177,7 +186,11 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      sky_last_build_profile (about 3 microseconds each; a small graph pays 20 % of its build for them).
  *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:
  *      0 builds, before every step, the rows the walkers stand on; 1 builds every row first and walks as
- *      sky_walk_offline does; -1 takes whichever is estimated to be faster.  The paths are the same. ---- */
+ *      sky_walk_offline does; -1 takes whichever is estimated to be faster.  The paths are the same.
+ *      "walk_compact_every" (default 0): k > 0 makes sky_walk_offline run k steps per launch and hand the next
+ *      launch the list of walkers that are still walking (the reference's walker queue,
+ *      include/sampler_result.cuh:646-669), so that walkers that have stopped no longer hold a lane; 0 keeps every
+ *      walker on its lane for the whole walk in one launch.  The paths are the same. ---- */
 int sky_set_option(const char* name, long value);
 
 /* ---- per-kernel timing of the last sky_alias_build_all on this graph, for roofline reporting:

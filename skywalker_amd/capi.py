@@ -22,7 +22,7 @@ EXPORTS = [
     "sky_device_fill_u32", "sky_device_copy_u32", "sky_device_synchronize", "sky_device_name", "sky_graph_upload",
     "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
     "sky_alias_build_all", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
-    "sky_walk_offline_noalloc",
+    "sky_walk_offline_noalloc", "sky_walk_index_build",
     "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_philox_selftest",
     "sky_last_build_profile", "sky_set_option",
 ]
@@ -206,6 +206,12 @@ class Graph:
     def walk_offline(self, seeds, length, stop_prob, seed, out=None):
         """OfflineWalk: returns (paths DeviceArray, lengths DeviceArray, sampled, seconds)."""
         return self._walk(lib().sky_walk_offline, (), seeds, length, stop_prob, seed, out)
+
+    def build_walk_index(self):
+        """sky_walk_index_build: returns the kernel-region seconds."""
+        sec = C.c_double(0)
+        _ck(lib().sky_walk_index_build(self.h, C.byref(sec)))
+        return sec.value
 
     def walk_offline_noalloc(self, seeds_d, length, stop_prob, seed, paths, lengths, sampled_d):
         """sky_walk_offline_noalloc: every buffer is the caller's; enqueues and returns (synchronize() before reading)."""

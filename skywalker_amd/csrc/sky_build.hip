@@ -1038,6 +1038,7 @@ int prepare_build_scratch(uint32_t max_rows) {
 // prepare_build_scratch(n) and ensure_table_storage must have been called.
 int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   hipStream_t st = g->stream;
+  g->has_walk_index = false;  // the table entries it was made from are about to change
   BuildScratch& sc = g_scratch;
   uint32_t counts[CLS_COUNT] = {0}, starts[CLS_COUNT] = {0};
   struct {

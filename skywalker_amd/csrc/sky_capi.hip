@@ -182,7 +182,7 @@ int sky_graph_device_ptrs(const sky_graph* g, const uint32_t** xadj, const uint3
 
 int sky_graph_free(sky_graph* g) {
   if (!g) return SKY_OK;
-  void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->table, g->valid};
+  void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->table, g->valid, g->walk_index};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   pool_release(g);
@@ -251,6 +251,7 @@ int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, con
   }
   if (g->V) SKY_HIP(hipMemcpy(g->valid, valid, (size_t)g->V, hipMemcpyHostToDevice));
   g->has_tables = true;
+  g->has_walk_index = false;
   return SKY_OK;
 }
 
@@ -276,6 +277,12 @@ int sky_walk_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uin
   SKY_TRY(check_walk_args("sky_walk_offline", g, seeds_device, N, len, stop_prob, paths_device, lengths_device));
   if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_walk_offline: alias tables have not been built");
   return walk_offline(g, seeds_device, N, len, stop_prob, philox_seed, paths_device, lengths_device, sampled, seconds);
+}
+
+int sky_walk_index_build(sky_graph* g, double* seconds) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_walk_index_build: null graph");
+  if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_walk_index_build: alias tables have not been built");
+  return build_walk_index(g, seconds);
 }
 
 int sky_walk_offline_noalloc(sky_graph* g, const uint32_t* seeds_device, uint32_t N, uint32_t len, float stop_prob,
@@ -365,6 +372,11 @@ int sky_set_option(const char* name, long value) {
   }
   if (!strcmp(name, "build_profile")) {
     set_build_profile(value != 0);
+    return SKY_OK;
+  }
+  if (!strcmp(name, "walk_compact_every")) {
+    if (value < 0) return fail(SKY_ERR_ARG, "sky_set_option: walk_compact_every must be >= 0");
+    set_walk_compact_every((uint32_t)value);
     return SKY_OK;
   }
   if (!strcmp(name, "online_full_build")) {

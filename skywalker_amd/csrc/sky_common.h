@@ -250,6 +250,13 @@ struct AliasEntry {
   float prob;
   uint32_t alias;
 };
+// Entry of the optional walk index: the table entry of a slot together with the neighbour ids of the slot
+// itself and of its alias slot, so that a step needs no gather from the adjacency array.
+struct WalkEntry {
+  float prob;
+  uint32_t alias;
+  uint32_t nbr_col, nbr_alias;
+};
 // Four consecutive entries starting at a 32-byte aligned slot, as two 16-byte stores.
 __device__ __forceinline__ void store_entries4(AliasEntry* t, const float (&p)[4], const uint32_t (&a)[4]) {
   uint4* o = reinterpret_cast<uint4*>(t);

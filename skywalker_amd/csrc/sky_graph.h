@@ -15,6 +15,10 @@ struct sky_graph {
   sky::AliasEntry* table = nullptr;  // [E] {prob, alias}
   int8_t* valid = nullptr;    // [V]
   bool has_tables = false;
+  // optional walk index: one 16-byte entry per CSR slot that also holds the two neighbour ids a draw can
+  // lead to; null unless sky_walk_index_build has run since the tables were last written
+  sky::WalkEntry* walk_index = nullptr;  // [E] storage, kept once allocated
+  bool has_walk_index = false;           // its contents match the tables
   hipStream_t stream = nullptr;  // null stream, like the reference ("0 stream everywhere")
 
   struct ProfileEntry {
@@ -104,6 +108,8 @@ void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);
 void set_build_profile(bool on);
 void set_online_full_build(int mode);
+void set_walk_compact_every(uint32_t steps);
+int build_walk_index(sky_graph* g, double* seconds);
 uint32_t tiled_max_tiles();
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
                  uint32_t* paths, uint32_t* lengths, uint64_t* sampled, double* seconds);

@@ -12,39 +12,113 @@
 namespace sky {
 
 constexpr int WALK_BLOCK = 256;
+constexpr int WALK_STAGE = 4;  // steps whose vertices leave together as one 16-byte store
 
+typedef uint32_t path4u __attribute__((ext_vector_type(4), aligned(4)));
+
+// One draw from the row of v.  With the walk index one 16-byte entry holds both possible next vertices (two
+// cache lines per step: xadj and the entry); without it the neighbour id is a third gather.
+template <bool INDEXED>
+__device__ __forceinline__ bool walk_draw(const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
+                                          const AliasEntry* __restrict__ table, const WalkEntry* __restrict__ index,
+                                          const u32x4& r, uint32_t v, uint32_t& next) {
+  const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
+  if (deg == 0) return false;
+  const uint32_t col = __umulhi(r.x, deg);
+  if (INDEXED) {
+    const WalkEntry e = index[off + col];
+    const bool keep = u24(r.y) < e.prob;
+    if (!keep && e.alias == SKY_INVALID) return false;
+    next = keep ? e.nbr_col : e.nbr_alias;
+  } else {
+    const AliasEntry e = table[off + col];
+    const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
+    if (cand == SKY_INVALID) return false;
+    next = adjncy[off + cand];
+  }
+  return true;
+}
+
+// Steps [s_begin, s_end) of the walkers listed in `live` (null: walkers 0..n_live-1, which then also record
+// their start vertex).  A walker that is still walking at s_end is appended to `next_live` when that list is
+// given: the next launch then runs on full wavefronts again (walkers that reached a vertex without out-edges
+// or stopped no longer hold a lane).  The vertices of WALK_STAGE steps leave as one store.
+template <bool INDEXED>
 __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
-    const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
-    const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t V, uint32_t len,
-    float stop_prob, uint64_t seed, uint32_t* __restrict__ paths, uint32_t* __restrict__ lengths,
-    unsigned long long* __restrict__ sampled, unsigned long long* __restrict__ block_partials) {
+    const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy, const AliasEntry* __restrict__ table,
+    const WalkEntry* __restrict__ index, const uint32_t* __restrict__ seeds, const uint32_t* __restrict__ live,
+    const uint32_t* __restrict__ n_live_dev, uint32_t n_live, uint32_t V, uint32_t len, uint32_t s_begin,
+    uint32_t s_end, float stop_prob, uint64_t seed, uint32_t* __restrict__ paths, uint32_t* __restrict__ lengths,
+    uint32_t* __restrict__ next_live, uint32_t* __restrict__ n_next, unsigned long long* __restrict__ sampled,
+    unsigned long long* __restrict__ block_partials) {
   __shared__ unsigned long long s_part[WALK_BLOCK / 64];
-  const uint32_t i = blockIdx.x * WALK_BLOCK + threadIdx.x;
-  uint32_t s = 0;
-  if (i < N) {
+  const uint32_t t = blockIdx.x * WALK_BLOCK + threadIdx.x;
+  if (n_live_dev) n_live = min(n_live, *n_live_dev);  // the list's length is only known on the device
+  uint32_t steps = 0;
+  bool walking = false;
+  uint32_t i = 0;
+  if (t < n_live) {
+    i = live ? live[t] : t;
     uint32_t* path = paths + (size_t)i * (len + 1);
-    uint32_t v = seeds[i];
-    path[0] = v;
-    for (; s < len && v < V; ++s) {  // a start vertex that does not exist is recorded and never left
-      const u32x4 r = philox(seed, i, s, 0, DOM_WALK);
-      if (stop_prob > 0.0f && u24(r.z) < stop_prob) break;
-      const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
-      if (deg == 0) break;
-      const uint32_t col = __umulhi(r.x, deg);
-      const AliasEntry e = table[off + col];
-      const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
-      if (cand == SKY_INVALID) break;
-      v = adjncy[off + cand];
-      path[s + 1] = v;
+    uint32_t v;
+    if (s_begin == 0) {
+      v = seeds[i];
+      path[0] = v;
+    } else {
+      v = path[s_begin];
     }
-    lengths[i] = s;
+    uint32_t s = s_begin;
+    walking = v < V;  // a start vertex that does not exist is recorded and never left
+    while (walking && s < s_end) {
+      uint32_t b[WALK_STAGE];
+      uint32_t got = 0;
+#pragma unroll
+      for (int k = 0; k < WALK_STAGE; ++k) {
+        b[k] = 0;
+        if (walking && s + got < s_end) {
+          const u32x4 r = philox(seed, i, s + got, 0, DOM_WALK);
+          uint32_t nx = 0;
+          if ((stop_prob > 0.0f && u24(r.z) < stop_prob) || !walk_draw<INDEXED>(xadj, adjncy, table, index, r, v, nx)) {
+            walking = false;
+          } else {
+            v = nx;
+            b[k] = nx;
+            got = k + 1;
+          }
+        }
+      }
+      uint32_t* dst = path + s + 1;
+      if (got == WALK_STAGE) {
+        path4u o;
+        o.x = b[0]; o.y = b[1]; o.z = b[2]; o.w = b[3];
+        *reinterpret_cast<path4u*>(dst) = o;
+      } else {
+#pragma unroll
+        for (int k = 0; k < WALK_STAGE - 1; ++k)
+          if ((uint32_t)k < got) dst[k] = b[k];
+      }
+      s += got;
+    }
+    steps = s - s_begin;
+    if (!walking || s_end == len) lengths[i] = s;
+    walking = walking && s_end < len;
+  }
+  if (next_live) {  // survivors, one atomic per wavefront
+    const unsigned long long m = __ballot(walking);
+    if (m) {
+      const int lane = threadIdx.x & 63;
+      uint32_t base = 0;
+      if (lane == __ffsll((long long)m) - 1) base = atomicAdd(n_next, (uint32_t)__popcll(m));
+      base = (uint32_t)__shfl((int)base, __ffsll((long long)m) - 1, 64);
+      if (walking) next_live[base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = i;
+    }
   }
   // exact 64-bit count of sampled edges (the reference reduces lengths through float, sampler_result.cuh:57-67)
-  unsigned long long t = s;
+  unsigned long long tot = steps;
 #pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) t += shfl_xor_u64(t, m);
+  for (int m = 32; m >= 1; m >>= 1) tot += shfl_xor_u64(tot, m);
   if (block_partials) {  // one sum per workgroup, added up by reduce_partials_kernel: no counter to clear
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = t;
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = tot;
     __syncthreads();
     if (threadIdx.x == 0) {
       unsigned long long b = 0;
@@ -52,9 +126,22 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
       for (int w = 0; w < WALK_BLOCK / 64; ++w) b += s_part[w];
       block_partials[blockIdx.x] = b;
     }
-  } else if ((threadIdx.x & 63) == 0 && t) {
-    atomicAdd(sampled, t);
+  } else if ((threadIdx.x & 63) == 0 && tot) {
+    atomicAdd(sampled, tot);
   }
+}
+
+static uint32_t g_walk_compact_every = 0;  // 0: one launch, every walker keeps its lane for the whole walk
+void set_walk_compact_every(uint32_t steps) { g_walk_compact_every = steps; }
+
+template <bool INDEXED>
+static void launch_walk(sky_graph* g, const uint32_t* seeds, const uint32_t* live, const uint32_t* n_live_dev,
+                        uint32_t n_live, uint32_t len, uint32_t s_begin, uint32_t s_end, float stop_prob, uint64_t seed,
+                        uint32_t* paths, uint32_t* lengths, uint32_t* next_live, uint32_t* n_next,
+                        unsigned long long* sampled, unsigned long long* partials) {
+  hipLaunchKernelGGL(walk_offline_kernel<INDEXED>, dim3((n_live + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0,
+                     g->stream, g->xadj, g->adjncy, g->table, INDEXED ? g->walk_index : nullptr, seeds, live, n_live_dev, n_live, g->V, len,
+                     s_begin, s_end, stop_prob, seed, paths, lengths, next_live, n_next, sampled, partials);
 }
 
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
@@ -62,18 +149,111 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   hipStream_t st = g->stream;
   unsigned long long* d_sampled = nullptr;
   SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
+  const uint32_t every = g_walk_compact_every;
+  const bool segmented = every > 0 && every < len && N > 0;
+  const uint32_t nseg = segmented ? (len + every - 1) / every : 1;
+  uint32_t *lists = nullptr, *counts = nullptr;
+  if (segmented) {  // two lists of walker numbers used in turn, one survivor count per segment
+    SKY_TRY(pool_get(g, sky_graph::POOL_LIST, (size_t)2 * N * 4, (void**)&lists));
+    SKY_TRY(pool_get(g, sky_graph::POOL_BITMAP, (size_t)(nseg + 1) * 4, (void**)&counts));
+    SKY_HIP(hipMemsetAsync(counts, 0, (size_t)(nseg + 1) * 4, st));
+  }
   SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
   EventTimer tm(g);
   SKY_TRY(tm.mark("start", 0));
-  if (N)
-    hipLaunchKernelGGL(walk_offline_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st, g->xadj,
-                       g->adjncy, g->table, seeds, N, g->V, len, stop_prob, seed, paths, lengths, d_sampled,
-                       (unsigned long long*)nullptr);
+  auto run = [&](auto... a) {
+    if (g->has_walk_index) launch_walk<true>(g, a...);
+    else launch_walk<false>(g, a...);
+  };
+  if (N && !segmented) {
+    run(seeds, (const uint32_t*)nullptr, (const uint32_t*)nullptr, N, len, 0u, len, stop_prob, seed, paths, lengths,
+        (uint32_t*)nullptr, (uint32_t*)nullptr, d_sampled, (unsigned long long*)nullptr);
+  } else if (N) {
+    for (uint32_t k = 0; k < nseg; ++k) {
+      const uint32_t s0 = k * every, s1 = std::min(len, s0 + every);
+      const uint32_t* in = k ? lists + (size_t)((k - 1) & 1) * N : nullptr;
+      uint32_t* out = s1 < len ? lists + (size_t)(k & 1) * N : nullptr;
+      // the survivors of segment k - 1 are counted in counts[k]; the grid covers all N, blocks past the count leave
+      run(seeds, in, k ? counts + k : (const uint32_t*)nullptr, N, len, s0, s1, stop_prob, seed, paths, lengths, out,
+          counts + k + 1, d_sampled, (unsigned long long*)nullptr);
+    }
+  }
   SKY_TRY(tm.mark("walk", 0));
   SKY_TRY(tm.finish(nullptr, seconds));
   unsigned long long h = 0;
   SKY_HIP(hipMemcpy(&h, d_sampled, 8, hipMemcpyDeviceToHost));
   if (sampled) *sampled = h;
+  return SKY_OK;
+}
+
+// ---------------------------------------------------------------- walk index
+// Optional 16-byte entries {prob, alias, neighbour of this slot, neighbour of the alias slot} beside the 8-byte
+// table: a step then reads one entry and needs no gather from adjncy.  Built from the finished tables by one pass
+// over the slots; a tile of 1024 slots finds its rows through the row that holds the tile's first slot.
+constexpr uint32_t IDX_TILE = 1024;
+constexpr uint32_t IDX_ROWS = 4096;  // row offsets of a tile kept in LDS; tiles that span more rows search xadj itself
+
+__global__ __launch_bounds__(256) void index_tile_rows_kernel(const uint32_t* __restrict__ xadj, uint32_t V,
+                                                              uint32_t* __restrict__ row_of_tile) {
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  if (v >= V) return;
+  const uint32_t lo = xadj[v], hi = xadj[v + 1];
+  for (uint64_t t = ((uint64_t)lo + IDX_TILE - 1) / IDX_TILE; t * IDX_TILE < hi; ++t) row_of_tile[t] = v;
+}
+
+__global__ __launch_bounds__(256) void index_fill_kernel(const uint32_t* __restrict__ xadj,
+                                                         const uint32_t* __restrict__ adjncy,
+                                                         const AliasEntry* __restrict__ table,
+                                                         const uint32_t* __restrict__ row_of_tile, uint32_t ntiles,
+                                                         uint32_t V, uint32_t E, WalkEntry* __restrict__ index) {
+  __shared__ uint32_t s_x[IDX_ROWS];
+  const uint32_t t = blockIdx.x;
+  const uint32_t v0 = row_of_tile[t], v1 = t + 1 < ntiles ? row_of_tile[t + 1] : V - 1;
+  const uint32_t rows = v1 - v0 + 1;  // rows v0..v1 hold every slot of the tile
+  const bool in_lds = rows <= IDX_ROWS;
+  if (in_lds)
+    for (uint32_t k = threadIdx.x; k < rows; k += 256u) s_x[k] = xadj[v0 + k];
+  __syncthreads();
+  const uint32_t* x = in_lds ? s_x : xadj + v0;
+#pragma unroll
+  for (int k = 0; k < (int)(IDX_TILE / 256); ++k) {
+    const uint32_t i = t * IDX_TILE + k * 256u + threadIdx.x;
+    if (i >= E) continue;
+    // the last row of v0..v1 that starts at or before slot i (rows without entries share their start with the
+    // next row and are passed over)
+    uint32_t lo = 0, n = rows;
+    while (n > 1) {
+      const uint32_t half = n >> 1;
+      lo = x[lo + half] <= i ? lo + half : lo;
+      n -= half;
+    }
+    const uint32_t off = x[lo];
+    const AliasEntry e = table[i];
+    WalkEntry w;
+    w.prob = e.prob;
+    w.alias = e.alias;
+    w.nbr_col = adjncy[i];
+    w.nbr_alias = e.alias == SKY_INVALID ? SKY_INVALID : adjncy[off + e.alias];
+    index[i] = w;
+  }
+}
+
+int build_walk_index(sky_graph* g, double* seconds) {
+  hipStream_t st = g->stream;
+  if (seconds) *seconds = 0;
+  if (!g->walk_index) SKY_TRY(alloc_padded(&g->walk_index, (size_t)g->E));
+  if (g->E == 0) return SKY_OK;
+  const uint32_t ntiles = (g->E + IDX_TILE - 1) / IDX_TILE;
+  uint32_t* row_of_tile = nullptr;
+  SKY_TRY(pool_get(g, sky_graph::POOL_LIST, (size_t)ntiles * 4, (void**)&row_of_tile));
+  EventTimer tm(g);
+  SKY_TRY(tm.mark("start", 0));
+  hipLaunchKernelGGL(index_tile_rows_kernel, dim3((g->V + 255) / 256), dim3(256), 0, st, g->xadj, g->V, row_of_tile);
+  hipLaunchKernelGGL(index_fill_kernel, dim3(ntiles), dim3(256), 0, st, g->xadj, g->adjncy, g->table, row_of_tile,
+                     ntiles, g->V, g->E, g->walk_index);
+  SKY_TRY(tm.mark("index", 0));
+  SKY_TRY(tm.finish(nullptr, seconds));
+  g->has_walk_index = true;
   return SKY_OK;
 }
 
@@ -122,9 +302,14 @@ int walk_offline_noalloc(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32
   unsigned long long* const partials = g_scratch_ptr[dev];
   hipStream_t st = g->stream;
   const uint32_t blocks = (N + WALK_BLOCK - 1) / WALK_BLOCK;
-  if (blocks)
-    hipLaunchKernelGGL(walk_offline_kernel, dim3(blocks), dim3(WALK_BLOCK), 0, st, g->xadj, g->adjncy, g->table, seeds,
-                       N, g->V, len, stop_prob, seed, paths, lengths, (unsigned long long*)nullptr, partials);
+  if (blocks) {
+    if (g->has_walk_index)
+      launch_walk<true>(g, seeds, nullptr, nullptr, N, len, 0u, len, stop_prob, seed, paths, lengths, nullptr, nullptr,
+                        nullptr, partials);
+    else
+      launch_walk<false>(g, seeds, nullptr, nullptr, N, len, 0u, len, stop_prob, seed, paths, lengths, nullptr, nullptr,
+                         nullptr, partials);
+  }
   if (sampled_device)
     hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, blocks,
                        reinterpret_cast<unsigned long long*>(sampled_device));

@@ -237,3 +237,54 @@ def test_start_vertices_that_do_not_exist_never_move(orc):
     want = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, 2.0, 0.5, seeds, 12, 0.05, 9)
     assert np.array_equal(rej[1], want[1]) and np.array_equal(rej[0], want[0]) and rej[2] == want[2]
     assert np.all(off[1][seeds >= V] == 0)
+
+
+@pytest.mark.parametrize("every", [0, 1, 7, 16])
+@pytest.mark.parametrize("indexed", [False, True])
+def test_walk_index_and_walker_lists_give_the_same_paths(orc, indexed, every):
+    # the 16-byte walk index and the hand-over of live walkers between launches change how a walk is run, not what
+    # it finds: DeepWalk and PPR paths, lengths and counts equal the oracle's
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(14, 8, 17)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 17, len(adjncy), 0.0, 2.0)
+    w[xadj[5]:xadj[6]] = 0.0  # a row without weight: walkers that reach it stop there
+    V = len(xadj) - 1
+    seeds = orc.gen_seeds(4, V, 20011)
+    seeds[3] = V + 7
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    prob, alias, _ = g.tables()
+    if indexed:
+        g.build_walk_index()
+    capi.set_option("walk_compact_every", every)
+    try:
+        for length, stop, seed in ((80, 0.0, 5), (100, 0.15, 6), (3, 0.0, 7)):
+            paths, lengths, sampled, _ = g.walk_offline(seeds, length, stop, seed)
+            opaths, olengths, osampled = orc.walk_offline(xadj, adjncy, prob, alias, seeds, length, stop, seed)
+            assert np.array_equal(lengths.to_host(), olengths)
+            assert np.array_equal(paths.to_host((len(seeds), length + 1)), opaths)
+            assert sampled == osampled
+    finally:
+        capi.set_option("walk_compact_every", 0)
+    g.free()
+
+
+def test_walk_index_goes_stale_when_tables_change(orc):
+    # the index is a copy of table entries: a rebuild with other weights must not be walked with the old copy
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 8, 19)
+    w1 = orc.gen_weights(orc.W_UNIFORM, 19, len(adjncy), 1.0, 100.0)
+    w2 = orc.gen_weights(orc.W_LOGNORMAL, 20, len(adjncy), 0.0, 2.0)
+    seeds = orc.gen_seeds(5, len(xadj) - 1, 3000)
+    g = capi.Graph.upload(xadj, adjncy, w1)
+    g.build_tables()
+    g.build_walk_index()
+    p2, a2, v2 = orc.alias_build(xadj, w2)
+    g.upload_tables(p2, a2, v2)
+    paths, lengths, sampled, _ = g.walk_offline(seeds, 30, 0.0, 2)
+    opaths, olengths, osampled = orc.walk_offline(xadj, adjncy, p2, a2, seeds, 30, 0.0, 2)
+    assert np.array_equal(paths.to_host((3000, 31)), opaths) and sampled == osampled
+    g.build_walk_index()
+    paths, lengths, sampled, _ = g.walk_offline(seeds, 30, 0.0, 2)
+    assert np.array_equal(paths.to_host((3000, 31)), opaths) and sampled == osampled
+    g.free()
