@@ -100,6 +100,10 @@ int sky_graph_free(sky_graph* g);
  *      index, same slot as the CSR edge) and valid[V] i8 inside the graph.  Unlike the reference the
  *      edge weights are kept (createTable.cu:175-177 frees them). ---- */
 int sky_alias_build_all(sky_graph* g, double* seconds);
+/* The same build from a weight array of the caller (E floats in device memory, CSR slot order) instead of the graph's
+ * own weights, which are left as they are: for weights that a bias operator computes (include/skywalker_bias.h), as
+ * the reference's constructors take them from gpu_graph::getBias (include/alias_table_new.cuh:1090-1091). */
+int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, double* seconds);
 /* Copies the table to host as two arrays (any destination may be NULL). */
 int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid);
 /* Installs caller-built tables (host arrays) instead of building: for tests and table persistence.  The arrays are

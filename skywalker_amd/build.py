@@ -42,8 +42,42 @@ def build_library(verbose=False, jobs=6):
     return LIB
 
 
+PLUGINS = ["static", "node2vec", "degree"]
+
+
+def plugin_path(name):
+    return os.path.join(HERE, "libskywalker_bias_%s.so" % name)
+
+
+def build_plugins(names=PLUGINS):
+    """One shared library per bias plug-in: the engine that calls the operator and the plug-in that defines it are
+    compiled as relocatable device code and linked together, as the reference links one executable per plug-in."""
+    pdir = os.path.join(HERE, "plugins")
+    rdc = FLAGS + ["-fgpu-rdc"]
+
+    def cc(src, obj):
+        r = subprocess.run([HIPCC] + rdc + ["-c", src, "-o", obj], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+        return obj
+
+    engine = cc(os.path.join(CSRC, "sky_bias_engine.hip"), os.path.join(CSRC, "sky_bias_engine.o"))
+    out = []
+    for name in names:
+        obj = cc(os.path.join(pdir, "bias_%s.hip" % name), os.path.join(pdir, "bias_%s.o" % name))
+        lib = plugin_path(name)
+        cmd = [HIPCC, "--offload-arch=gfx950", "-fgpu-rdc", "--hip-link", "-shared", "-fPIC", "-o", lib, engine, obj,
+               "-L" + HERE, "-lskywalker_hip", "-Wl,-rpath,$ORIGIN"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed for %s:\n%s\n%s" % (lib, r.stdout, r.stderr))
+        out.append(lib)
+    return out
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_plugins())
 
 
 def build_host():

@@ -21,7 +21,7 @@ EXPORTS = [
     "sky_last_error", "sky_version", "sky_device_malloc", "sky_device_free", "sky_memcpy_h2d", "sky_memcpy_d2h",
     "sky_device_fill_u32", "sky_device_copy_u32", "sky_device_synchronize", "sky_device_name", "sky_graph_upload",
     "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
-    "sky_alias_build_all", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
+    "sky_alias_build_all", "sky_alias_build_from_weights", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
     "sky_walk_offline_noalloc", "sky_walk_index_build",
     "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_philox_selftest",
     "sky_last_build_profile", "sky_set_option",
@@ -257,6 +257,40 @@ class Graph:
             self.free()
         except Exception:
             pass
+
+
+class BiasPlugin:
+    """A bias-operator library (include/skywalker_bias.h): libskywalker_bias_<name>.so next to the main library."""
+
+    def __init__(self, name):
+        path = os.path.join(HERE, "libskywalker_bias_%s.so" % name)
+        if not os.path.exists(path):
+            raise ImportError("%s is missing: run `python -c 'import __graft_entry__ as g; g.build()'`" % path)
+        lib()  # the plug-in links against the main library
+        self.lib = C.CDLL(path)
+        self.lib.sky_bias_name.restype = C.c_char_p
+        self.lib.sky_bias_last_error.restype = C.c_char_p
+        self.name = self.lib.sky_bias_name().decode()
+
+    def _ck(self, rc):
+        if rc != 0:
+            raise SkyError(rc, self.lib.sky_bias_last_error().decode() or lib().sky_last_error().decode())
+
+    def build_all(self, g, p=1.0, q=1.0):
+        sec = C.c_double(0)
+        self._ck(self.lib.sky_bias_build_all(g.h, C.c_float(p), C.c_float(q), C.byref(sec)))
+        return sec.value
+
+    def walk_online(self, g, p, q, seeds, length, stop_prob, seed):
+        seeds_d = seeds if isinstance(seeds, DeviceArray) else DeviceArray.from_host(np.asarray(seeds, np.uint32))
+        N = seeds_d.count
+        paths = DeviceArray(N * (length + 1), np.uint32, fill=FILL)
+        lengths = DeviceArray(N, np.uint32, fill=0)
+        sampled, sec = C.c_uint64(0), C.c_double(0)
+        self._ck(self.lib.sky_bias_walk_online(g.h, C.c_float(p), C.c_float(q), seeds_d.ptr, C.c_uint32(N),
+                                               C.c_uint32(length), C.c_float(stop_prob), C.c_uint64(seed), paths.ptr,
+                                               lengths.ptr, C.byref(sampled), C.byref(sec)))
+        return paths, lengths, sampled.value, sec.value
 
 
 def set_option(name, value):

@@ -196,6 +196,16 @@ int sky_alias_build_all(sky_graph* g, double* seconds) {
   return build_all_tables(g, seconds);
 }
 
+int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, double* seconds) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null graph");
+  if (g->E && !weights_device) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null weights");
+  float* const own = g->adjwgt;
+  g->adjwgt = const_cast<float*>(weights_device);  // the build only reads it
+  const int rc = build_all_tables(g, seconds);
+  g->adjwgt = own;
+  return rc;
+}
+
 int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid) {
   if (!g) return fail(SKY_ERR_ARG, "sky_alias_download: null graph");
   if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_alias_download: tables have not been built");

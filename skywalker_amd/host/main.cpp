@@ -64,6 +64,8 @@ DEFINE_bool(newsampler, true, "use new sampler");
 DEFINE_bool(csv, false, "CSV output");
 // defined by the bias plugin in the reference (src/api/bias_static.cu:9, bias_node2vec.cu:11)
 DEFINE_bool(weight, true, "load edge weight from file");
+// new here: the bias operator as a shared library (include/skywalker_bias.h) instead of a link-time choice
+DEFINE_string(biasplugin, "", "bias plug-in library, e.g. libskywalker_bias_degree.so (default: built-in static / node2vec bias)");
 // new here: key of the Philox streams (the reference seeds cuRAND with the thread id)
 DEFINE_int32(seed, 0, "Philox seed of the samplers");
 
@@ -93,6 +95,7 @@ int main(int argc, char* argv[]) {
     FLAGS_weight = false;
     FLAGS_randomweight = false;
   }
+  if (!FLAGS_biasplugin.empty() && !BiasPlugin().Load(FLAGS_biasplugin)) return 1;
   if (FLAGS_node2vec && !FLAGS_ol) {
     LOG("node2vec is second-order: switching to --ol=1\n");
     FLAGS_ol = true;

@@ -6,9 +6,13 @@
 // Each returns the elapsed seconds of its kernel region and sets sampled_edges; results stay
 // in device memory.  Errors print file:line and exit, as the reference does.
 #pragma once
+#include <dlfcn.h>
+
 #include <cstdint>
+#include <cstring>
 #include <vector>
 
+#include "../../include/skywalker_bias.h"
 #include "gpu_graph.hpp"
 
 DECLARE_bool(itl);
@@ -20,6 +24,46 @@ DECLARE_double(p);
 DECLARE_double(q);
 DECLARE_double(tp);
 DECLARE_int32(seed);
+DECLARE_string(biasplugin);
+
+// The reference links one bias plug-in into every executable (src/api/bias_*.cu, CMakeLists.txt:54-57,84-87).
+// Here the plug-in is a shared library named at run time (--biasplugin); without one the built-in biases run.
+struct BiasPluginLib {
+  void* handle = nullptr;
+  decltype(&sky_bias_name) name = nullptr;
+  decltype(&sky_bias_last_error) last_error = nullptr;
+  decltype(&sky_bias_build_all) build_all = nullptr;
+  decltype(&sky_bias_walk_online) walk_online = nullptr;
+  bool Load(const std::string& path) {
+    handle = dlopen(path.c_str(), RTLD_NOW | RTLD_GLOBAL);
+    if (!handle) {
+      fprintf(stderr, "cannot load bias plug-in %s: %s\n", path.c_str(), dlerror());
+      return false;
+    }
+    name = (decltype(name))dlsym(handle, "sky_bias_name");
+    last_error = (decltype(last_error))dlsym(handle, "sky_bias_last_error");
+    build_all = (decltype(build_all))dlsym(handle, "sky_bias_build_all");
+    walk_online = (decltype(walk_online))dlsym(handle, "sky_bias_walk_online");
+    if (!name || !last_error || !build_all || !walk_online) {
+      fprintf(stderr, "%s does not export the entry points of include/skywalker_bias.h\n", path.c_str());
+      return false;
+    }
+    return true;
+  }
+};
+inline BiasPluginLib& BiasPlugin() {
+  static BiasPluginLib lib;
+  return lib;
+}
+#define SKY_PLUGIN_CALL(call)                                                                              \
+  do {                                                                                                     \
+    int _status = (call);                                                                                  \
+    if (_status != 0) {                                                                                    \
+      const char* _m = BiasPlugin().last_error();                                                          \
+      fprintf(stderr, "ERROR: %s:%d, error %d: %s\n", __FILE__, __LINE__, _status, _m[0] ? _m : sky_last_error()); \
+      exit(_status < 0 ? -_status : _status);                                                              \
+    }                                                                                                      \
+  } while (0)
 
 #define LOG(...)                                           \
   do {                                                     \
@@ -204,7 +248,10 @@ inline float ConstructTable(Sampler& sampler, uint ngpu = 1, uint index = 0) {
   (void)ngpu;
   (void)index;
   double sec = 0;
-  SKY_RT_CALL(sky_alias_build_all(sampler.ggraph.handle, &sec));
+  if (BiasPlugin().handle)
+    SKY_PLUGIN_CALL(BiasPlugin().build_all(sampler.ggraph.handle, (float)FLAGS_p, (float)FLAGS_q, &sec));
+  else
+    SKY_RT_CALL(sky_alias_build_all(sampler.ggraph.handle, &sec));
   sampler.ggraph.Refresh();
   sampler.alias_table = sampler.ggraph.alias_table;
   sampler.valid = sampler.ggraph.valid;
@@ -279,7 +326,11 @@ inline float walk_common(Walker& walker, bool online, const char* who) {
   uint64_t sampled = 0;
   const uint len = walker.result.hop_num - 1;
   const uint* seeds = (const uint*)walker.result.seed_buf.ptr;
-  if (online) {
+  if (online && BiasPlugin().handle) {
+    SKY_PLUGIN_CALL(BiasPlugin().walk_online(walker.ggraph.handle, (float)FLAGS_p, (float)FLAGS_q, seeds, walker.num_seed,
+                                             len, (float)FLAGS_tp, (uint64_t)FLAGS_seed, walker.result.data,
+                                             walker.result.length, &sampled, &sec));
+  } else if (online) {
     SKY_RT_CALL(sky_walk_online(walker.ggraph.handle, !FLAGS_node2vec  ? SKY_BIAS_STATIC
                                 : FLAGS_n2v_table ? SKY_BIAS_NODE2VEC
                                                   : SKY_BIAS_NODE2VEC_REJECT,

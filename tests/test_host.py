@@ -288,3 +288,27 @@ def test_cli_rejects_a_graph_without_vertices(tmp_path):
 def test_cli_rejects_multi_gpu(tmp_path):
     rc, out, err = run([os.path.join(HOST, "skywalker"), "--ngpu", "2", "--input", "/nonexistent"])
     assert rc == 1 and "one GPU" in err
+
+
+@pytest.mark.gpu
+def test_cli_degree_bias_plugin(tmp_path, orc):
+    # --biasplugin: the operator library takes the place of the reference's link-time bias (src/api/bias_degree.cu)
+    xadj, adjncy = orc.rmat_csr(11, 8, 27)
+    p = str(tmp_path / "d.gr")
+    write_gr(p, xadj, adjncy, np.ones(len(adjncy), np.uint32))
+    deg = np.diff(xadj.astype(np.int64))
+    wd = deg[adjncy].astype(np.float32)
+    plug = os.path.join(ROOT, "skywalker_amd", "libskywalker_bias_degree.so")
+    seeds = np.arange(300, dtype=np.uint32)
+    for online in (0, 1):
+        rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--bias=1", "--ol=%d" % online, "--input", p,
+                            "-n", "300", "--d", "12", "--printresult", "--seed", "6", "--biasplugin", plug])
+        assert rc == 0, err
+        lines = out.splitlines()
+        prob, alias, valid = orc.alias_build(xadj, wd)
+        paths, lengths, sampled = orc.walk_offline(xadj, adjncy, prob, alias, seeds, 12, 0.0, 6)
+        for j in range(3):
+            i = lines.index("%drd path len %d " % (j, lengths[j]))
+            assert [int(x) for x in lines[i + 1].split()] == paths[j, :min(lengths[j], 13)].tolist()
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--input", p, "--biasplugin", "/nonexistent.so"])
+    assert rc == 1 and "cannot load bias plug-in" in err
