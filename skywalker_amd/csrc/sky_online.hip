@@ -34,17 +34,30 @@ __global__ __launch_bounds__(256) void walk_collect_kernel(const uint32_t* __res
                                                            uint32_t* __restrict__ bitmap, uint32_t* __restrict__ list,
                                                            uint32_t* __restrict__ counters) {
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-  if (i >= N || lengths[i] != len) return;
-  const u32x4 r = philox(seed, i, s, 0, DOM_WALK);
-  const uint32_t v = paths[(size_t)i * (len + 1) + s];
-  if ((stop_prob > 0.0f && u24(r.z) < stop_prob) || xadj[v + 1] == xadj[v]) {
-    lengths[i] = s;
-    return;
+  bool draws = false, fresh = false;
+  uint32_t v = 0;
+  if (i < N && lengths[i] == len) {
+    const u32x4 r = philox(seed, i, s, 0, DOM_WALK);
+    v = paths[(size_t)i * (len + 1) + s];
+    if ((stop_prob > 0.0f && u24(r.z) < stop_prob) || xadj[v + 1] == xadj[v]) {
+      lengths[i] = s;
+    } else {
+      draws = true;
+      const uint32_t bit = 1u << (v & 31);  // look before the atomic: walkers crowd on hubs
+      if (!(__builtin_nontemporal_load(&bitmap[v >> 5]) & bit)) fresh = !(atomicOr(&bitmap[v >> 5], bit) & bit);
+    }
   }
-  atomicAdd(&counters[1], 1u);
-  const uint32_t bit = 1u << (v & 31);
-  if (atomicOr(&bitmap[v >> 5], bit) & bit) return;
-  list[atomicAdd(&counters[0], 1u)] = v;
+  // one counter update per wavefront and counter
+  const int lane = threadIdx.x & 63;
+  const unsigned long long md = __ballot(draws), mf = __ballot(fresh);
+  if (md && lane == __ffsll((long long)md) - 1) atomicAdd(&counters[1], (uint32_t)__popcll(md));
+  if (mf) {
+    const int first = __ffsll((long long)mf) - 1;
+    uint32_t base = 0;
+    if (lane == first) base = atomicAdd(&counters[0], (uint32_t)__popcll(mf));
+    base = (uint32_t)__shfl((int)base, first, 64);
+    if (fresh) list[base + (uint32_t)__popcll(mf & ((1ull << lane) - 1ull))] = v;
+  }
 }
 
 __global__ __launch_bounds__(256) void walk_step_kernel(const uint32_t* __restrict__ xadj,

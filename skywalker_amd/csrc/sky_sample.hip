@@ -25,31 +25,46 @@ struct HopGeom {
 
 __device__ __forceinline__ bool slot_filled(const HopGeom& g, const uint32_t* sl, uint64_t si, uint64_t s) {
   if (g.h == 0) return true;
-  return sl[si * g.slen + g.loff_prev + s / g.fan_h] > (uint32_t)(s % g.fan_h);
+  // slots of a hop fit 32 bits (sky_sample_layout checks the fanout product)
+  const uint32_t s32 = (uint32_t)s;
+  return sl[si * g.slen + g.loff_prev + s32 / g.fan_h] > s32 % g.fan_h;
 }
 
+// One lane per (seed, slot, draw).  `narrow` (N * width * k below 2^32, the usual case) keeps the index
+// arithmetic in 32 bits: three 64-bit divisions per lane cost more than the draw itself.
 __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restrict__ xadj,
                                                          const uint32_t* __restrict__ adjncy,
-                                                         const AliasEntry* __restrict__ table, uint64_t total,
-                                                         uint32_t V, HopGeom g, uint64_t seed,
+                                                         const AliasEntry* __restrict__ table,
+                                                         const int8_t* __restrict__ valid, uint64_t total,
+                                                         uint32_t V, HopGeom g, uint64_t seed, bool narrow,
                                                          uint32_t* __restrict__ data,
-                                                         uint32_t* __restrict__ sl,
-                                                         unsigned long long* __restrict__ sampled) {
+                                                         uint32_t* __restrict__ sl) {
   const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-  unsigned long long mine = 0;
   if (tid < total) {
-    const uint64_t per_seed = g.width * g.k;
-    const uint64_t si = tid / per_seed, rem = tid % per_seed;
-    const uint64_t s = rem / g.k;
-    const uint32_t i = (uint32_t)(rem % g.k);
+    uint64_t si, s;
+    uint32_t i;
+    if (narrow) {
+      const uint32_t t32 = (uint32_t)tid, width = (uint32_t)g.width;
+      const uint32_t parent = t32 / g.k;
+      i = t32 - parent * g.k;
+      const uint32_t si32 = parent / width;
+      si = si32;
+      s = parent - si32 * width;
+    } else {
+      const uint64_t per_seed = g.width * g.k;
+      const uint64_t rem = tid % per_seed;
+      si = tid / per_seed;
+      s = rem / g.k;
+      i = (uint32_t)(rem % g.k);
+    }
     if (slot_filled(g, sl, si, s)) {
       const uint32_t v = data[si * g.lps + g.off + s];
       uint32_t o = 0, deg = 0;
-      if (v < V) {  // a seed that does not exist has no children
+      if (v < V && valid[v]) {  // a seed that does not exist, or a row without weight, has no children
         o = xadj[v];
         deg = xadj[v + 1] - o;
       }
-      if (deg != 0 && table[o].alias != SKY_INVALID) {
+      if (deg != 0) {
         uint32_t* out = data + si * g.lps + g.off_next + s * g.k;
         uint32_t cnt;
         if (g.k >= deg) {
@@ -63,34 +78,67 @@ __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restr
           const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
           out[i] = adjncy[o + cand];
         }
-        if (i == 0) {
-          sl[si * g.slen + g.loff + s] = cnt;
-          mine = cnt;
-        }
+        if (i == 0) sl[si * g.slen + g.loff + s] = cnt;
       }
     }
   }
+}
+
+// Sampled edges of the call = sum of sample_lengths (as the reference counts them, src/main.cu:378-394): one pass
+// at the end, one atomic per workgroup; a counter bumped by every wavefront of every hop is a hot spot.
+__global__ __launch_bounds__(256) void sum_u32_kernel(const uint32_t* __restrict__ x, uint64_t n,
+                                                      unsigned long long* __restrict__ out) {
+  __shared__ unsigned long long s_w[4];
+  unsigned long long t = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256u) t += x[i];
 #pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) mine += shfl_xor_u64(mine, m);
-  if ((threadIdx.x & 63) == 0 && mine) atomicAdd(sampled, mine);
+  for (int m = 32; m >= 1; m >>= 1) t += shfl_xor_u64(t, m);
+  if ((threadIdx.x & 63) == 0) s_w[threadIdx.x >> 6] = t;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned long long b = s_w[0] + s_w[1] + s_w[2] + s_w[3];
+    if (b) atomicAdd(out, b);
+  }
 }
 
 // Collects the distinct vertices of the filled slots of hop h whose table has not been built
-// during this call: first setter of the vertex's bit appends it.
+// during this call: first setter of the vertex's bit appends it (one counter update per wavefront).
 __global__ __launch_bounds__(256) void frontier_collect_kernel(const uint32_t* __restrict__ data,
                                                                const uint32_t* __restrict__ sl, uint64_t total,
                                                                uint32_t V, HopGeom g, uint32_t* __restrict__ bitmap,
                                                                uint32_t* __restrict__ list,
                                                                uint32_t* __restrict__ count) {
   const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-  if (tid >= total) return;
-  const uint64_t si = tid / g.width, s = tid % g.width;
-  if (!slot_filled(g, sl, si, s)) return;
-  const uint32_t v = data[si * g.lps + g.off + s];
-  if (v >= V) return;
-  const uint32_t bit = 1u << (v & 31);
-  if (atomicOr(&bitmap[v >> 5], bit) & bit) return;
-  list[atomicAdd(count, 1u)] = v;
+  bool fresh = false;
+  uint32_t v = 0;
+  if (tid < total) {
+    uint64_t si, s;
+    if (total <= 0xFFFFFFFFull) {
+      const uint32_t si32 = (uint32_t)tid / (uint32_t)g.width;
+      si = si32;
+      s = (uint32_t)tid - si32 * (uint32_t)g.width;
+    } else {
+      si = tid / g.width;
+      s = tid % g.width;
+    }
+    if (slot_filled(g, sl, si, s)) {
+      v = data[si * g.lps + g.off + s];
+      if (v < V) {
+        // hubs fill many slots: look before the atomic, which only the first few visitors of a word then issue
+        // (a stale look only costs an atomic)
+        const uint32_t bit = 1u << (v & 31);
+        if (!(__builtin_nontemporal_load(&bitmap[v >> 5]) & bit)) fresh = !(atomicOr(&bitmap[v >> 5], bit) & bit);
+      }
+    }
+  }
+  const unsigned long long m = __ballot(fresh);
+  if (m) {
+    const int lane = threadIdx.x & 63, first = __ffsll((long long)m) - 1;
+    uint32_t base = 0;
+    if (lane == first) base = atomicAdd(count, (uint32_t)__popcll(m));
+    base = (uint32_t)__shfl((int)base, first, 64);
+    if (fresh) list[base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = v;
+  }
 }
 
 __global__ __launch_bounds__(256) void sample_init_kernel(const uint32_t* __restrict__ seeds, uint32_t N, uint64_t lps,
@@ -160,7 +208,13 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
       const uint64_t total = (uint64_t)N * hg.width * hg.k;
       if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");
       hipLaunchKernelGGL(sample_hop_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, g->xadj,
-                         g->adjncy, g->table, total, g->V, hg, seed, data, sample_lengths, d_sampled);
+                         g->adjncy, g->table, g->valid, total, g->V, hg, seed, total <= 0xFFFFFFFFull, data,
+                         sample_lengths);
+    }
+    if (N && slen) {
+      const uint64_t n = (uint64_t)N * slen;
+      hipLaunchKernelGGL(sum_u32_kernel, dim3((uint32_t)std::min<uint64_t>((n + 255) / 256, 1024)), dim3(256), 0, st,
+                         sample_lengths, n, d_sampled);
     }
     SKY_TRY(tm.mark("sample", 0));
     SKY_TRY(tm.finish(nullptr, seconds));
