@@ -43,8 +43,8 @@ __global__ __launch_bounds__(256) void walk_collect_kernel(const uint32_t* __res
       lengths[i] = s;
     } else {
       draws = true;
-      const uint32_t bit = 1u << (v & 31);  // look before the atomic: walkers crowd on hubs
-      if (!(__builtin_nontemporal_load(&bitmap[v >> 5]) & bit)) fresh = !(atomicOr(&bitmap[v >> 5], bit) & bit);
+      const uint32_t bit = 1u << (v & 31);
+      fresh = !(atomicOr(&bitmap[v >> 5], bit) & bit);
     }
   }
   // one counter update per wavefront and counter

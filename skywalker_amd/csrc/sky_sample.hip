@@ -124,10 +124,8 @@ __global__ __launch_bounds__(256) void frontier_collect_kernel(const uint32_t* _
     if (slot_filled(g, sl, si, s)) {
       v = data[si * g.lps + g.off + s];
       if (v < V) {
-        // hubs fill many slots: look before the atomic, which only the first few visitors of a word then issue
-        // (a stale look only costs an atomic)
         const uint32_t bit = 1u << (v & 31);
-        if (!(__builtin_nontemporal_load(&bitmap[v >> 5]) & bit)) fresh = !(atomicOr(&bitmap[v >> 5], bit) & bit);
+        fresh = !(atomicOr(&bitmap[v >> 5], bit) & bit);
       }
     }
   }
