@@ -45,6 +45,7 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
   if (nw <= 16) return CLS_MW2 + (int)nw - 2;
   if (d > STREAM_MAX_DEG) return CLS_HUGE;
+  if (d > 65533u) return CLS_STREAM_WIDE;
   return d > 24576u ? CLS_STREAM : CLS_STREAM_LAST;
 }
 
@@ -1163,7 +1164,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
 
   uint32_t stream_rows = 0;
   uint64_t stream_edges = 0;
-  for (int c = CLS_STREAM; c <= CLS_STREAM_LAST; ++c) {
+  for (int c = CLS_STREAM_WIDE; c <= CLS_STREAM_LAST; ++c) {
     stream_rows += counts[c];
     stream_edges += host.edges[c];
   }
@@ -1171,12 +1172,12 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   // with the HUGE class that follows them in the list.
   const bool stream_to_tiled = !g_row_merge || stream_edges <= g_stream_min_edges;
   if (stream_rows && !stream_to_tiled) {  // one launch over the two lists, which lie back to back
-    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM], stream_rows));
+    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], stream_rows));
     if (tm) SKY_TRY(tm->mark("stream", stream_edges));
   }
   const uint32_t tiled_rows = counts[CLS_HUGE] + (stream_to_tiled ? stream_rows : 0);
   const uint64_t tiled_edges = host.edges[CLS_HUGE] + (stream_to_tiled ? stream_edges : 0);
-  const RowRef* tiled_list = vlist + (stream_to_tiled ? starts[CLS_STREAM] : starts[CLS_HUGE]);
+  const RowRef* tiled_list = vlist + (stream_to_tiled ? starts[CLS_STREAM_WIDE] : starts[CLS_HUGE]);
   if (tiled_rows) {
     const uint32_t cnt = tiled_rows;
     uint32_t skipped = 0;

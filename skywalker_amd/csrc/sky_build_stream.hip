@@ -1,4 +1,4 @@
-// Alias tables of rows of 8190..65533 entries: one workgroup streams the row and keeps a window of
+// Alias tables of rows of 8190..524287 entries: one workgroup streams the row and keeps a window of
 // the row's heavies in LDS.
 //
 // The table is the same pure function of the weights as everywhere else (see sky_build.hip).
@@ -6,7 +6,7 @@
 // prefix exceeds the light's exclusive deficit prefix, and a heavy's residual probability belongs
 // to the one light whose deficit interval (SL - D, SL] contains the heavy's surplus prefix.  So
 //   pass A   exact sum of the weights -> ledger
-//   collect  the next ST_CAP heavies in slot order into LDS, {surplus prefix, slot, residual}, 14 bytes
+//   collect  the next ST_CAP heavies in slot order into LDS, {surplus prefix, slot, residual}, 16 bytes
 //            each, and the slot of the heavy after them, if there is one
 //   emit     classify every entry, running deficit prefix; a light whose alias lies in the window
 //            gets its entry, and every light leaves the residual of the window's heavies that fall
@@ -28,8 +28,8 @@ constexpr int ST_T = 512;                 // threads per row
 constexpr int ST_PER = 8;                 // consecutive slots per thread and chunk
 constexpr int ST_CH = ST_T * ST_PER;      // slots per chunk
 constexpr int ST_NW = ST_T / 64;
-constexpr uint32_t ST_CAP = 5815;         // heavies per row kept in LDS (and one sentinel): two workgroups share a CU's 160 KB
-static_assert(STREAM_MAX_DEG + 3 <= 65536, "heavy slots are stored as 16-bit numbers");
+constexpr uint32_t ST_CAP = 5085;         // heavies per row kept in LDS (and one sentinel): two workgroups share a CU's 160 KB
+static_assert(STREAM_MAX_DEG + 3 < (1u << 20), "the three-limb sum is exact for rows of fewer than 2^20 entries");
 
 struct StreamRow {
   uint32_t base, lead, span;
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
                                                             int8_t* __restrict__ valid) {
   __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the window's h-th heavy, then a sentinel
   __shared__ float s_prob[ST_CAP + 1];     // its residual probability, left by the light that reaches it
-  __shared__ uint16_t s_slot[ST_CAP + 1];  // its span slot; after them the slot lights beyond the window take
+  __shared__ uint32_t s_slot[ST_CAP + 1];  // its span slot; after them the slot lights beyond the window take
   __shared__ WSum3 s_w[ST_NW];
   __shared__ uint64_t s_a[2][ST_NW];  // two sets of wavefront sums, used alternately
   __shared__ uint32_t s_c[2][ST_NW];
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
           const uint32_t slot = c * ST_CH + (uint32_t)ST_PER * tid + j;
           if (rank >= hb && rank < hb + ST_CAP) {
             s_w32[2 * (rank - hb)] = cw[j];
-            s_slot[rank - hb] = (uint16_t)slot;
+            s_slot[rank - hb] = slot;
           } else if (rank == hb + ST_CAP) {
             s_next = slot;
           }
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     const bool whole_row = hb == 0 && !more;  // the usual case: one window holds every heavy of the row
     if (tid == 0) {  // after the list: a sentinel, and the slot that lights beyond the window's last heavy take
       s_sh[nw] = ~0ull;
-      s_slot[nw] = more ? (uint16_t)next_slot : (nw ? s_slot[nw - 1] : (uint16_t)0);
+      s_slot[nw] = more ? next_slot : (nw ? s_slot[nw - 1] : 0u);
     }
     __syncthreads();
 

@@ -61,11 +61,12 @@ enum BuildClass : int {
   CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
   CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..16 (class CLS_MW2 + nw - 2): one workgroup per row whose
   CLS_MW16 = 24,    //                  threads cover 512 * nw slots
-  CLS_STREAM = 25,  // deg 24577..65533 one workgroup streams the row, its heavies stay in LDS.  Two classes, the
-  CLS_STREAM_LAST = 26,  // deg 8190..24576  longer rows first, listed back to back and built by one launch, which so
+  CLS_STREAM_WIDE = 25,  // deg 65534..524287  one workgroup streams the row, a window of its heavies stays in LDS.
+  CLS_STREAM = 26,       // deg 24577..65533   Three classes, the longer rows first, listed back to back and built
+  CLS_STREAM_LAST = 27,  // deg 8190..24576    by one launch, which so
                     //                  does not end on its longest rows
-  CLS_HUGE = 27,    // above            built tile by tile by the whole GPU
-  CLS_COUNT = 28
+  CLS_HUGE = 28,    // above            built tile by tile by the whole GPU
+  CLS_COUNT = 29
 };
 
 // One listed row of a degree class: the build kernels read where the row lies from the list itself
@@ -102,7 +103,7 @@ constexpr uint32_t TILED_TILE = 1024;  // slots per tile of the tile-parallel pa
 int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
                      uint64_t edges);
 void set_tiled_max_tiles(uint32_t n);
-constexpr uint32_t STREAM_MAX_DEG = 65533;  // longest row of the streaming class
+constexpr uint32_t STREAM_MAX_DEG = 524287;  // longest row of the streaming classes (one workgroup takes 1.5 ms for it)
 int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n);
 void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);

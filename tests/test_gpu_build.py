@@ -11,7 +11,7 @@ TOL = 1e-6
 # degrees that straddle every dispatch class boundary of the build
 EDGE_DEGREES = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 16, 17, 22, 23, 24, 25, 28, 29, 30, 32, 33, 46, 47, 48,
                 49, 60, 61, 62, 63, 64, 65, 66, 67, 68, 94, 95, 96, 97, 124, 125, 126, 127, 190, 191, 192, 193, 253, 254, 255, 256, 257, 1021,
-                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 8189, 8190, 8191, 8192, 8193, 20000, 70001]
+                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 8189, 8190, 8191, 8192, 8193, 20000, 70001, 128, 129]
 
 
 def build_and_compare(orc, xadj, adjncy, w, label):
@@ -19,9 +19,9 @@ def build_and_compare(orc, xadj, adjncy, w, label):
     print("case", label, "V", len(xadj) - 1, "E", len(w), flush=True)
     oprob, oalias, ovalid = orc.alias_build(xadj, w)
     deg = np.diff(xadj)
-    # rows of 8190..65533 entries: once through their own kernel, once (the default for so few of them)
+    # rows of 8190..524287 entries: once through their own kernel, once (the default for so few of them)
     # through the tile-parallel path
-    routes = (0, 4000000) if ((deg >= 8190) & (deg <= 65533)).any() else (4000000,)
+    routes = (0, 4000000) if ((deg >= 8190) & (deg <= 524287)).any() else (4000000,)
     for stream_min_edges in routes:
         g = capi.Graph.upload(xadj, adjncy, w)
         capi.set_option("stream_min_edges", stream_min_edges)
@@ -157,11 +157,11 @@ def test_search_variant_of_the_row_kernels_gives_the_same_table(orc):
 
 @pytest.mark.parametrize("dist", ["lognormal2", "uniform", "nearequal", "sparse", "fewlights", "fewheavies"])
 def test_rows_streamed_by_one_workgroup(orc, dist):
-    # rows of 8190..65533 entries: a window of 8063 heavies kept in LDS ("fewlights" and "uniform" have rows with
-    # up to eight windows, "nearequal" rows without a heavy); 65534 is the first degree of the tile-parallel class
+    # rows of 8190..524287 entries: a window of 5085 heavies kept in LDS ("fewlights" and "uniform" have rows with
+    # many windows, "nearequal" rows without a heavy); 524288 is the first degree of the tile-parallel class
     from helpers import weights
     rng = np.random.default_rng(31)
-    degs = [8190, 8191, 7, 8193, 12288, 2, 12289, 16385, 1, 30000, 65533, 65534, 0, 9001]
+    degs = [8190, 8191, 7, 8193, 12288, 2, 12289, 16385, 1, 30000, 65533, 65534, 0, 9001, 150001, 524287, 524288]
     xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=4096)
     if dist == "fewlights":
         w = np.where(rng.random(len(w)) < 0.01, 0.01, 1.01).astype(np.float32)
@@ -254,7 +254,8 @@ def test_random_mixtures_of_every_class(orc, seed):
     # special values sprinkled into some
     from helpers import weights
     rng = np.random.default_rng(1000 + seed)
-    ends = [0, 1, 2, 3, 5, 6, 13, 14, 29, 30, 61, 62, 125, 126, 191, 192, 253, 254, 509, 8190, 24576, 24577, 65533, 65534]
+    ends = [0, 1, 2, 3, 5, 6, 8, 9, 13, 14, 16, 17, 29, 30, 32, 33, 61, 62, 64, 65, 125, 126, 128, 129, 191, 192, 193, 253, 254,
+            509, 8190, 24576, 24577, 65533, 65534]
     for nw in range(2, 17):
         ends += [512 * (nw - 1) - 2, 512 * nw - 3]
     degs = ends + list(rng.integers(0, 70, 3000)) + list(rng.integers(60, 600, 600)) + \
