@@ -260,21 +260,27 @@ __device__ __forceinline__ uint32_t first_tile_above(const uint64_t* B, uint32_t
 }
 
 // Per row: BL[t], BH[t] = deficits / surpluses before tile t (t = 0..ntiles, the last entry is the
-// row total), stored at index tile0 + row + t; nfh[tile] = first heavy in any later tile.
-__global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ rows, uint32_t count,
-                                                        const TileTotals* __restrict__ ttot,
-                                                        uint64_t* __restrict__ BL, uint64_t* __restrict__ BH,
-                                                        uint32_t* __restrict__ nfh, uint4* __restrict__ ranges) {
+// row total), stored at index tile0 + row + t; nfh[tile] = first heavy in any later tile.  One workgroup
+// of 1024 threads per row: a row of a million entries has a thousand tiles, and one wavefront walking
+// them 64 at a time with dependent loads was a sixth of a millisecond on the critical path.
+constexpr int TS_T = 1024;
+__global__ __launch_bounds__(TS_T) void tiled_scan_kernel(TiledRow* __restrict__ rows, uint32_t count,
+                                                          const TileTotals* __restrict__ ttot,
+                                                          uint64_t* __restrict__ BL, uint64_t* __restrict__ BH,
+                                                          uint32_t* __restrict__ nfh, uint4* __restrict__ ranges) {
+  constexpr int NW = TS_T / 64;
+  __shared__ uint64_t s_wl[NW], s_wh[NW];
+  __shared__ uint32_t s_wm[NW];
   const uint32_t r = blockIdx.x;
   if (r >= count) return;
   const uint32_t t0 = rows[r].tile0, nt = rows[r].ntiles;
   if (nt == 0 || !rows[r].ok) return;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t b0 = rows[r].bofs;
   uint64_t cl = 0, ch = 0;
   uint32_t last = NONE32;
-  for (uint32_t c = 0; c < nt; c += 64) {
-    const uint32_t t = c + lane;
+  for (uint32_t c = 0; c < nt; c += TS_T) {
+    const uint32_t t = c + tid;
     uint64_t d = 0, u = 0;
     uint32_t lh = 0;
     if (t < nt) {
@@ -284,23 +290,41 @@ __global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ r
       lh = x.last_heavy == NONE32 ? 0 : x.last_heavy + 1;
     }
     const uint64_t il = group_scan_u64<64>(d), ih = group_scan_u64<64>(u);
-    if (t < nt) {
-      BL[b0 + t] = cl + il - d;
-      BH[b0 + t] = ch + ih - u;
-    }
-    cl += shfl_u64(il, 63);
-    ch += shfl_u64(ih, 63);
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) lh = max(lh, (uint32_t)__shfl_xor((int)lh, m, 64));
-    if (lh) last = lh - 1;
+    if (lane == 63) {
+      s_wl[wave] = il;
+      s_wh[wave] = ih;
+      s_wm[wave] = lh;
+    }
+    __syncthreads();
+    uint64_t bl = cl, bh = ch, tl = 0, th = 0;
+    uint32_t lm = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      if (w == wave) {
+        bl += tl;
+        bh += th;
+      }
+      tl += s_wl[w];
+      th += s_wh[w];
+      lm = max(lm, s_wm[w]);
+    }
+    if (t < nt) {
+      BL[b0 + t] = bl + il - d;
+      BH[b0 + t] = bh + ih - u;
+    }
+    cl += tl;
+    ch += th;
+    if (lm) last = lm - 1;
+    __syncthreads();  // the wavefront totals are rewritten by the next round
   }
-  // next first heavy: walk the tiles backwards
+  // next first heavy: the tiles backwards, exclusive suffix minimum of first_heavy
   uint32_t carry = NONE32;
-  for (int32_t c = (int32_t)((nt - 1) / 64 * 64); c >= 0; c -= 64) {
-    const uint32_t t = (uint32_t)c + lane;
-    uint32_t fh = t < nt ? ttot[t0 + t].first_heavy : NONE32;
-    // exclusive suffix minimum over lanes
-    uint32_t suf = fh;
+  for (int32_t c = (int32_t)((nt - 1) / TS_T * TS_T); c >= 0; c -= TS_T) {
+    const uint32_t t = (uint32_t)c + tid;
+    const uint32_t fh = t < nt ? ttot[t0 + t].first_heavy : NONE32;
+    uint32_t suf = fh;  // inclusive suffix minimum over the lanes of the wavefront
 #pragma unroll
     for (int dlt = 1; dlt < 64; dlt <<= 1) {
       const uint32_t o = (uint32_t)__shfl_down((int)suf, dlt, 64);
@@ -308,10 +332,19 @@ __global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ r
     }
     uint32_t excl = (uint32_t)__shfl_down((int)suf, 1, 64);
     if (lane == 63) excl = NONE32;
-    if (t < nt) nfh[t0 + t] = min(excl, carry);
-    carry = min(carry, (uint32_t)__shfl((int)suf, 0, 64));
+    if (lane == 0) s_wm[wave] = suf;  // minimum of the wavefront
+    __syncthreads();
+    uint32_t later = carry, all = carry;  // minimum over the later wavefronts of this round and the later rounds
+#pragma unroll
+    for (int w = NW - 1; w >= 0; --w) {
+      if (w == wave) later = all;
+      all = min(all, s_wm[w]);
+    }
+    if (t < nt) nfh[t0 + t] = min(excl, later);
+    carry = all;
+    __syncthreads();
   }
-  if (lane == 0) {
+  if (tid == 0) {
     BL[b0 + nt] = cl;
     BH[b0 + nt] = ch;
     rows[r].total_h = ch;
@@ -323,7 +356,7 @@ __global__ __launch_bounds__(64) void tiled_scan_kernel(TiledRow* __restrict__ r
   __syncthreads();
   const uint64_t* rl = BL + b0;
   const uint64_t* rh = BH + b0;
-  for (uint32_t t = lane; t < nt; t += 64) {
+  for (uint32_t t = tid; t < nt; t += TS_T) {
     uint4 g;
     g.x = first_tile_above(rh, nt, rl[t]);
     g.y = min(first_tile_above(rh, nt, rl[t + 1]), nt - 1);
@@ -658,7 +691,7 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
   hipLaunchKernelGGL(tiled_ledger_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.tsum);
   hipLaunchKernelGGL(tiled_totals_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.geom, sc.rows, g->adjwgt, sc.ttot);
   if (tm) SKY_TRY(tm->mark("tiled_totals", edges));
-  hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(64), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh, sc.ranges);
+  hipLaunchKernelGGL(tiled_scan_kernel, dim3(n), dim3(TS_T), 0, st, sc.rows, n, sc.ttot, sc.BL, sc.BH, sc.nfh, sc.ranges);
   hipLaunchKernelGGL(tiled_emit_kernel, dim3(ntiles), dim3(TL_T), 0, st, sc.geom, sc.rows, g->adjwgt, sc.BL,
                      sc.BH, sc.nfh, sc.ranges, g->table, g->valid);
   if (tm) SKY_TRY(tm->mark("tiled_emit", edges));
