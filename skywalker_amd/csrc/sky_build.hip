@@ -220,8 +220,8 @@ __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restri
 // leaves one row of class counts per block, bin_offsets_kernel turns the rows into each block's
 // first position inside every class segment, and the scatter kernel hands out positions from
 // cursors it keeps in LDS, so no global atomic is involved and the lists come out grouped by block.
-constexpr int BIN_BLOCKS = 2048;  // most blocks a binning pass uses
-constexpr int BIN_ITEMS = 4;      // vertices per thread and step of the scatter pass
+constexpr int BIN_BLOCKS = 4096;  // most blocks a binning pass uses
+constexpr int BIN_ITEMS = 4;      // vertices per thread and step
 
 __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restrict__ xadj,
                                                         const uint32_t* __restrict__ src, uint32_t n,
@@ -236,15 +236,28 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
   __syncthreads();
   const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
   uint32_t tiny_edges = 0;  // rows of 1..2 entries, the commonest kind of a power-law graph, stay out of the LDS atomics
-  for (uint32_t i = lo + threadIdx.x; i < hi; i += 256u) {
-    const uint32_t v = src ? src[i] : i;
-    const uint32_t d = xadj[v + 1] - xadj[v];
-    const int c = degree_class(d);
-    if (c >= CLS_G2) {
-      atomicAdd(&s_cnt[c], 1u);
-      atomicAdd(&s_edges[c], (unsigned long long)d);
-    } else {
-      tiny_edges += d;  // 0 for an empty row
+  // four vertices per thread and step: their loads are in flight together (one at a time, the loop waits a
+  // memory round trip per vertex)
+  for (uint32_t chunk = lo; chunk < hi; chunk += 256u * BIN_ITEMS) {
+    uint32_t d[BIN_ITEMS];
+#pragma unroll
+    for (int k = 0; k < BIN_ITEMS; ++k) {
+      const uint32_t i = chunk + k * 256u + threadIdx.x;
+      d[k] = 0;
+      if (i < hi) {
+        const uint32_t v = src ? src[i] : i;
+        d[k] = xadj[v + 1] - xadj[v];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < BIN_ITEMS; ++k) {
+      const int c = degree_class(d[k]);
+      if (c >= CLS_G2) {
+        atomicAdd(&s_cnt[c], 1u);
+        atomicAdd(&s_edges[c], (unsigned long long)d[k]);
+      } else {
+        tiny_edges += d[k];  // 0 for an empty row
+      }
     }
   }
 #pragma unroll
@@ -257,19 +270,31 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
   }
 }
 
-// One wavefront per class: exclusive prefix of the class's per-block counts (in place), total to counts[c].
-__global__ __launch_bounds__(64) void bin_offsets_kernel(uint32_t* __restrict__ blk_cnt, uint32_t blocks,
-                                                         uint32_t* __restrict__ counts) {
-  const uint32_t c = blockIdx.x, lane = threadIdx.x;
-  uint32_t run = 0;
-  for (uint32_t b0 = 0; b0 < blocks; b0 += 64) {
-    const uint32_t b = b0 + lane;
-    const uint32_t x = b < blocks ? blk_cnt[b * CLS_COUNT + c] : 0u;
-    const uint32_t inc = group_scan_u32<64>(x);
-    if (b < blocks) blk_cnt[b * CLS_COUNT + c] = run + inc - x;
-    run += (uint32_t)__shfl((int)inc, 63, 64);
+// One workgroup per class: exclusive prefix of the class's per-block counts (in place), total to counts[c].
+// Thread t owns a run of consecutive blocks: its loads do not wait for one another.
+__global__ __launch_bounds__(256) void bin_offsets_kernel(uint32_t* __restrict__ blk_cnt, uint32_t blocks,
+                                                          uint32_t* __restrict__ counts) {
+  __shared__ uint32_t s_w[4];
+  const uint32_t c = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr uint32_t RUN = (BIN_BLOCKS + 255) / 256;
+  const uint32_t b0 = tid * RUN;
+  uint32_t x[RUN], sum = 0;
+#pragma unroll
+  for (uint32_t k = 0; k < RUN; ++k) {
+    x[k] = b0 + k < blocks ? blk_cnt[(b0 + k) * CLS_COUNT + c] : 0u;
+    sum += x[k];
   }
-  if (lane == 0) counts[c] = run;
+  const uint32_t inc = group_scan_u32<64>(sum);
+  if (lane == 63) s_w[wave] = inc;
+  __syncthreads();
+  uint32_t run = inc - sum;
+  for (uint32_t w = 0; w < wave; ++w) run += s_w[w];
+#pragma unroll
+  for (uint32_t k = 0; k < RUN; ++k) {
+    if (b0 + k < blocks) blk_cnt[(b0 + k) * CLS_COUNT + c] = run;
+    run += x[k];
+  }
+  if (tid == 0) counts[c] = s_w[0] + s_w[1] + s_w[2] + s_w[3];
 }
 
 // A row of one or two entries in closed form.
@@ -1055,7 +1080,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t blocks = (n + per_block - 1) / per_block;
     hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n, per_block, sc.blk_cnt,
                        reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
-    hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(64), 0, st, sc.blk_cnt, blocks, sc.counters);
+    hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(256), 0, st, sc.blk_cnt, blocks, sc.counters);
     hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n, per_block,
                        sc.counters, sc.blk_cnt, sc.vlist, g->table, g->valid);
     // The class sizes decide the launches that follow.  Those of all vertices depend on xadj alone and are kept
