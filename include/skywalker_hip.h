@@ -183,9 +183,12 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      fall to a kernel in which one workgroup walks the whole row.  Tests lower it to exercise that kernel.
  *      "row_merge" (default 1): rows of 62..8189 entries pair lights and heavies by a merge of their prefix
  *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table.
- *      "stream_min_edges" (default 4000000): rows of 8190..65533 entries have a kernel of their own (one workgroup
+ *      "stream_min_edges" (default 4000000): rows of 8190..524287 entries have a kernel of their own (one workgroup
  *      streams a row); when a build holds no more than this many entries in such rows, too few to fill the GPU
  *      with one workgroup each, they go to the tile-parallel path instead.  Tests set 0.
+ *      "stream_wide_min_edges" (default 134217216): the rows of more than 65533 entries among them keep a workgroup
+ *      busy for up to 1.5 ms; they join that kernel only when the build holds at least this many entries in rows
+ *      of 8190..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
  *      "build_profile" (default 0): 1 records a HIP event after every kernel of sky_alias_build_all for
  *      sky_last_build_profile (about 3 microseconds each; a small graph pays 20 % of its build for them).
  *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:

@@ -968,6 +968,8 @@ int enable_big_lds(K kernel, size_t bytes) {
 
 }  // namespace
 static uint64_t g_stream_min_edges = 4000000;
+static uint64_t g_stream_wide_min_edges = 512ull * (STREAM_MAX_DEG / 2);  // 512 workgroups run at a time
+void set_stream_wide_min_edges(uint64_t n) { g_stream_wide_min_edges = n; }
 static bool g_build_profile = false;
 void set_build_profile(bool on) { g_build_profile = on; }
 void set_stream_min_edges(uint64_t n) { g_stream_min_edges = n; }
@@ -1187,22 +1189,26 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
   }
 
-  uint32_t stream_rows = 0;
-  uint64_t stream_edges = 0;
-  for (int c = CLS_STREAM_WIDE; c <= CLS_STREAM_LAST; ++c) {
-    stream_rows += counts[c];
-    stream_edges += host.edges[c];
+  // Rows of 8190..STREAM_MAX_DEG entries: one workgroup streams a row.  A small streaming class is not worth its
+  // own launch (too few workgroups to fill the GPU): its rows then go to the tile-parallel path together with the
+  // HUGE class.  The rows above 65533 entries keep one workgroup busy for up to 1.5 ms; they join the launch (and
+  // start first) only when it holds enough other rows to run that long anyway, else they are built tile by tile.
+  // The lists lie back to back: STREAM, STREAM_LAST, STREAM_WIDE, HUGE.
+  const uint32_t narrow_rows = counts[CLS_STREAM] + counts[CLS_STREAM_LAST];
+  const uint64_t narrow_edges = host.edges[CLS_STREAM] + host.edges[CLS_STREAM_LAST];
+  const uint64_t all_stream_edges = narrow_edges + host.edges[CLS_STREAM_WIDE];
+  const bool stream_to_tiled = !g_row_merge || all_stream_edges <= g_stream_min_edges;
+  const bool wide_streamed = !stream_to_tiled && all_stream_edges >= g_stream_wide_min_edges;
+  const uint32_t wide_rows = wide_streamed ? counts[CLS_STREAM_WIDE] : 0;
+  if (!stream_to_tiled && narrow_rows + wide_rows) {
+    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], wide_rows, vlist + starts[CLS_STREAM], narrow_rows));
+    if (tm) SKY_TRY(tm->mark("stream", narrow_edges + (wide_streamed ? host.edges[CLS_STREAM_WIDE] : 0)));
   }
-  // A small streaming class is not worth its own launch: its rows then go to the tile-parallel path together
-  // with the HUGE class that follows them in the list.
-  const bool stream_to_tiled = !g_row_merge || stream_edges <= g_stream_min_edges;
-  if (stream_rows && !stream_to_tiled) {  // one launch over the two lists, which lie back to back
-    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], stream_rows));
-    if (tm) SKY_TRY(tm->mark("stream", stream_edges));
-  }
-  const uint32_t tiled_rows = counts[CLS_HUGE] + (stream_to_tiled ? stream_rows : 0);
-  const uint64_t tiled_edges = host.edges[CLS_HUGE] + (stream_to_tiled ? stream_edges : 0);
-  const RowRef* tiled_list = vlist + (stream_to_tiled ? starts[CLS_STREAM_WIDE] : starts[CLS_HUGE]);
+  const uint32_t tiled_rows = counts[CLS_HUGE] + (wide_streamed ? 0 : counts[CLS_STREAM_WIDE]) + (stream_to_tiled ? narrow_rows : 0);
+  const uint64_t tiled_edges =
+      host.edges[CLS_HUGE] + (wide_streamed ? 0 : host.edges[CLS_STREAM_WIDE]) + (stream_to_tiled ? narrow_edges : 0);
+  const RowRef* tiled_list =
+      vlist + (stream_to_tiled ? starts[CLS_STREAM] : (wide_streamed ? starts[CLS_HUGE] : starts[CLS_STREAM_WIDE]));
   if (tiled_rows) {
     const uint32_t cnt = tiled_rows;
     uint32_t skipped = 0;

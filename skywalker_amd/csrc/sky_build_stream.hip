@@ -153,7 +153,8 @@ __device__ __forceinline__ uint64_t uniform_u64(uint64_t x) {
   return ((uint64_t)uniform_u32((uint32_t)(x >> 32)) << 32) | uniform_u32((uint32_t)x);
 }
 
-__global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __restrict__ vlist,
+__global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __restrict__ first_list, uint32_t n_first,
+                                                            const RowRef* __restrict__ vlist,
                                                             const float* __restrict__ wgt,
                                                             AliasEntry* __restrict__ table,
                                                             int8_t* __restrict__ valid) {
@@ -164,7 +165,8 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   __shared__ uint64_t s_a[2][ST_NW];  // two sets of wavefront sums, used alternately
   __shared__ uint32_t s_c[2][ST_NW];
   __shared__ uint32_t s_next;  // slot of the first heavy after the window
-  const RowRef rr = vlist[blockIdx.x];
+  // the first n_first workgroups take the rows of first_list (the longest ones), the others those of vlist
+  const RowRef rr = blockIdx.x < n_first ? first_list[blockIdx.x] : vlist[blockIdx.x - n_first];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   StreamRow r;
   r.base = rr.off & ~3u;
@@ -445,11 +447,12 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   }
 }
 
-// Builds the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each).
-int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n) {
-  if (n == 0) return SKY_OK;
-  hipLaunchKernelGGL(build_stream_kernel, dim3(n), dim3(ST_T), 0, g->stream, rows_list, g->adjwgt, g->table,
-                     g->valid);
+// Builds the n_first rows of `first_list` and the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each) in one
+// launch that starts with the former.
+int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n) {
+  if (n + n_first == 0) return SKY_OK;
+  hipLaunchKernelGGL(build_stream_kernel, dim3(n + n_first), dim3(ST_T), 0, g->stream, first_list, n_first, rows_list,
+                     g->adjwgt, g->table, g->valid);
   return SKY_OK;
 }
 

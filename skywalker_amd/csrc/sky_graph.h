@@ -61,9 +61,9 @@ enum BuildClass : int {
   CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
   CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..16 (class CLS_MW2 + nw - 2): one workgroup per row whose
   CLS_MW16 = 24,    //                  threads cover 512 * nw slots
-  CLS_STREAM_WIDE = 25,  // deg 65534..524287  one workgroup streams the row, a window of its heavies stays in LDS.
-  CLS_STREAM = 26,       // deg 24577..65533   Three classes, the longer rows first, listed back to back and built
-  CLS_STREAM_LAST = 27,  // deg 8190..24576    by one launch, which so
+  CLS_STREAM = 25,       // deg 24577..65533   one workgroup streams the row, a window of its heavies stays in LDS.
+  CLS_STREAM_LAST = 26,  // deg 8190..24576    Three classes built by one launch that takes the longest rows first
+  CLS_STREAM_WIDE = 27,  // deg 65534..524287  and so
                     //                  does not end on its longest rows
   CLS_HUGE = 28,    // above            built tile by tile by the whole GPU
   CLS_COUNT = 29
@@ -104,9 +104,10 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
                      uint64_t edges);
 void set_tiled_max_tiles(uint32_t n);
 constexpr uint32_t STREAM_MAX_DEG = 524287;  // longest row of the streaming classes (one workgroup takes 1.5 ms for it)
-int build_rows_stream(sky_graph* g, const RowRef* rows_list, uint32_t n);
+int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n);
 void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);
+void set_stream_wide_min_edges(uint64_t n);
 void set_build_profile(bool on);
 void set_online_full_build(int mode);
 void set_walk_compact_every(uint32_t steps);

@@ -25,10 +25,12 @@ def build_and_compare(orc, xadj, adjncy, w, label):
     for stream_min_edges in routes:
         g = capi.Graph.upload(xadj, adjncy, w)
         capi.set_option("stream_min_edges", stream_min_edges)
+        capi.set_option("stream_wide_min_edges", stream_min_edges)  # 0: also the rows above 65533 entries are streamed
         try:
             g.build_tables()
         finally:
             capi.set_option("stream_min_edges", 4000000)
+            capi.set_option("stream_wide_min_edges", 512 * 262143)
         prob, alias, valid = g.tables()
         g.free()
         st = orc.alias_check(xadj, w, prob, alias, valid)
