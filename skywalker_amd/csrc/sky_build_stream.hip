@@ -55,20 +55,33 @@ __device__ __forceinline__ RawChunk fetch_chunk(const float* __restrict__ wgt, c
   }
   return x;
 }
-// Clamped weights as doubles (0 outside the row) and the mask of slots that belong to the row.
+// Whether every slot of wavefront `wave` in chunk c lies inside the row: true for all but the row's first wavefront
+// (when the row starts after its 16-byte aligned base) and the one that holds its end.  Such a wavefront needs
+// no per-slot masks.
+__device__ __forceinline__ bool wave_inside_row(const StreamRow& r, uint32_t c, int wave) {
+  const uint32_t w0 = c * ST_CH + (uint32_t)(ST_PER * 64) * (uint32_t)wave;
+  return w0 >= r.lead && w0 + (uint32_t)(ST_PER * 64) <= r.span;
+}
+// Clamped weights (0 outside the row) and the mask of slots that belong to the row.  EDGE false: the caller
+// knows that every slot does.
+template <bool EDGE>
 __device__ __forceinline__ uint32_t unpack_chunk(const RawChunk& x, const StreamRow& r, uint32_t c, int tid,
-                                                 double (&wd)[ST_PER]) {
-  uint32_t live = 0;
+                                                 float (&cw)[ST_PER]) {
+  uint32_t live = EDGE ? 0u : (1u << ST_PER) - 1u;
 #pragma unroll
   for (int q = 0; q < ST_PER / 4; ++q) {
     const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
     const float xs[4] = {x.q[q].x, x.q[q].y, x.q[q].z, x.q[q].w};
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const uint32_t idx = pos + k;
-      const bool in = idx - r.lead < r.span - r.lead;
-      if (in) live |= 1u << (q * 4 + k);
-      wd[q * 4 + k] = (double)masked_weight(xs[k], in);
+      if constexpr (EDGE) {
+        const uint32_t idx = pos + k;
+        const bool in = idx - r.lead < r.span - r.lead;
+        if (in) live |= 1u << (q * 4 + k);
+        cw[q * 4 + k] = masked_weight(xs[k], in);
+      } else {
+        cw[q * 4 + k] = clamp_weight(xs[k]);
+      }
     }
   }
   return live;
@@ -181,10 +194,13 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     const RawChunk cur = nx;
     if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
     if (!wave_in_row(r, c, wave)) continue;
-    double wd[ST_PER];
-    unpack_chunk(cur, r, c, tid, wd);
+    float cw[ST_PER];
+    if (wave_inside_row(r, c, wave))
+      unpack_chunk<false>(cur, r, c, tid, cw);
+    else
+      unpack_chunk<true>(cur, r, c, tid, cw);
 #pragma unroll
-    for (int j = 0; j < ST_PER; ++j) wsum3_add(sum, wd[j]);
+    for (int j = 0; j < ST_PER; ++j) wsum3_add(sum, (double)cw[j]);
   }
   sum = group_sum_wsum3<64>(sum);
   if (lane == 0) s_w[wave] = sum;
@@ -212,7 +228,6 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   // t = fma(p, 2^F, -2^F) are monotone, heavy iff t >= 0.5), so one compare against the smallest heavy weight
   // of this row decides it; the surplus is then computed for the heavies alone, from the compacted list.
   uint32_t thr_bits;  // bit pattern of the smallest clamped weight that is heavy (above 2^32: none is)
-  bool thr_ok;        // false: the boundary was not found where it must be; every entry is classified in full
   {
     auto is_heavy = [&](uint32_t bits) {
       const double p = (double)__uint_as_float(bits) * L.scale;
@@ -222,15 +237,22 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     constexpr uint32_t MAXW = 0x4F800000u;  // 2^32
     uint32_t bits = est >= 4294967296.0 ? MAXW : __float_as_uint((float)est);
     int guard = 0;
-    while (bits > 0 && is_heavy(bits - 1) && guard < 64) {
+    while (bits > 0 && is_heavy(bits - 1) && guard < 8) {
       --bits;
       ++guard;
     }
-    while (bits <= MAXW && !is_heavy(bits) && guard < 64) {
+    while (bits <= MAXW && !is_heavy(bits) && guard < 8) {
       ++bits;
       ++guard;
     }
-    thr_ok = guard < 64;  // the estimate is within a step or two of the boundary
+    if (guard >= 8) {  // the estimate is normally within a step or two of the boundary; if not, bisect for it
+      uint32_t lo = 0, hi = MAXW + 1;  // smallest pattern in [0, MAXW + 1) that is heavy, MAXW + 1 if none
+      while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo) / 2;
+        if (is_heavy(mid)) hi = mid; else lo = mid + 1;
+      }
+      bits = lo;
+    }
     thr_bits = bits;
   }
   float* s_w32 = reinterpret_cast<float*>(s_sh);  // weight of heavy h in the low half of s_sh[h], until its prefix replaces it
@@ -251,20 +273,17 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
       float cw[ST_PER];
       uint32_t heavy = 0;
-      if (wave_in_row(r, c, wave))
+      if (wave_in_row(r, c, wave)) {
+        uint32_t live;
+        if (wave_inside_row(r, c, wave))
+          live = unpack_chunk<false>(cur, r, c, tid, cw);
+        else
+          live = unpack_chunk<true>(cur, r, c, tid, cw);
 #pragma unroll
-        for (int q = 0; q < ST_PER / 4; ++q) {
-          const uint32_t pos = c * ST_CH + (uint32_t)ST_PER * tid + 4u * q;
-          const float xs[4] = {cur.q[q].x, cur.q[q].y, cur.q[q].z, cur.q[q].w};
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const uint32_t idx = pos + k;
-            cw[q * 4 + k] = clamp_weight(xs[k]);
-            const bool hv = thr_ok ? __float_as_uint(cw[q * 4 + k]) >= thr_bits
-                                   : classify_fast((double)cw[q * 4 + k], true, L).heavy;
-            if (idx - r.lead < r.span - r.lead && hv) heavy |= 1u << (q * 4 + k);
-          }
-        }
+        for (int j = 0; j < ST_PER; ++j)
+          if (__float_as_uint(cw[j]) >= thr_bits) heavy |= 1u << j;
+        heavy &= live;
+      }
       uint32_t ex_c, tot_c;
       stream_excl_c((uint32_t)__popc(heavy), s_c[c & 1], ex_c, tot_c);
       uint32_t rank = cnt + ex_c;
@@ -351,17 +370,27 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       uint32_t heavy = 0;
       uint64_t run = 0;
       if (on) {
-        double wd[ST_PER];
-        live = unpack_chunk(cur, r, c, tid, wd);
+        float cw[ST_PER];
+        if (wave_inside_row(r, c, wave))
+          live = unpack_chunk<false>(cur, r, c, tid, cw);
+        else
+          live = unpack_chunk<true>(cur, r, c, tid, cw);
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
-          // only the lights' amounts are used here, and a deficit stays below 2^F: the short rounding will do
-          const Entry e = classify_small_unmasked(wd[j], L);
-          const bool in = (live >> j) & 1;
-          op[j] = (float)e.p;
-          dl[j] = (e.heavy || !in) ? 0 : e.amount;
+          // only the lights' amounts are used here: |t| <= 2^F, so the sum with 2^52 holds rint(|t|) in its low bits
+          // (0 for a light with 0 < t < 0.5).  Heavy slots and slots outside the row come out as anything and are dropped.
+          const double pj = (double)cw[j] * L.scale;
+          const double t = (pj - 1.0) * L.fs;
+          op[j] = (float)pj;
+          dl[j] = (uint64_t)__double_as_longlong(fabs(t) + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
+          if (__float_as_uint(cw[j]) >= thr_bits) heavy |= 1u << j;
+        }
+        heavy &= live;
+        const uint32_t light = live & ~heavy;
+#pragma unroll
+        for (int j = 0; j < ST_PER; ++j) {
+          dl[j] = ((light >> j) & 1) ? dl[j] : 0;
           run += dl[j];
-          if (e.heavy) heavy |= 1u << j;
         }
       }
       uint64_t ex_d, tot_d;
@@ -384,27 +413,25 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
         uint32_t oa[ST_PER];
         uint32_t wr = 0;  // entries this window writes: its lights, and heavies as placeholders unless an earlier window owns them
         uint32_t hrank = carry_c + ex_c;
+        // One path for every slot: a heavy slot, or one outside the row, adds no deficit, so the list does not move.
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
-          const uint32_t idx = pos0 + j;
-          oa[j] = idx - r.lead;
-          if (!((live >> j) & 1)) continue;
-          if ((heavy >> j) & 1) {
-            op[j] = 1.0f;
-            if (hrank >= hb) wr |= 1u << j;
-            ++hrank;
-            continue;
-          }
-          // the light's alias is the first heavy whose surplus prefix exceeds sl: in this window iff
+          const bool lv = (live >> j) & 1, hj = (heavy >> j) & 1;
+          // a light's alias is the first heavy whose surplus prefix exceeds sl: in this window iff
           // sh_lo <= sl < sh_hi, or beyond every heavy of the row
-          if (whole_row || (sl >= sh_lo && (sl < sh_hi || !more))) wr |= 1u << j;
-          if (any_heavy) oa[j] = hslot - r.lead;
+          const bool w = whole_row ? lv : hj ? hrank >= hb : lv && sl >= sh_lo && (sl < sh_hi || !more);
+          if (w) wr |= 1u << j;
+          oa[j] = (lv && !hj && any_heavy ? hslot : pos0 + (uint32_t)j) - r.lead;
+          op[j] = hj ? 1.0f : op[j];
+          hrank += hj ? 1u : 0u;
           // heavies of the window whose surplus prefix lies in (sl, sl + D]: this light finishes them
           sl += dl[j];
-          while (hv <= sl) {
-            s_prob[b] = residual_prob(L.one + hv - sl, L);
-            ++b;
-            hv = s_sh[b];
+          if (hv <= sl) {
+            do {
+              s_prob[b] = residual_prob(L.one + hv - sl, L);
+              ++b;
+              hv = s_sh[b];
+            } while (hv <= sl);
             hslot = s_slot[b];
           }
         }
