@@ -189,6 +189,9 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      "stream_wide_min_edges" (default 134217216): the rows of more than 65533 entries among them keep a workgroup
  *      busy for up to 1.5 ms; they join that kernel only when the build holds at least this many entries in rows
  *      of 8190..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
+ *      "build_streams" (default 1): a build of 2 M .. 1 G entries without per-kernel timing sends the kernels of
+ *      its degree classes out over the graph's stream and three side streams (small builds are bound by one
+ *      kernel waiting for the one before); 0 keeps every kernel on the graph's stream.  Same tables.
  *      "build_profile" (default 0): 1 records a HIP event after every kernel of sky_alias_build_all for
  *      sky_last_build_profile (about 3 microseconds each; a small graph pays 20 % of its build for them).
  *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:

@@ -972,6 +972,8 @@ static uint64_t g_stream_wide_min_edges = 512ull * (STREAM_MAX_DEG / 2);  // 512
 void set_stream_wide_min_edges(uint64_t n) { g_stream_wide_min_edges = n; }
 static bool g_build_profile = false;
 void set_build_profile(bool on) { g_build_profile = on; }
+static bool g_build_streams = true;
+void set_build_streams(bool on) { g_build_streams = on; }
 void set_stream_min_edges(uint64_t n) { g_stream_min_edges = n; }
 void set_row_merge(bool on) { g_row_merge = on; }
 
@@ -999,7 +1001,66 @@ void pool_release(sky_graph* g) {
     if (e) (void)hipEventDestroy(e);
     e = nullptr;
   }
+  for (hipStream_t& s : g->side) {
+    if (s) (void)hipStreamDestroy(s);
+    s = nullptr;
+  }
+  for (hipEvent_t& e : g->join_ev) {
+    if (e) (void)hipEventDestroy(e);
+    e = nullptr;
+  }
+  if (g->fork_ev) (void)hipEventDestroy(g->fork_ev);
+  g->fork_ev = nullptr;
 }
+
+// The class kernels of one build are independent of one another once the binning pass has run.  A small build is
+// bound by launching them one after another (a class of a few hundred rows takes as long as one row), so it sends
+// them out in turn over the graph's stream and three side streams; the graph's stream waits for the others at
+// the end.  Not used when every kernel is timed on its own, nor for builds so large that each kernel fills the GPU.
+constexpr uint64_t FAN_MIN_EDGES = 2000000, FAN_MAX_EDGES = 1ull << 30;
+struct StreamFan {
+  sky_graph* g;
+  hipStream_t main;
+  bool on = false, used[sky_graph::SIDE_STREAMS] = {false, false, false};
+  int turn = 0;
+  StreamFan(sky_graph* g_, hipStream_t m) : g(g_), main(m) {}
+  int start() {  // after the binning pass has been enqueued on the graph's stream
+    for (int k = 0; k < sky_graph::SIDE_STREAMS; ++k) {
+      if (!g->side[k]) SKY_HIP(hipStreamCreateWithFlags(&g->side[k], hipStreamNonBlocking));
+      if (!g->join_ev[k]) SKY_HIP(hipEventCreateWithFlags(&g->join_ev[k], hipEventDisableTiming));
+    }
+    if (!g->fork_ev) SKY_HIP(hipEventCreateWithFlags(&g->fork_ev, hipEventDisableTiming));
+    SKY_HIP(hipEventRecord(g->fork_ev, main));
+    for (int k = 0; k < sky_graph::SIDE_STREAMS; ++k) SKY_HIP(hipStreamWaitEvent(g->side[k], g->fork_ev, 0));
+    on = true;
+    return SKY_OK;
+  }
+  hipStream_t next() {
+    if (!on) return main;
+    const int k = turn++ % (sky_graph::SIDE_STREAMS + 1);
+    if (k == sky_graph::SIDE_STREAMS) return main;
+    used[k] = true;
+    return g->side[k];
+  }
+  int join() {
+    if (!on) return SKY_OK;
+    on = false;
+    for (int k = 0; k < sky_graph::SIDE_STREAMS; ++k)
+      if (used[k]) {
+        SKY_HIP(hipEventRecord(g->join_ev[k], g->side[k]));
+        SKY_HIP(hipStreamWaitEvent(main, g->join_ev[k], 0));
+      }
+    return SKY_OK;
+  }
+  ~StreamFan() { (void)join(); }  // an error in between still leaves the graph's stream behind every kernel
+};
+// The graph's stream replaced for the duration of a call that takes it from the graph.
+struct StreamSwap {
+  sky_graph* g;
+  hipStream_t saved;
+  StreamSwap(sky_graph* g_, hipStream_t s) : g(g_), saved(g_->stream) { g->stream = s; }
+  ~StreamSwap() { g->stream = saved; }
+};
 
 int EventTimer::mark(const char* name, uint64_t e) {
   hipEvent_t x;
@@ -1113,12 +1174,16 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   }
   if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
   RowRef* const vlist = sc.vlist;
+  uint64_t call_edges = 0;
+  for (int c = 0; c < CLS_COUNT; ++c) call_edges += host.edges[c];
+  StreamFan fan(g, st);
+  if (!tm && g_build_streams && call_edges >= FAN_MIN_EDGES && call_edges < FAN_MAX_EDGES) SKY_TRY(fan.start());
 
   auto grp = [&](int cls, auto kernel, int G, const char* name) -> int {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const uint32_t per_block = 256 / G;
-      hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, st, vlist + starts[cls],
+      hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, fan.next(), vlist + starts[cls],
                          cnt, g->adjwgt, g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
@@ -1134,7 +1199,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const size_t bytes = (size_t)rowt * 4 * t * 16;
-      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
+      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(), vlist + starts[cls], g->xadj, g->adjwgt,
                          g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
@@ -1143,7 +1208,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const size_t bytes = ((size_t)rowt * per + 2) * 14;
-      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, st, vlist + starts[cls], g->xadj, g->adjwgt,
+      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(), vlist + starts[cls], g->xadj, g->adjwgt,
                          g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
@@ -1181,6 +1246,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       else {  // this variant has no kernel for rows of 4094..8189 entries: tile-parallel path
         if (counts[cls]) {
           uint32_t skipped = 0;
+          SKY_TRY(fan.join());  // the tile-parallel path's scratch serves one call at a time
           SKY_TRY(build_rows_tiled(g, vlist + starts[cls], counts[cls], &skipped, nullptr, 0));
           if (skipped) return fail(SKY_ERR_STATE, "tiled_max_tiles below 9 needs row_merge");
         }
@@ -1201,6 +1267,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   const bool wide_streamed = !stream_to_tiled && all_stream_edges >= g_stream_wide_min_edges;
   const uint32_t wide_rows = wide_streamed ? counts[CLS_STREAM_WIDE] : 0;
   if (!stream_to_tiled && narrow_rows + wide_rows) {
+    StreamSwap sw(g, fan.next());
     SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], wide_rows, vlist + starts[CLS_STREAM], narrow_rows));
     if (tm) SKY_TRY(tm->mark("stream", narrow_edges + (wide_streamed ? host.edges[CLS_STREAM_WIDE] : 0)));
   }
@@ -1212,7 +1279,11 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   if (tiled_rows) {
     const uint32_t cnt = tiled_rows;
     uint32_t skipped = 0;
-    SKY_TRY(build_rows_tiled(g, tiled_list, cnt, &skipped, tm, tiled_edges));
+    {
+      StreamSwap sw(g, fan.next());
+      SKY_TRY(build_rows_tiled(g, tiled_list, cnt, &skipped, tm, tiled_edges));
+    }
+    SKY_TRY(fan.join());
     if (skipped) {  // rows with more tiles than the tile-parallel path takes: one workgroup streams each
       const uint32_t max_tiles = tiled_max_tiles();
       if (sc.huge_cap < cnt) {
@@ -1240,7 +1311,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       if (tm) SKY_TRY(tm->mark("streamed", 0));
     }
   }
-  return SKY_OK;
+  return fan.join();
 }
 
 int build_all_tables(sky_graph* g, double* seconds) {

@@ -37,6 +37,12 @@ struct sky_graph {
   };
   PoolBuf pool[POOL_SLOTS];
   hipEvent_t ev[2] = {nullptr, nullptr};
+  // Side streams (default priority) over which a small build spreads its class kernels, the event they wait for
+  // and the events the graph's stream waits for afterwards; created on first use.
+  static constexpr int SIDE_STREAMS = 3;
+  hipStream_t side[SIDE_STREAMS] = {nullptr, nullptr, nullptr};
+  hipEvent_t fork_ev = nullptr;
+  hipEvent_t join_ev[SIDE_STREAMS] = {nullptr, nullptr, nullptr};
 
   // Class sizes of the last binning of all vertices.  They depend on xadj alone, which never changes, so a
   // later build of all vertices sizes its launches from them without waiting for the device.
@@ -108,6 +114,7 @@ int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, 
 void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);
 void set_stream_wide_min_edges(uint64_t n);
+void set_build_streams(bool on);
 void set_build_profile(bool on);
 void set_online_full_build(int mode);
 void set_walk_compact_every(uint32_t steps);

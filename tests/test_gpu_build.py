@@ -54,6 +54,24 @@ def test_every_degree_class(orc, dist):
     build_and_compare(orc, xadj, adjncy, w, "classes/" + dist)
 
 
+def test_class_kernels_over_side_streams_give_the_same_table(orc):
+    # a build of 2 M .. 1 G entries spreads its class kernels over side streams; option build_streams = 0 keeps
+    # them on the graph's stream
+    from skywalker_amd import capi
+    rng = np.random.default_rng(21)
+    degs = EDGE_DEGREES[:60] + list(rng.integers(1, 300, 3000)) + list(rng.integers(300, 9000, 400)) + [30_000, 70_000, 600_000]
+    rng.shuffle(degs)
+    xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal")
+    assert 2_000_000 <= len(w) < (1 << 30)
+    for on in (0, 1):
+        capi.set_option("build_streams", on)
+        try:
+            for rep in range(2):  # twice: the second build finds the side streams and their events in place
+                build_and_compare(orc, xadj, adjncy, w, "side streams %d" % on)
+        finally:
+            capi.set_option("build_streams", 1)
+
+
 def test_unaligned_row_starts(orc):
     # rows of every residue mod 4 in front of each LDS-class row
     rng = np.random.default_rng(5)
