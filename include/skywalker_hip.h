@@ -189,6 +189,12 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      "stream_wide_min_edges" (default 134217216): the rows of more than 65533 entries among them keep a workgroup
  *      busy for up to 1.5 ms; they join that kernel only when the build holds at least this many entries in rows
  *      of 8190..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
+ *      "sample_distinct" (default 0): 1 makes sky_sample_offline and sky_sample_online give every parent distinct
+ *      children, the rule of the reference's online sampler (roll_atomic / roll_once, src/online_sample_new.cu:72-105),
+ *      in a form that does not depend on scheduling: draw i of a parent tries up to 11 candidates (Philox counter
+ *      word 2 = hop + 256 * try) and keeps the first slot of the row that no earlier draw of the parent kept; a draw
+ *      whose candidates were all kept already adds nothing, so sample_lengths may be below the fanout.  Fanouts of
+ *      at most 64, at most 256 hops (SKY_ERR_LIMIT otherwise).
  *      "build_streams" (default 1): a build of 2 M .. 1 G entries without per-kernel timing sends the kernels of
  *      its degree classes out over the graph's stream and three side streams (small builds are bound by one
  *      kernel waiting for the one before); 0 keeps every kernel on the graph's stream.  Same tables.

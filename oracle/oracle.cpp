@@ -565,9 +565,22 @@ int orc_walk_node2vec_reject(const uint32_t* xadj, uint32_t V, const uint32_t* a
 // A parent with an invalid row (zero total weight) yields no children (CheckValid, offline_sample.cu:86).
 // Slots that receive no vertex are not written.
 // online != 0 rebuilds each parent's table from w with the sweep instead of reading prob/alias.
+// distinct != 0 is the rule of the reference's online sampler (roll_atomic / roll_once, src/online_sample_new.cu:72-105:
+// up to 11 rounds of draws, a candidate whose slot of the row is already selected is dropped, so a parent may end
+// with fewer than k children), made sequential so that it does not depend on scheduling: draw i tries
+//   r = Philox(seed; seed_index, s*k + i, h + 256 t, DOM_SAMPLE), t = 0..10
+// and takes the first candidate slot that no earlier draw of this parent took; a draw whose 11 candidates were
+// all taken yields nothing.  The children are written densely in the order of i.  Needs k <= 64 and hops <= 256.
+constexpr uint32_t SAMPLE_ROUNDS = 11;
 static int sample_impl(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* w, const float* prob,
-                       const uint32_t* alias, int online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout,
-                       uint32_t hops, uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled) {
+                       const uint32_t* alias, int online, int distinct, const uint32_t* seeds, uint32_t N,
+                       const uint32_t* fanout, uint32_t hops, uint64_t seed, uint32_t* data, uint32_t* sample_lengths,
+                       uint64_t* sampled) {
+  if (distinct) {
+    if (hops > 256) return -1;
+    for (uint32_t h = 1; h < hops; ++h)
+      if (fanout[h] > 64) return -1;
+  }
   // fanout[0..hops-1], fanout[0] == 1
   std::vector<uint64_t> width(hops), off(hops), loff(hops);
   uint64_t lps = 0, slen = 0, wd = 1;
@@ -615,6 +628,22 @@ static int sample_impl(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy,
           if (k >= deg) {
             cnt = deg;
             for (uint32_t i = 0; i < deg; ++i) out[i] = adjncy[o + i];
+          } else if (distinct) {
+            uint32_t taken[64];
+            cnt = 0;
+            for (uint32_t i = 0; i < k; ++i)
+              for (uint32_t t = 0; t < SAMPLE_ROUNDS; ++t) {
+                uint32_t r[4];
+                philox(seed, (uint32_t)si, (uint32_t)(s * k + i), h + 256u * t, DOM_SAMPLE, r);
+                const uint32_t col = mulhi32(r[0], deg);
+                const uint32_t cand = u24(r[1]) < pr[col] ? col : al[col];
+                bool seen = false;
+                for (uint32_t j = 0; j < cnt; ++j) seen = seen || taken[j] == cand;
+                if (seen) continue;
+                taken[cnt] = cand;
+                out[cnt++] = adjncy[o + cand];
+                break;
+              }
           } else {
             cnt = k;
             for (uint32_t i = 0; i < k; ++i) {
@@ -640,13 +669,26 @@ static int sample_impl(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy,
 int orc_sample_offline(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* prob, const uint32_t* alias,
                        const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops, uint64_t seed,
                        uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled) {
-  return sample_impl(xadj, V, adjncy, nullptr, prob, alias, 0, seeds, N, fanout, hops, seed, data, sample_lengths,
+  return sample_impl(xadj, V, adjncy, nullptr, prob, alias, 0, 0, seeds, N, fanout, hops, seed, data, sample_lengths,
                      sampled);
 }
 int orc_sample_online(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* w, const uint32_t* seeds, uint32_t N,
                       const uint32_t* fanout, uint32_t hops, uint64_t seed, uint32_t* data, uint32_t* sample_lengths,
                       uint64_t* sampled) {
-  return sample_impl(xadj, V, adjncy, w, nullptr, nullptr, 1, seeds, N, fanout, hops, seed, data, sample_lengths,
+  return sample_impl(xadj, V, adjncy, w, nullptr, nullptr, 1, 0, seeds, N, fanout, hops, seed, data, sample_lengths,
+                     sampled);
+}
+// The same two with distinct children per parent (see sample_impl); -1 for a fanout above 64 or more than 256 hops.
+int orc_sample_offline_distinct(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* prob,
+                                const uint32_t* alias, const uint32_t* seeds, uint32_t N, const uint32_t* fanout,
+                                uint32_t hops, uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled) {
+  return sample_impl(xadj, V, adjncy, nullptr, prob, alias, 0, 1, seeds, N, fanout, hops, seed, data, sample_lengths,
+                     sampled);
+}
+int orc_sample_online_distinct(const uint32_t* xadj, uint32_t V, const uint32_t* adjncy, const float* w,
+                               const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops, uint64_t seed,
+                               uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled) {
+  return sample_impl(xadj, V, adjncy, w, nullptr, nullptr, 1, 1, seeds, N, fanout, hops, seed, data, sample_lengths,
                      sampled);
 }
 

@@ -54,6 +54,8 @@ def lib():
                                      _u32p, _u32p, C.POINTER(C.c_uint64)]
     L.orc_sample_online.argtypes = [_u32p, C.c_uint32, _u32p, _f32p, _u32p, C.c_uint32, _u32p, C.c_uint32, C.c_uint64, _u32p,
                                     _u32p, C.POINTER(C.c_uint64)]
+    L.orc_sample_offline_distinct.argtypes = L.orc_sample_offline.argtypes
+    L.orc_sample_online_distinct.argtypes = L.orc_sample_online.argtypes
     L.orc_num_threads.restype = C.c_int
     _lib = L
     return L
@@ -177,28 +179,34 @@ def sample_layout(fanout):
     return lps, slen, offs, loffs
 
 
-def sample_offline(xadj, adjncy, prob, alias, seeds, fanout, seed):
+def sample_offline(xadj, adjncy, prob, alias, seeds, fanout, seed, distinct=False):
+    """distinct: children of a parent are distinct slots of its row (the reference's online rule), at most 11 tries each."""
     N = len(seeds)
     fan = np.asarray(fanout, np.uint32)
     lps, slen, _, _ = sample_layout(list(fanout))
     data = np.full((N, lps), FILL, np.uint32)
     sl = np.zeros((N, slen), np.uint32)
     sampled = C.c_uint64(0)
-    lib().orc_sample_offline(xadj, len(xadj) - 1, adjncy, prob, alias, np.ascontiguousarray(seeds, np.uint32), N, fan, len(fan),
-                             seed, data, sl, C.byref(sampled))
+    fn = lib().orc_sample_offline_distinct if distinct else lib().orc_sample_offline
+    rc = fn(xadj, len(xadj) - 1, adjncy, prob, alias, np.ascontiguousarray(seeds, np.uint32), N, fan, len(fan),
+            seed, data, sl, C.byref(sampled))
+    if rc:
+        raise ValueError("distinct sampling needs fanouts <= 64 and at most 256 hops")
     return data, sl, sampled.value
 
 
-def sample_online(xadj, adjncy, w, seeds, fanout, seed):
+def sample_online(xadj, adjncy, w, seeds, fanout, seed, distinct=False):
     N = len(seeds)
     fan = np.asarray(fanout, np.uint32)
     lps, slen, _, _ = sample_layout(list(fanout))
     data = np.full((N, lps), FILL, np.uint32)
     sl = np.zeros((N, slen), np.uint32)
     sampled = C.c_uint64(0)
-    lib().orc_sample_online(xadj, len(xadj) - 1, adjncy, np.ascontiguousarray(w, np.float32),
-                            np.ascontiguousarray(seeds, np.uint32), N, fan, len(fan), seed, data, sl,
-                            C.byref(sampled))
+    fn = lib().orc_sample_online_distinct if distinct else lib().orc_sample_online
+    rc = fn(xadj, len(xadj) - 1, adjncy, np.ascontiguousarray(w, np.float32),
+            np.ascontiguousarray(seeds, np.uint32), N, fan, len(fan), seed, data, sl, C.byref(sampled))
+    if rc:
+        raise ValueError("distinct sampling needs fanouts <= 64 and at most 256 hops")
     return data, sl, sampled.value
 
 

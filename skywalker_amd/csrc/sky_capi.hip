@@ -380,6 +380,10 @@ int sky_set_option(const char* name, long value) {
     set_stream_min_edges((uint64_t)value);
     return SKY_OK;
   }
+  if (!strcmp(name, "sample_distinct")) {
+    set_sample_distinct(value != 0);
+    return SKY_OK;
+  }
   if (!strcmp(name, "build_streams")) {
     set_build_streams(value != 0);
     return SKY_OK;

@@ -84,6 +84,50 @@ __global__ __launch_bounds__(256) void sample_hop_kernel(const uint32_t* __restr
   }
 }
 
+// Distinct children (the rule of the reference's online sampler, roll_atomic / roll_once of
+// src/online_sample_new.cu:72-105: up to 11 rounds, a candidate whose slot of the row is already selected is
+// dropped, a parent may end with fewer than k children), made sequential so that the result does not depend on
+// scheduling: draw i of slot s tries Philox(seed; seed index, s*k + i, h + 256 t, DOM_SAMPLE) for t = 0..10 and
+// keeps the first candidate slot that no earlier draw of this parent kept; the children are written densely in
+// the order of i.  One lane per (seed, slot); the slots it has kept so far sit in LDS, one column per lane.
+constexpr int DISTINCT_T = 128;          // threads per workgroup
+constexpr uint32_t DISTINCT_MAX_K = 64;  // largest fanout of this rule
+constexpr uint32_t DISTINCT_ROUNDS = 11;
+__global__ __launch_bounds__(DISTINCT_T) void sample_hop_distinct_kernel(
+    const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy, const AliasEntry* __restrict__ table,
+    const int8_t* __restrict__ valid, uint64_t total, uint32_t V, HopGeom g, uint64_t seed,
+    uint32_t* __restrict__ data, uint32_t* __restrict__ sl) {
+  __shared__ uint32_t s_taken[DISTINCT_MAX_K][DISTINCT_T];
+  const uint64_t tid = (uint64_t)blockIdx.x * DISTINCT_T + threadIdx.x;
+  if (tid >= total) return;
+  const uint64_t si = tid / g.width, s = tid % g.width;
+  if (!slot_filled(g, sl, si, s)) return;
+  const uint32_t v = data[si * g.lps + g.off + s];
+  if (v >= V || !valid[v]) return;
+  const uint32_t o = xadj[v], deg = xadj[v + 1] - o;
+  if (deg == 0) return;
+  uint32_t* out = data + si * g.lps + g.off_next + s * g.k;
+  uint32_t cnt = 0;
+  if (g.k >= deg) {
+    for (; cnt < deg; ++cnt) out[cnt] = adjncy[o + cnt];
+  } else {
+    for (uint32_t i = 0; i < g.k; ++i)
+      for (uint32_t t = 0; t < DISTINCT_ROUNDS; ++t) {
+        const u32x4 r = philox(seed, (uint32_t)si, (uint32_t)(s * g.k + i), g.h + 256u * t, DOM_SAMPLE);
+        const uint32_t col = __umulhi(r.x, deg);
+        const AliasEntry e = table[o + col];
+        const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
+        bool seen = false;
+        for (uint32_t j = 0; j < cnt; ++j) seen = seen || s_taken[j][threadIdx.x] == cand;
+        if (seen) continue;
+        s_taken[cnt][threadIdx.x] = cand;
+        out[cnt++] = adjncy[o + cand];
+        break;
+      }
+  }
+  sl[si * g.slen + g.loff + s] = cnt;
+}
+
 // Sampled edges of the call = sum of sample_lengths (as the reference counts them, src/main.cu:378-394): one pass
 // at the end, one atomic per workgroup; a counter bumped by every wavefront of every hop is a hot spot.
 __global__ __launch_bounds__(256) void sum_u32_kernel(const uint32_t* __restrict__ x, uint64_t n,
@@ -145,9 +189,18 @@ __global__ __launch_bounds__(256) void sample_init_kernel(const uint32_t* __rest
   if (i < N) data[(uint64_t)i * lps] = seeds[i];
 }
 
+static bool g_sample_distinct = false;
+void set_sample_distinct(bool on) { g_sample_distinct = on; }
+
 int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
                 uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds) {
   hipStream_t st = g->stream;
+  const bool distinct = g_sample_distinct;
+  if (distinct) {
+    if (hops > 256) return fail(SKY_ERR_LIMIT, "sample: distinct children need at most 256 hops");
+    for (uint32_t h = 1; h < hops; ++h)
+      if (fanout[h] > DISTINCT_MAX_K) return fail(SKY_ERR_LIMIT, "sample: distinct children need fanouts of at most 64");
+  }
   if (g->has_tables) online = false;  // every row is already there: nothing to build on the way
   std::vector<uint64_t> width(hops), off(hops), loff(hops, 0);
   uint64_t lps = 0, slen = 0, wd = 1;
@@ -205,6 +258,13 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
       }
       const uint64_t total = (uint64_t)N * hg.width * hg.k;
       if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");
+      if (distinct) {
+        const uint64_t slots = (uint64_t)N * hg.width;
+        hipLaunchKernelGGL(sample_hop_distinct_kernel, dim3((uint32_t)((slots + DISTINCT_T - 1) / DISTINCT_T)),
+                           dim3(DISTINCT_T), 0, st, g->xadj, g->adjncy, g->table, g->valid, slots, g->V, hg, seed, data,
+                           sample_lengths);
+        continue;
+      }
       hipLaunchKernelGGL(sample_hop_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, g->xadj,
                          g->adjncy, g->table, g->valid, total, g->V, hg, seed, total <= 0xFFFFFFFFull, data,
                          sample_lengths);

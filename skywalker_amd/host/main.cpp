@@ -66,6 +66,9 @@ DEFINE_bool(csv, false, "CSV output");
 DEFINE_bool(weight, true, "load edge weight from file");
 // new here: the bias operator as a shared library (include/skywalker_bias.h) instead of a link-time choice
 DEFINE_string(biasplugin, "", "bias plug-in library, e.g. libskywalker_bias_degree.so (default: built-in static / node2vec bias)");
+// new here: the reference's online sampler never takes a slot of a row twice (roll_once, online_sample_new.cu:83-105),
+// its offline sampler may; here one flag selects the rule for both
+DEFINE_bool(replace, true, "k-hop sampling draws with replacement; 0: distinct neighbours (fanouts of at most 64)");
 // new here: key of the Philox streams (the reference seeds cuRAND with the thread id)
 DEFINE_int32(seed, 0, "Philox seed of the samplers");
 
@@ -107,6 +110,10 @@ int main(int argc, char* argv[]) {
   }
   if (!(FLAGS_tp >= 0.0 && FLAGS_tp <= 1.0) || !(FLAGS_p > 0.0) || !(FLAGS_q > 0.0)) {
     fprintf(stderr, "skywalker: need 0 <= --tp <= 1, --p > 0 and --q > 0\n");
+    return 1;
+  }
+  if (!FLAGS_replace && sky_set_option("sample_distinct", 1) != SKY_OK) {
+    fprintf(stderr, "skywalker: %s\n", sky_last_error());
     return 1;
   }
   int sample_size = FLAGS_n;

@@ -37,6 +37,38 @@ def test_offline_and_online_match_oracle(orc, fanout):
     assert osampled == int(osl.sum())
 
 
+@pytest.mark.parametrize("fanout", [[1, 25, 10], [1, 3, 2, 2], [1, 64]])
+def test_distinct_children_match_oracle(orc, fanout):
+    # option sample_distinct: the reference's online rule (no slot of a row twice, at most 11 tries per draw)
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(13, 8, 22)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 22, len(adjncy), 0.0, 2.0)  # skewed rows: tries do run out
+    seeds = orc.gen_seeds(5, 1 << 13, 1500)
+    lps, slen = capi.sample_layout(fanout)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    capi.set_option("sample_distinct", 1)
+    try:
+        d_on, sl_on, s_on, _ = g.sample_online(seeds, fanout, 23)
+        on = (d_on.to_host((1500, lps)), sl_on.to_host((1500, slen)))
+        g.build_tables()
+        d_off, sl_off, s_off, _ = g.sample_offline(seeds, fanout, 23)
+        off = (d_off.to_host((1500, lps)), sl_off.to_host((1500, slen)))
+        with pytest.raises(capi.SkyError):
+            g.sample_offline(seeds, [1, 65], 23)
+    finally:
+        capi.set_option("sample_distinct", 0)
+    prob, alias, valid = g.tables()
+    g.free()
+    odata, osl, osampled = orc.sample_offline(xadj, adjncy, prob, alias, seeds, fanout, 23, distinct=True)
+    assert np.array_equal(off[1], osl) and np.array_equal(off[0], odata) and s_off == osampled
+    assert np.array_equal(on[0], off[0]) and np.array_equal(on[1], off[1]) and s_on == s_off
+    assert osampled == int(osl.sum())
+    if fanout[1] >= 25:
+        deg = np.diff(xadj)
+        big = deg[seeds] > fanout[1]
+        assert (osl[big, 0] < fanout[1]).any()  # a parent that ended with fewer children than its fanout is among the cases
+
+
 def test_exact_count_when_every_degree_exceeds_fanout(orc):
     from skywalker_amd import capi
     rng = np.random.default_rng(6)

@@ -243,6 +243,32 @@ def test_cli_unbiased_two_hop_sampling(tmp_path, orc, online):
 
 
 @pytest.mark.gpu
+def test_cli_two_hop_sampling_without_replacement(tmp_path, orc):
+    # --replace=0: every parent's children are distinct slots of its row, as in the reference's online sampler
+    xadj, adjncy = orc.rmat_csr(11, 16, 25)
+    w = (orc.gen_weights(orc.W_UNIFORM, 25, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "nr.w.gr")
+    write_gr(p, xadj, adjncy, w)
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--sage", "--bias=1", "--ol=1", "--replace=0", "--input", p, "-n", "300",
+                        "--printresult", "--seed", "6"])
+    assert rc == 0, err
+    data, sl, sampled = orc.sample_online(xadj, adjncy, w.astype(np.float32), np.arange(300, dtype=np.uint32), [1, 25, 10], 6,
+                                          distinct=True)
+    blocks = out.split("th sample src: ")[1:]
+    assert len(blocks) == 4
+    for j, blk in enumerate(blocks):
+        m = re.match(r"(\d+), 1-hop len: (\d+)", blk)
+        assert int(m.group(1)) == j and int(m.group(2)) == sl[j, 0]
+        hop1 = [int(x) for x in blk.split("1-hop : ")[1].splitlines()[0].split()]
+        assert hop1 == data[j, 1:1 + sl[j, 0]].tolist()
+    lines = [l for l in out.splitlines() if l.strip()]
+    sample_ms, mseps = float(lines[-2]), float(lines[-1])
+    assert abs(mseps - sampled / (sample_ms * 1e-3) / 1e6) <= 0.02 * mseps + 0.02
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--replace=0", "--k", "70", "--d", "2", "--input", p, "-n", "10"])
+    assert rc != 0 and "64" in err
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("table", [False, True])
 def test_cli_unbiased_node2vec(tmp_path, orc, table):
     # --bias=0 --node2vec: the reference's unbiased node2vec walker (src/unbiased_walk.cu:14-60) = unit weights here

@@ -256,6 +256,81 @@ def test_sample_draw_law_and_online_equals_offline(orc):
     assert np.array_equal(data, d2) and np.array_equal(sl, sl2) and sampled == s2
 
 
+def distinct_law(p, k, rounds=11):
+    """Exact law of the ordered list of distinct slots that k draws leave: draw i tries up to `rounds` times and
+    keeps the first slot not taken yet; a draw whose tries all hit taken slots leaves nothing."""
+    dist = {(): 1.0}
+    for _ in range(k):
+        nxt = {}
+        for taken, pr in dist.items():
+            m = sum(p[c] for c in taken)
+            tries = sum(m ** t for t in range(rounds))  # a free slot c is kept with probability p[c] * sum_t m^t
+            nxt[taken] = nxt.get(taken, 0.0) + pr * m ** rounds
+            for c in range(len(p)):
+                if c not in taken:
+                    nxt[taken + (c,)] = nxt.get(taken + (c,), 0.0) + pr * p[c] * tries
+        dist = nxt
+    return dist
+
+
+def test_distinct_sampling_law_brute_force(orc):
+    # a row of five slots, one of which holds 70 % of the weight, so that tries do run out now and then
+    w = np.array([70.0, 12.0, 9.0, 6.0, 3.0], np.float32)
+    d, k = len(w), 3
+    xadj = np.zeros(d + 2, np.uint32)
+    xadj[1:] = d
+    adjncy = np.arange(1, d + 1, dtype=np.uint32)
+    prob, alias, _ = orc.alias_build(xadj, w)
+    N = 200000
+    data, sl, sampled = orc.sample_offline(xadj, adjncy, prob, alias, np.zeros(N, np.uint32), [1, k], 9, distinct=True)
+    assert sampled == int(sl.sum()) and sl.max() <= k
+    law = distinct_law((w.astype(np.float64) / w.sum(dtype=np.float64)).tolist(), k)
+    assert abs(sum(law.values()) - 1.0) < 1e-12
+    keys = sorted(law)
+    index = {key: i for i, key in enumerate(keys)}
+    counts = np.zeros(len(keys))
+    for row, n in zip(data, sl[:, 0]):
+        got = tuple(int(x) - 1 for x in row[1:1 + n])
+        assert len(set(got)) == len(got) and np.all(row[1 + n:] == orc.FILL)
+        counts[index[got]] += 1
+    expect = np.array([law[key] for key in keys])
+    rare = expect * N < 5  # pooled: too few expected for a chi-square cell of their own
+    c = np.append(counts[~rare], counts[rare].sum())
+    e = np.append(expect[~rare], expect[rare].sum())
+    assert chi_square_p(c[e > 0], e[e > 0]) > 0.01
+    assert (sl[:, 0] < k).mean() > 0.001  # the case of a draw that leaves nothing is in the sample
+    # same tables rebuilt on the way: same result
+    d2, sl2, s2 = orc.sample_online(xadj, adjncy, w, np.zeros(N, np.uint32), [1, k], 9, distinct=True)
+    assert np.array_equal(data, d2) and np.array_equal(sl, sl2) and sampled == s2
+    # the first child is the first draw of the rule with replacement (try 0 uses the same random numbers)
+    d3, _, _ = orc.sample_offline(xadj, adjncy, prob, alias, np.zeros(N, np.uint32), [1, k], 9)
+    assert np.array_equal(data[:, 1], d3[:, 1])
+
+
+def test_distinct_sampling_counts_and_limits(orc):
+    rng = np.random.default_rng(12)
+    V = 300
+    xadj, adjncy, w = graph_from_degrees(rng.integers(0, 60, V), rng, "lognormal", V=V)
+    prob, alias, valid = orc.alias_build(xadj, w)
+    seeds = rng.integers(0, V, 500, dtype=np.uint32)
+    data, sl, sampled = orc.sample_offline(xadj, adjncy, prob, alias, seeds, [1, 25, 10], 2, distinct=True)
+    deg = np.diff(xadj)
+    assert sampled == int(sl.sum())
+    for s in range(len(seeds)):
+        n = sl[s, 0]
+        if deg[seeds[s]] <= 25:
+            assert n == deg[seeds[s]] * valid[seeds[s]]
+        else:
+            assert 1 <= n <= 25
+        for j in range(n):
+            par = data[s, 1 + j]
+            m = sl[s, 1 + j]
+            assert m == deg[par] * valid[par] if deg[par] <= 10 else 1 <= m <= 10
+    import pytest
+    with pytest.raises(ValueError):
+        orc.sample_offline(xadj, adjncy, prob, alias, seeds, [1, 65], 2, distinct=True)
+
+
 def test_start_vertices_that_do_not_exist_never_move(orc):
     # every walk and the sampler record such a seed and stop there: length 0, no children
     xadj, adjncy = orc.rmat_csr(8, 8, 3)
