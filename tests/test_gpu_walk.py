@@ -173,6 +173,25 @@ def test_node2vec_rejection_bit_exact(orc, scale, ef, stop, p, q):
     assert sampled == osampled
 
 
+def test_node2vec_rejection_one_walker_per_lane_for_large_batches(orc):
+    # up to 262,144 walkers take 16 lanes each (they search the previous row together); larger batches one lane each
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 16, 35)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 35, len(adjncy), 0.0, 1.0)
+    seeds = orc.gen_seeds(8, 1 << 12, 300000)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    paths, lengths, sampled, _ = g.walk_online(capi.BIAS_NODE2VEC_REJECT, 2.0, 0.5, seeds, 10, 0.0, 19)
+    big = (paths.to_host((300000, 11)), lengths.to_host())
+    small, _, _, _ = g.walk_online(capi.BIAS_NODE2VEC_REJECT, 2.0, 0.5, seeds[:70000], 10, 0.0, 19)
+    small = small.to_host((70000, 11))
+    prob, alias, valid = g.tables()
+    g.free()
+    opaths, olengths, osampled = orc.walk_node2vec_reject(xadj, adjncy, prob, alias, 2.0, 0.5, seeds, 10, 0.0, 19)
+    assert np.array_equal(big[0], opaths) and np.array_equal(big[1], olengths) and sampled == osampled
+    assert np.array_equal(small, opaths[:70000])
+
+
 def test_node2vec_rejection_second_step_law(orc):
     # exact second-order law on a small graph, sampled on the device
     from skywalker_amd import capi
