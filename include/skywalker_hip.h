@@ -189,6 +189,10 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      "stream_wide_min_edges" (default 134217216): the rows of more than 65533 entries among them keep a workgroup
  *      busy for up to 1.5 ms; they join that kernel only when the build holds at least this many entries in rows
  *      of 8190..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
+ *      "walk_read_once" (default -1): 1 makes the walks load a step's table entry and neighbour id as read-once
+ *      data, which keeps the row offsets of the well-connected vertices in L2 on a graph whose tables are far larger
+ *      than the caches; 0 loads them as ordinary data (better when the tables fit the caches); -1 decides by the size of
+ *      the tables (read-once above 2 GiB).  Same paths.
  *      "sample_distinct" (default 0): 1 makes sky_sample_offline and sky_sample_online give every parent distinct
  *      children, the rule of the reference's online sampler (roll_atomic / roll_once, src/online_sample_new.cu:72-105),
  *      in a form that does not depend on scheduling: draw i of a parent tries up to 11 candidates (Philox counter

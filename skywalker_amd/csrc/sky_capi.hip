@@ -380,6 +380,11 @@ int sky_set_option(const char* name, long value) {
     set_stream_min_edges((uint64_t)value);
     return SKY_OK;
   }
+  if (!strcmp(name, "walk_read_once")) {
+    if (value < -1 || value > 1) return fail(SKY_ERR_ARG, "sky_set_option: walk_read_once is -1, 0 or 1");
+    set_walk_read_once((int)value);
+    return SKY_OK;
+  }
   if (!strcmp(name, "sample_distinct")) {
     set_sample_distinct(value != 0);
     return SKY_OK;

@@ -116,6 +116,7 @@ void set_stream_min_edges(uint64_t n);
 void set_stream_wide_min_edges(uint64_t n);
 void set_build_streams(bool on);
 void set_sample_distinct(bool on);
+void set_walk_read_once(int mode);
 void set_build_profile(bool on);
 void set_online_full_build(int mode);
 void set_walk_compact_every(uint32_t steps);

@@ -18,7 +18,7 @@ typedef uint32_t path4u __attribute__((ext_vector_type(4), aligned(4)));
 
 // One draw from the row of v.  With the walk index one 16-byte entry holds both possible next vertices (two
 // cache lines per step: xadj and the entry); without it the neighbour id is a third gather.
-template <bool INDEXED>
+template <bool INDEXED, bool ONCE>
 __device__ __forceinline__ bool walk_draw(const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
                                           const AliasEntry* __restrict__ table, const WalkEntry* __restrict__ index,
                                           const u32x4& r, uint32_t v, uint32_t& next) {
@@ -28,7 +28,8 @@ __device__ __forceinline__ bool walk_draw(const uint32_t* __restrict__ xadj, con
   if (INDEXED) {
     // like the table entry below: read once, so it should not push the row offsets out of L2
     typedef uint32_t idx4 __attribute__((ext_vector_type(4)));
-    const idx4 eb = __builtin_nontemporal_load(reinterpret_cast<const idx4*>(index + off + col));
+    const idx4* ep = reinterpret_cast<const idx4*>(index + off + col);
+    const idx4 eb = ONCE ? __builtin_nontemporal_load(ep) : *ep;
     WalkEntry e;
     e.prob = __uint_as_float(eb.x);
     e.alias = eb.y;
@@ -38,13 +39,14 @@ __device__ __forceinline__ bool walk_draw(const uint32_t* __restrict__ xadj, con
     if (!keep && e.alias == SKY_INVALID) return false;
     next = keep ? e.nbr_col : e.nbr_alias;
   } else {
-    // The entry and the neighbour id are read once per step, the row offsets of the well-connected vertices many
-    // times by many walkers: the two gathers go past the cache's usual replacement order so that they do not
-    // evict the offsets (1 M walkers x 80 steps on the scale-26 graph: 2.16 -> 1.86 ms).
-    const AliasEntry e = load_entry_once(table + off + col);
+    // On a graph whose tables are far larger than the caches the entry and the neighbour id are read once per
+    // step, the row offsets of the well-connected vertices many times by many walkers: the two gathers then go
+    // past the cache's usual replacement order so that they do not evict the offsets (1 M walkers x 80 steps on the
+    // scale-26 graph: 2.16 -> 1.86 ms).  On a small graph the entries are hit again and stay ordinary loads.
+    const AliasEntry e = ONCE ? load_entry_once(table + off + col) : table[off + col];
     const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
     if (cand == SKY_INVALID) return false;
-    next = __builtin_nontemporal_load(adjncy + off + cand);
+    next = ONCE ? __builtin_nontemporal_load(adjncy + off + cand) : adjncy[off + cand];
   }
   return true;
 }
@@ -53,7 +55,7 @@ __device__ __forceinline__ bool walk_draw(const uint32_t* __restrict__ xadj, con
 // their start vertex).  A walker that is still walking at s_end is appended to `next_live` when that list is
 // given: the next launch then runs on full wavefronts again (walkers that reached a vertex without out-edges
 // or stopped no longer hold a lane).  The vertices of WALK_STAGE steps leave as one store.
-template <bool INDEXED>
+template <bool INDEXED, bool ONCE>
 __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
     const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy, const AliasEntry* __restrict__ table,
     const WalkEntry* __restrict__ index, const uint32_t* __restrict__ seeds, const uint32_t* __restrict__ live,
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
         if (walking && s + got < s_end) {
           const u32x4 r = philox(seed, i, s + got, 0, DOM_WALK);
           uint32_t nx = 0;
-          if ((stop_prob > 0.0f && u24(r.z) < stop_prob) || !walk_draw<INDEXED>(xadj, adjncy, table, index, r, v, nx)) {
+          if ((stop_prob > 0.0f && u24(r.z) < stop_prob) || !walk_draw<INDEXED, ONCE>(xadj, adjncy, table, index, r, v, nx)) {
             walking = false;
           } else {
             v = nx;
@@ -143,15 +145,27 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
 
 static uint32_t g_walk_compact_every = 0;  // 0: one launch, every walker keeps its lane for the whole walk
 void set_walk_compact_every(uint32_t steps) { g_walk_compact_every = steps; }
+static int g_walk_read_once = -1;  // -1: by the size of the tables, 0 / 1: never / always load entries as read-once data
+void set_walk_read_once(int mode) { g_walk_read_once = mode; }
+// Tables of more than 2 GiB (the last-level cache holds 256 MiB) are gathered from as read-once data.
+static bool walk_reads_once(const sky_graph* g) {
+  return g_walk_read_once < 0 ? (uint64_t)g->E * sizeof(AliasEntry) > (2ull << 30) : g_walk_read_once != 0;
+}
 
 template <bool INDEXED>
 static void launch_walk(sky_graph* g, const uint32_t* seeds, const uint32_t* live, const uint32_t* n_live_dev,
                         uint32_t n_live, uint32_t len, uint32_t s_begin, uint32_t s_end, float stop_prob, uint64_t seed,
                         uint32_t* paths, uint32_t* lengths, uint32_t* next_live, uint32_t* n_next,
                         unsigned long long* sampled, unsigned long long* partials) {
-  hipLaunchKernelGGL(walk_offline_kernel<INDEXED>, dim3((n_live + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0,
-                     g->stream, g->xadj, g->adjncy, g->table, INDEXED ? g->walk_index : nullptr, seeds, live, n_live_dev, n_live, g->V, len,
-                     s_begin, s_end, stop_prob, seed, paths, lengths, next_live, n_next, sampled, partials);
+  const dim3 grid((n_live + WALK_BLOCK - 1) / WALK_BLOCK), block(WALK_BLOCK);
+  if (walk_reads_once(g))
+    hipLaunchKernelGGL((walk_offline_kernel<INDEXED, true>), grid, block, 0, g->stream, g->xadj, g->adjncy, g->table,
+                       INDEXED ? g->walk_index : nullptr, seeds, live, n_live_dev, n_live, g->V, len, s_begin, s_end, stop_prob,
+                       seed, paths, lengths, next_live, n_next, sampled, partials);
+  else
+    hipLaunchKernelGGL((walk_offline_kernel<INDEXED, false>), grid, block, 0, g->stream, g->xadj, g->adjncy, g->table,
+                       INDEXED ? g->walk_index : nullptr, seeds, live, n_live_dev, n_live, g->V, len, s_begin, s_end, stop_prob,
+                       seed, paths, lengths, next_live, n_next, sampled, partials);
 }
 
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,

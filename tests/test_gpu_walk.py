@@ -173,6 +173,32 @@ def test_node2vec_rejection_bit_exact(orc, scale, ef, stop, p, q):
     assert sampled == osampled
 
 
+def test_read_once_gathers_give_the_same_paths(orc):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 16, 36)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 36, len(adjncy), 0.0, 1.0)
+    seeds = orc.gen_seeds(9, 1 << 12, 3000)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    prob, alias, _ = g.tables()
+    want = orc.walk_offline(xadj, adjncy, prob, alias, seeds, 30, 0.02, 21)
+    try:
+        for mode in (0, 1):
+            for indexed in (False, True):
+                capi.set_option("walk_read_once", mode)
+                g.build_tables()
+                if indexed:
+                    g.build_walk_index()
+                paths, lengths, sampled, _ = g.walk_offline(seeds, 30, 0.02, 21)
+                assert np.array_equal(paths.to_host((3000, 31)), want[0]) and np.array_equal(lengths.to_host(), want[1])
+                assert sampled == want[2]
+        with pytest.raises(capi.SkyError):
+            capi.set_option("walk_read_once", 2)
+    finally:
+        capi.set_option("walk_read_once", -1)
+        g.free()
+
+
 def test_node2vec_rejection_one_walker_per_lane_for_large_batches(orc):
     # up to 262,144 walkers take 16 lanes each (they search the previous row together); larger batches one lane each
     from skywalker_amd import capi
