@@ -363,7 +363,7 @@ __device__ __forceinline__ bool row_has(const uint32_t* __restrict__ row, uint32
 __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_kernel(
     const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
     const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t V, uint32_t len,
-    float fp, float fq, float fmax, float stop_prob, uint64_t seed, uint32_t* __restrict__ paths,
+    float fp, float fq, float fmax, float stop_prob, uint64_t seed, bool once, uint32_t* __restrict__ paths,
     uint32_t* __restrict__ lengths, unsigned long long* __restrict__ sampled) {
   const uint32_t i = blockIdx.x * WALK_BLOCK + threadIdx.x;
   uint32_t s = 0;
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_kernel(
       for (uint32_t t = 0;; ++t) {
         if (t) r = philox(seed, i, s, t, DOM_WALK);
         const uint32_t col = __umulhi(r.x, deg);
-        const AliasEntry e = load_entry_once(table + off + col);
+        const AliasEntry e = once ? load_entry_once(table + off + col) : table[off + col];
         const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
         if (cand == SKY_INVALID) {
           dead = true;
@@ -436,7 +436,7 @@ __device__ __forceinline__ bool group_row_has(const uint32_t* __restrict__ row, 
 __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_group_kernel(
     const uint32_t* __restrict__ xadj, const uint32_t* __restrict__ adjncy,
     const AliasEntry* __restrict__ table, const uint32_t* __restrict__ seeds, uint32_t N, uint32_t V, uint32_t len,
-    float fp, float fq, float fmax, float stop_prob, uint64_t seed, uint32_t* __restrict__ paths,
+    float fp, float fq, float fmax, float stop_prob, uint64_t seed, bool once, uint32_t* __restrict__ paths,
     uint32_t* __restrict__ lengths, unsigned long long* __restrict__ sampled) {
   const uint32_t i = (blockIdx.x * WALK_BLOCK + threadIdx.x) / N2V_G;
   const bool first = (threadIdx.x & (N2V_G - 1)) == 0;  // the lane that writes for the group
@@ -455,7 +455,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_group_kernel(
       for (uint32_t t = 0;; ++t) {
         if (t) r = philox(seed, i, s, t, DOM_WALK);
         const uint32_t col = __umulhi(r.x, deg);
-        const AliasEntry e = load_entry_once(table + off + col);
+        const AliasEntry e = once ? load_entry_once(table + off + col) : table[off + col];
         const uint32_t cand = u24(r.y) < e.prob ? col : e.alias;
         if (cand == SKY_INVALID) {
           dead = true;
@@ -498,12 +498,12 @@ int walk_node2vec_reject(sky_graph* g, float p, float q, const uint32_t* seeds, 
     if (N && N <= N2V_GROUP_MAX_WALKERS)
       hipLaunchKernelGGL(walk_n2v_reject_group_kernel,
                          dim3((uint32_t)(((uint64_t)N * N2V_G + WALK_BLOCK - 1) / WALK_BLOCK)), dim3(WALK_BLOCK), 0, st,
-                         g->xadj, g->adjncy, g->table, seeds, N, g->V, len, fp, fq, fmax, stop_prob, seed, paths, lengths,
-                         d_sampled);
+                         g->xadj, g->adjncy, g->table, seeds, N, g->V, len, fp, fq, fmax, stop_prob, seed, walk_reads_once(g), paths,
+                         lengths, d_sampled);
     else if (N)
       hipLaunchKernelGGL(walk_n2v_reject_kernel, dim3((N + WALK_BLOCK - 1) / WALK_BLOCK), dim3(WALK_BLOCK), 0, st,
-                         g->xadj, g->adjncy, g->table, seeds, N, g->V, len, fp, fq, fmax, stop_prob, seed, paths, lengths,
-                         d_sampled);
+                         g->xadj, g->adjncy, g->table, seeds, N, g->V, len, fp, fq, fmax, stop_prob, seed, walk_reads_once(g), paths,
+                         lengths, d_sampled);
     SKY_TRY(tm.mark("walk", 0));
     double sec = 0;
     SKY_TRY(tm.finish(nullptr, &sec));
