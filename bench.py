@@ -204,7 +204,7 @@ def online_bench(args, cfg, capi, g, seeds, name, cus, t_gen, torch):
             alg_bytes = 12 * g.E + 5 * g.V + 24 * steps
             detail = {"formula": "12 E + 5 V (first-order tables) + 24 per step; the rejection trials' reads "
                                  "(12 + 4 log2 d_prev each) are not counted: a lower bound"}
-            kernel = "one batch: the offline build kernels, walk_n2v_reject_kernel"
+            kernel = "one batch: the offline build kernels, walk_n2v_reject_group_kernel"
     roofline = {"bound": "hbm", "kernel": kernel, "achieved": alg_bytes / ksec / 1e9, "peak": HBM_PEAK / 1e9,
                 "unit": "GB/s", "frac": alg_bytes / ksec / HBM_PEAK, "traffic": None,
                 "launch_ms": ksec * 1e3, "algorithmic_bytes_per_launch": alg_bytes, "detail": detail}
