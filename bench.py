@@ -38,7 +38,7 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "c5_kernel_traffic.txt")
 METRIC = "sampled edges/sec (SEPS) + alias-table build edges/sec on 1 MI355X; % HBM peak"
 ARITHMETIC = "f64 classification and exact three-limb sums, u64 fixed-point ledger, f32 tables, u32 indices"
 KERNEL_OF = {  # build_profile entry -> kernel symbol
-    "bin": "bin_count_kernel+bin_scatter_kernel", "lds_w1": "build_merge_kernel<64,4>",
+    "bin": "bin_count_kernel+bin_scatter_kernel", "small": "small_rows_kernel", "lds_w1": "build_merge_kernel<64,4>",
     "lds_w2": "build_merge_kernel<64,8>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",

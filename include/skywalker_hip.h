@@ -199,6 +199,9 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      word 2 = hop + 256 * try) and keeps the first slot of the row that no earlier draw of the parent kept; a draw
  *      whose candidates were all kept already adds nothing, so sample_lengths may be below the fanout.  Fanouts of
  *      at most 64, at most 256 hops (SKY_ERR_LIMIT otherwise).
+ *      "small_in_place" (default -1): 1 builds the rows of at most 32 entries in one kernel that walks the vertices
+ *      in order and needs no row lists (it runs beside the binning pass and the kernels of the long rows); 0 builds
+ *      them by degree class like all other rows; -1 takes the former for builds of at least 2^25 rows.  Same tables.
  *      "build_streams" (default 1): a build of 2 M .. 1 G entries without per-kernel timing sends the kernels of
  *      its degree classes out over the graph's stream and three side streams (small builds are bound by one
  *      kernel waiting for the one before); 0 keeps every kernel on the graph's stream.  Same tables.

@@ -62,21 +62,21 @@ typedef uint32_t uint4u __attribute__((ext_vector_type(4), aligned(4)));
 // nothing), which each entry then searches once with a fixed number of probes; the heavies' slots,
 // compacted by rank, give "next heavy" and "last heavy".  The rank rides in bits 52..63 of the SH scan.
 // Every lane of the wavefront must call this together (DPP); a group without a row passes d = 0.
-// s_pre: [2 * 256 * PER] u64 ([0, BLK): SL of every slot of the block; [BLK, 2 * BLK): SH), s_hs: [256 * PER]
+// s_pre: [2 * BLOCK * PER] u64 ([0, BLK): SL of every slot of the block; [BLK, 2 * BLK): SH), s_hs: [BLOCK * PER]
 // (per group: row-local slot of its h-th heavy).  Returns false for a row whose weights sum to zero.
 constexpr uint64_t GROUP_CNT = 1ull << 52;
 
-template <int G, int PER>
+template <int G, int PER, int BLOCK = 256>
 __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const float* __restrict__ wgt,
                                                 AliasEntry* __restrict__ table, uint64_t* __restrict__ s_pre,
-                                                uint8_t* __restrict__ s_hs) {
+                                                uint8_t* __restrict__ s_hs, uint32_t tid = threadIdx.x) {
   static_assert(PER == 4 || PER == 6, "a lane loads one float4 or three float2");
   constexpr uint32_t SLOTS = PER * G;
   constexpr uint32_t HB = PER == 4 ? SLOTS : SLOTS / 3 * 2;  // largest power of two <= SLOTS
-  constexpr uint32_t BLK = 256 * PER;                        // slots of one block's strips
-  const int gl = threadIdx.x & (G - 1);
-  const int lane = lane_id();
-  const uint32_t gbase = (uint32_t)PER * (threadIdx.x - gl);  // first LDS slot of the group
+  constexpr uint32_t BLK = BLOCK * PER;                      // slots of one block's strips (BLOCK threads)
+  const int gl = tid & (G - 1);
+  const int lane = tid & 63;
+  const uint32_t gbase = (uint32_t)PER * (tid - gl);  // first LDS slot of the group
   const uint32_t pos = (uint32_t)PER * gl;
 
   float xs[PER];
@@ -225,7 +225,8 @@ constexpr int BIN_ITEMS = 4;      // vertices per thread and step
 
 __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restrict__ xadj,
                                                         const uint32_t* __restrict__ src, uint32_t n,
-                                                        uint32_t per_block, uint32_t* __restrict__ blk_cnt,
+                                                        uint32_t per_block, int listed_from,
+                                                        uint32_t* __restrict__ blk_cnt,
                                                         unsigned long long* __restrict__ class_edges) {
   __shared__ uint32_t s_cnt[CLS_COUNT];
   __shared__ unsigned long long s_edges[CLS_COUNT];
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
     for (int k = 0; k < BIN_ITEMS; ++k) {
       const int c = degree_class(d[k]);
       if (c >= CLS_G2) {
-        atomicAdd(&s_cnt[c], 1u);
+        if (c >= listed_from) atomicAdd(&s_cnt[c], 1u);  // classes below get no list: small_rows_kernel builds them
         atomicAdd(&s_edges[c], (unsigned long long)d[k]);
       } else {
         tiny_edges += d[k];  // 0 for an empty row
@@ -335,7 +336,7 @@ __device__ __forceinline__ bool tiny_row(uint32_t off, uint32_t d, const float* 
 __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __restrict__ xadj,
                                                           const float* __restrict__ wgt,
                                                           const uint32_t* __restrict__ src, uint32_t n,
-                                                          uint32_t per_block,
+                                                          uint32_t per_block, int listed_from,
                                                           const uint32_t* __restrict__ counts,
                                                           const uint32_t* __restrict__ blk_off,
                                                           RowRef* __restrict__ vlist,
@@ -365,16 +366,19 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
         d = xadj[v + 1] - off;
         c = degree_class(d);
       }
-      const unsigned long long m = __ballot(c == CLS_TINY);
-      if (c == CLS_TINY) {
+      // listed_from > CLS_G2: the rows of the classes below it, empty rows included, belong to small_rows_kernel
+      const bool tiny_here = c == CLS_TINY && listed_from == CLS_G2;
+      const unsigned long long m = __ballot(tiny_here);
+      if (tiny_here) {
         const uint32_t p = nt + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
         s_tiny[wave][p] = make_uint2(off, v);
         s_tiny_d[wave][p] = (uint8_t)d;
-      } else if (c >= CLS_G2) {
+      } else if (c >= listed_from) {
         vlist[atomicAdd(&s_cur[c], 1u)] = RowRef{v, off, d, 0};
       }
       nt += (uint32_t)__popcll(m);
-      if (c >= 0) valid[v] = c != CLS_EMPTY;  // written here, next to its neighbours' flags; a row without weight clears it later
+      // written here, next to its neighbours' flags; a row without weight clears it later
+      if (c >= listed_from || (c >= 0 && listed_from == CLS_G2)) valid[v] = c != CLS_EMPTY;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -386,6 +390,119 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the next step's list entries stay behind these reads
     __builtin_amdgcn_wave_barrier();
   }
+}
+
+// ---------------------------------------------------------------- rows of at most 32 entries, where they lie
+// One wavefront walks a contiguous range of vertices, 64 at a time, and builds every row of 1..32 entries it
+// meets: the rows of a class queue up in LDS until they fill the wavefront (64 rows of 1..2 entries, 32 of 3..8 with
+// 2 lanes each, 16 of 9..16 with 4, 8 of 17..32 with 8) and are then built by the same code as in the class kernels.
+// Neighbouring rows of different classes share their cache lines, and here the same wavefront touches them within a
+// few steps; no row list is written or read for these classes.  Also sets valid[] of the vertices it owns (rows of
+// 0..32 entries).  Workgroups are single wavefronts: nothing in here waits for another wavefront.
+constexpr int SMALL_Q = 128;  // queue capacity: less than one batch left over plus the 64 vertices of a step
+__global__ __launch_bounds__(64) void small_rows_kernel(const uint32_t* __restrict__ xadj,
+                                                        const float* __restrict__ wgt,
+                                                        const uint32_t* __restrict__ src, uint32_t n,
+                                                        uint32_t per_wave, AliasEntry* __restrict__ table,
+                                                        int8_t* __restrict__ valid) {
+  __shared__ uint64_t s_pre[2 * 64 * 4];
+  __shared__ uint8_t s_hs[64 * 4];
+  __shared__ uint32_t q_off[4][SMALL_Q], q_v[4][SMALL_Q];
+  __shared__ uint8_t q_d[4][SMALL_Q];
+  const uint32_t lane = threadIdx.x;
+  const uint32_t lo = blockIdx.x * per_wave, hi = min(n, lo + per_wave);
+  uint32_t cnt[4] = {0, 0, 0, 0};  // wave-uniform queue lengths: rows of 1..2, 3..8, 9..16, 17..32 entries
+
+  // the last `rows` entries of queue q, one per group of G lanes; d = 0 for a group without a row.  `t` is the lane
+  // number behind an empty asm statement: it keeps what depends on the lane number inside one batch (hoisted
+  // out of the loop for all four row sizes at once, those values double the registers of the kernel).
+  auto take = [&](int q, uint32_t rows, uint32_t G, uint32_t& t, uint32_t& off, uint32_t& v, uint32_t& d) {
+    t = lane;
+    asm volatile("" : "+v"(t));
+    const uint32_t r = t / G;
+    off = v = d = 0;
+    if (r < rows) {
+      const uint32_t k = cnt[q] - rows + r;
+      off = q_off[q][k];
+      v = q_v[q][k];
+      d = q_d[q][k];
+    }
+  };
+  auto build_tiny = [&](uint32_t rows) {
+    uint32_t t, off, v, d;
+    take(0, rows, 1, t, off, v, d);
+    if (d && !tiny_row(off, d, wgt, table)) valid[v] = 0;
+    cnt[0] -= rows;
+  };
+  auto build_g2 = [&](uint32_t rows) {
+    uint32_t t, off, v, d;
+    take(1, rows, 2, t, off, v, d);
+    const bool ok = group_build_row<2, 4, 64>(off, d, wgt, table, s_pre, s_hs, t);
+    if ((t & 1) == 0 && !ok) valid[v] = 0;
+    cnt[1] -= rows;
+  };
+  auto build_g4 = [&](uint32_t rows) {
+    uint32_t t, off, v, d;
+    take(2, rows, 4, t, off, v, d);
+    const bool ok = group_build_row<4, 4, 64>(off, d, wgt, table, s_pre, s_hs, t);
+    if ((t & 3) == 0 && !ok) valid[v] = 0;
+    cnt[2] -= rows;
+  };
+  auto build_g8 = [&](uint32_t rows) {
+    uint32_t t, off, v, d;
+    take(3, rows, 8, t, off, v, d);
+    const bool ok = group_build_row<8, 4, 64>(off, d, wgt, table, s_pre, s_hs, t);
+    if ((t & 7) == 0 && !ok) valid[v] = 0;
+    cnt[3] -= rows;
+  };
+
+  // the row offsets of step i + 1 are requested before the batches of step i are built
+  auto fetch = [&](uint32_t base, uint32_t& v, uint32_t& off, uint32_t& end) {
+    const uint32_t item = base + lane;
+    v = 0xFFFFFFFFu;
+    off = end = 0;
+    if (item < hi) {
+      v = src ? src[item] : item;
+      off = xadj[v];
+      end = xadj[v + 1];
+    }
+  };
+  uint32_t nv, noff, nend;
+  fetch(lo, nv, noff, nend);
+  for (uint32_t base = lo; base < hi; base += 64u) {
+    const uint32_t v = nv, off = noff, d = nend - noff;
+    if (base + 64u < hi) fetch(base + 64u, nv, noff, nend);
+    int q = -1;
+    if (v != 0xFFFFFFFFu && d <= 32u) {
+      valid[v] = d != 0;  // a row without weight clears it when it is built
+      q = d == 0 ? -1 : d <= 2 ? 0 : d <= 8 ? 1 : d <= 16 ? 2 : 3;
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const unsigned long long m = __ballot(q == c);
+      if (q == c) {
+        const uint32_t p = cnt[c] + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+        q_off[c][p] = off;
+        q_v[c][p] = v;
+        q_d[c][p] = (uint8_t)d;
+      }
+      cnt[c] += (uint32_t)__popcll(m);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    while (cnt[0] >= 64u) build_tiny(64);
+    while (cnt[1] >= 32u) build_g2(32);
+    while (cnt[2] >= 16u) build_g4(16);
+    while (cnt[3] >= 8u) build_g8(8);
+    // the next step's queue entries stay behind this step's reads of the queues
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (cnt[0]) build_tiny(cnt[0]);
+  if (cnt[1]) build_g2(cnt[1]);
+  if (cnt[2]) build_g4(cnt[2]);
+  if (cnt[3]) build_g8(cnt[3]);
 }
 
 // ---------------------------------------------------------------- one row per workgroup, prefix arrays in LDS
@@ -974,6 +1091,8 @@ static bool g_build_profile = false;
 void set_build_profile(bool on) { g_build_profile = on; }
 static bool g_build_streams = true;
 void set_build_streams(bool on) { g_build_streams = on; }
+static int g_small_in_place = -1;  // -1: builds of at least 2^25 rows, 0: never, 1: always
+void set_small_in_place(int mode) { g_small_in_place = mode; }
 void set_stream_min_edges(uint64_t n) { g_stream_min_edges = n; }
 void set_row_merge(bool on) { g_row_merge = on; }
 
@@ -1021,18 +1140,34 @@ constexpr uint64_t FAN_MIN_EDGES = 2000000, FAN_MAX_EDGES = 1ull << 30;
 struct StreamFan {
   sky_graph* g;
   hipStream_t main;
-  bool on = false, used[sky_graph::SIDE_STREAMS] = {false, false, false};
+  bool on = false, joinable = false, used[sky_graph::SIDE_STREAMS] = {false, false, false};
   int turn = 0;
   StreamFan(sky_graph* g_, hipStream_t m) : g(g_), main(m) {}
-  int start() {  // after the binning pass has been enqueued on the graph's stream
+  int ensure() {
     for (int k = 0; k < sky_graph::SIDE_STREAMS; ++k) {
       if (!g->side[k]) SKY_HIP(hipStreamCreateWithFlags(&g->side[k], hipStreamNonBlocking));
       if (!g->join_ev[k]) SKY_HIP(hipEventCreateWithFlags(&g->join_ev[k], hipEventDisableTiming));
     }
     if (!g->fork_ev) SKY_HIP(hipEventCreateWithFlags(&g->fork_ev, hipEventDisableTiming));
+    return SKY_OK;
+  }
+  // One side stream that starts from the present end of the graph's stream, whatever start() does later; join()
+  // waits for it.
+  int branch(int k, hipStream_t* out) {
+    SKY_TRY(ensure());
+    SKY_HIP(hipEventRecord(g->fork_ev, main));
+    SKY_HIP(hipStreamWaitEvent(g->side[k], g->fork_ev, 0));
+    used[k] = true;
+    joinable = true;
+    *out = g->side[k];
+    return SKY_OK;
+  }
+  int start() {  // after the binning pass has been enqueued on the graph's stream
+    SKY_TRY(ensure());
     SKY_HIP(hipEventRecord(g->fork_ev, main));
     for (int k = 0; k < sky_graph::SIDE_STREAMS; ++k) SKY_HIP(hipStreamWaitEvent(g->side[k], g->fork_ev, 0));
     on = true;
+    joinable = true;
     return SKY_OK;
   }
   hipStream_t next() {
@@ -1043,10 +1178,11 @@ struct StreamFan {
     return g->side[k];
   }
   int join() {
-    if (!on) return SKY_OK;
-    on = false;
+    if (!joinable) return SKY_OK;
+    on = joinable = false;
     for (int k = 0; k < sky_graph::SIDE_STREAMS; ++k)
       if (used[k]) {
+        used[k] = false;
         SKY_HIP(hipEventRecord(g->join_ev[k], g->side[k]));
         SKY_HIP(hipStreamWaitEvent(main, g->join_ev[k], 0));
       }
@@ -1135,21 +1271,39 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     unsigned long long edges[CLS_COUNT];
   } host = {};
   static_assert(sizeof(host) == COUNTER_BYTES, "counter block layout");
+  // A large build leaves its rows of at most 32 entries to small_rows_kernel, which builds them where they lie,
+  // without lists.  Taken alone it is slower than the class kernels of these rows (1.39 against 1.12 ms on the
+  // scale-26 graph), but it does not depend on the binning pass: on a side stream it runs beside the binning and
+  // the kernels of the long rows (it waits on memory, they on the vector ALU): 10.2 -> 9.95 ms for the whole build.
+  // Smaller builds, whose class kernels already overlap, gain nothing (scale 24: 3 % slower).
+  const bool small_in_place = g_small_in_place < 0 ? n >= (1u << 25) : g_small_in_place != 0;
+  const int listed_from = small_in_place ? CLS_G16 : CLS_G2;
+  StreamFan fan(g, st);
+  auto launch_small = [&](hipStream_t s) {
+    const uint32_t per_wave = std::max(256u, std::min(2048u, n / 16384u / 64u * 64u));
+    hipLaunchKernelGGL(small_rows_kernel, dim3((n + per_wave - 1) / per_wave), dim3(64), 0, s, g->xadj, g->adjwgt, src, n,
+                       per_wave, g->table, g->valid);
+  };
   if (n > 0) {
+    if (small_in_place && !tm) {
+      hipStream_t side;
+      SKY_TRY(fan.branch(sky_graph::SIDE_STREAMS - 1, &side));
+      launch_small(side);
+    }
     SKY_HIP(hipMemsetAsync(sc.counters, 0, COUNTER_BYTES, st));
     // at most BIN_BLOCKS blocks, each a multiple of one scatter step
     const uint32_t step = 256u * BIN_ITEMS;
     const uint32_t per_block = ((n + BIN_BLOCKS - 1) / BIN_BLOCKS + step - 1) / step * step;
     const uint32_t blocks = (n + per_block - 1) / per_block;
-    hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n, per_block, sc.blk_cnt,
-                       reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
+    hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n, per_block, listed_from,
+                       sc.blk_cnt, reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
     hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(256), 0, st, sc.blk_cnt, blocks, sc.counters);
     hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n, per_block,
-                       sc.counters, sc.blk_cnt, sc.vlist, g->table, g->valid);
+                       listed_from, sc.counters, sc.blk_cnt, sc.vlist, g->table, g->valid);
     // The class sizes decide the launches that follow.  Those of all vertices depend on xadj alone and are kept
     // with the graph after the first time; any other list of rows is waited for.
     const bool all_rows = src == nullptr && n == g->V;
-    if (all_rows && g->bin_known) {
+    if (all_rows && g->bin_known && g->bin_listed_from == listed_from) {
       for (int c = 0; c < CLS_COUNT; ++c) {
         host.counts[c] = g->bin_counts[c];
         host.edges[c] = g->bin_edges[c];
@@ -1163,6 +1317,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
           g->bin_edges[c] = host.edges[c];
         }
         g->bin_known = true;
+        g->bin_listed_from = listed_from;
       }
     }
     for (int c = 0; c < CLS_COUNT; ++c) counts[c] = host.counts[c];
@@ -1172,11 +1327,15 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
       acc += counts[c];
     }
   }
-  if (tm) SKY_TRY(tm->mark("bin", host.edges[CLS_TINY]));
+  const uint64_t small_edges = host.edges[CLS_TINY] + host.edges[CLS_G2] + host.edges[CLS_G4] + host.edges[CLS_G8];
+  if (tm) SKY_TRY(tm->mark("bin", small_in_place ? 0 : host.edges[CLS_TINY]));
+  if (tm && small_in_place && n > 0) {
+    launch_small(st);
+    SKY_TRY(tm->mark("small", small_edges));
+  }
   RowRef* const vlist = sc.vlist;
   uint64_t call_edges = 0;
   for (int c = 0; c < CLS_COUNT; ++c) call_edges += host.edges[c];
-  StreamFan fan(g, st);
   if (!tm && g_build_streams && call_edges >= FAN_MIN_EDGES && call_edges < FAN_MAX_EDGES) SKY_TRY(fan.start());
 
   auto grp = [&](int cls, auto kernel, int G, const char* name) -> int {

@@ -389,6 +389,11 @@ int sky_set_option(const char* name, long value) {
     set_sample_distinct(value != 0);
     return SKY_OK;
   }
+  if (!strcmp(name, "small_in_place")) {
+    if (value < -1 || value > 1) return fail(SKY_ERR_ARG, "sky_set_option: small_in_place is -1, 0 or 1");
+    set_small_in_place((int)value);
+    return SKY_OK;
+  }
   if (!strcmp(name, "build_streams")) {
     set_build_streams(value != 0);
     return SKY_OK;

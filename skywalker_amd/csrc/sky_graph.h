@@ -47,6 +47,7 @@ struct sky_graph {
   // Class sizes of the last binning of all vertices.  They depend on xadj alone, which never changes, so a
   // later build of all vertices sizes its launches from them without waiting for the device.
   bool bin_known = false;
+  int bin_listed_from = 0;  // first class that the binning pass behind these sizes gave a list
   uint32_t bin_counts[32] = {0};
   unsigned long long bin_edges[32] = {0};
 };
@@ -115,6 +116,7 @@ void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);
 void set_stream_wide_min_edges(uint64_t n);
 void set_build_streams(bool on);
+void set_small_in_place(int mode);
 void set_sample_distinct(bool on);
 void set_walk_read_once(int mode);
 void set_build_profile(bool on);

@@ -22,15 +22,19 @@ def build_and_compare(orc, xadj, adjncy, w, label):
     # rows of 8190..524287 entries: once through their own kernel, once (the default for so few of them)
     # through the tile-parallel path
     routes = (0, 4000000) if ((deg >= 8190) & (deg <= 524287)).any() else (4000000,)
-    for stream_min_edges in routes:
+    # rows of at most 32 entries: by degree class (the default below 2^25 rows), and by the kernel that walks the
+    # vertices in order
+    for stream_min_edges, small_in_place in [(r, 0) for r in routes] + [(routes[0], 1)]:
         g = capi.Graph.upload(xadj, adjncy, w)
         capi.set_option("stream_min_edges", stream_min_edges)
         capi.set_option("stream_wide_min_edges", stream_min_edges)  # 0: also the rows above 65533 entries are streamed
+        capi.set_option("small_in_place", small_in_place)
         try:
             g.build_tables()
         finally:
             capi.set_option("stream_min_edges", 4000000)
             capi.set_option("stream_wide_min_edges", 512 * 262143)
+            capi.set_option("small_in_place", -1)
         prob, alias, valid = g.tables()
         g.free()
         st = orc.alias_check(xadj, w, prob, alias, valid)
@@ -39,9 +43,9 @@ def build_and_compare(orc, xadj, adjncy, w, label):
         bad = np.flatnonzero((prob != oprob) | (alias != oalias))
         if len(bad):
             v = int(np.searchsorted(xadj, bad[0], side="right") - 1)
-            raise AssertionError("%s (stream_min_edges %d): %d entries differ from the oracle, first at slot %d "
-                                 "(vertex %d, degree %d)" % (label, stream_min_edges, len(bad), bad[0], v,
-                                                             xadj[v + 1] - xadj[v]))
+            raise AssertionError("%s (stream_min_edges %d, small_in_place %d): %d entries differ from the oracle, first "
+                                 "at slot %d (vertex %d, degree %d)" % (label, stream_min_edges, small_in_place, len(bad),
+                                                                        bad[0], v, xadj[v + 1] - xadj[v]))
         assert np.array_equal(valid, ovalid)
 
 

@@ -69,6 +69,28 @@ def test_distinct_children_match_oracle(orc, fanout):
         assert (osl[big, 0] < fanout[1]).any()  # a parent that ended with fewer children than its fanout is among the cases
 
 
+def test_online_sampling_with_short_rows_built_in_vertex_order(orc):
+    # option small_in_place = 1 on a list of frontier vertices (by default only builds of 2^25 rows and more use it)
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(13, 8, 24)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 24, len(adjncy), 0.0, 1.0)
+    seeds = orc.gen_seeds(6, 1 << 13, 1200)
+    fanout = [1, 6, 4, 3]
+    lps, slen = capi.sample_layout(fanout)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    capi.set_option("small_in_place", 1)
+    try:
+        d_on, sl_on, s_on, _ = g.sample_online(seeds, fanout, 29)
+        with pytest.raises(capi.SkyError):
+            capi.set_option("small_in_place", 2)
+    finally:
+        capi.set_option("small_in_place", -1)
+    got = (d_on.to_host((1200, lps)), sl_on.to_host((1200, slen)))
+    g.free()
+    odata, osl, osampled = orc.sample_online(xadj, adjncy, w, seeds, fanout, 29)
+    assert np.array_equal(got[0], odata) and np.array_equal(got[1], osl) and s_on == osampled
+
+
 def test_exact_count_when_every_degree_exceeds_fanout(orc):
     from skywalker_amd import capi
     rng = np.random.default_rng(6)
