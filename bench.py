@@ -46,6 +46,7 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
 }
 KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
                   for g in (2, 4, 8, 16, 32) for x in ("", "x")})
+KERNEL_OF.update({"g32s": "build_group_kernel<32,5>"})
 KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,8>" % (64 * nw) for nw in range(2, 17)})
 KERNEL_OF.update({"mw3": "build_merge_kernel<256,6>", "mw5": "build_merge_kernel<256,10>", "mw6": "build_merge_kernel<512,6>",
                   "mw7": "build_merge_kernel<256,14>", "mw9": "build_merge_kernel<768,6>", "mw10": "build_merge_kernel<512,10>"})

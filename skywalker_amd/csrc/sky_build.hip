@@ -39,6 +39,7 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 32) return CLS_G8;
   if (d <= 64) return CLS_G16;
   if (d <= 128) return CLS_G32;
+  if (d <= 160) return CLS_G32S;
   if (d <= 192) return CLS_G32X;
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
@@ -70,9 +71,10 @@ template <int G, int PER, int BLOCK = 256>
 __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const float* __restrict__ wgt,
                                                 AliasEntry* __restrict__ table, uint64_t* __restrict__ s_pre,
                                                 uint8_t* __restrict__ s_hs, uint32_t tid = threadIdx.x) {
-  static_assert(PER == 4 || PER == 6, "a lane loads one float4 or three float2");
+  static_assert(PER >= 4 && PER <= 6, "a lane loads one float4 (and one float), or three float2");
   constexpr uint32_t SLOTS = PER * G;
-  constexpr uint32_t HB = PER == 4 ? SLOTS : SLOTS / 3 * 2;  // largest power of two <= SLOTS
+  constexpr uint32_t HB = PER == 4 ? SLOTS : PER == 5 ? SLOTS / 5 * 4 : SLOTS / 3 * 2;  // largest power of two <= SLOTS
+  static_assert((HB & (HB - 1)) == 0 && HB <= SLOTS && 2 * HB > SLOTS && SLOTS <= 256, "G is a power of two");
   constexpr uint32_t BLK = BLOCK * PER;                      // slots of one block's strips (BLOCK threads)
   const int gl = tid & (G - 1);
   const int lane = tid & 63;
@@ -82,7 +84,7 @@ __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const 
   float xs[PER];
 #pragma unroll
   for (int k = 0; k < PER; ++k) xs[k] = 0.0f;
-  if (PER == 4) {
+  if (PER == 4 || PER == 5) {
     if (pos < d) {
       const float4u x = *reinterpret_cast<const float4u*>(wgt + off + pos);
       xs[0] = x.x; xs[1] = x.y; xs[2] = x.z; xs[3] = x.w;
@@ -96,6 +98,7 @@ __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const 
         xs[2 * h + 1] = x.y;
       }
   }
+  if (PER % 2 == 1 && pos + PER - 1 < d) xs[PER - 1] = wgt[off + pos + PER - 1];
   double wd[PER];
   uint32_t live = 0;
   WSum3 S{0.0, 0.0, 0.0};
@@ -197,6 +200,7 @@ __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const 
       t[0] = AliasEntry{op[2 * h], oa[2 * h]};
     }
   }
+  if (PER % 2 == 1 && ((live >> (PER - 1)) & 1)) table[off + pos + PER - 1] = AliasEntry{op[PER - 1], oa[PER - 1]};
   return row_ok || d == 0;
 }
 
@@ -1352,6 +1356,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   SKY_TRY(grp(CLS_G8, build_group_kernel<8, 4>, 8, "g8"));
   SKY_TRY(grp(CLS_G16, build_group_kernel<16, 4>, 16, "g16"));
   SKY_TRY(grp(CLS_G32, build_group_kernel<32, 4>, 32, "g32"));
+  SKY_TRY(grp(CLS_G32S, build_group_kernel<32, 5>, 32, "g32s"));
   SKY_TRY(grp(CLS_G32X, build_group_kernel<32, 6>, 32, "g32x"));
 
   auto lds = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {

@@ -63,7 +63,7 @@ enum BuildClass : int {
   CLS_G8 = 4,       // deg <= 32        8 lanes
   CLS_G16 = 5,      // deg <= 64        16 lanes
   CLS_G32 = 6,      // deg <= 128       32 lanes
-  CLS_G32X = 7,     // deg <= 192       32 lanes, 6 slots per lane
+  CLS_G32X = 7,     // deg 161..192     32 lanes, 6 slots per lane
   CLS_LDS_W1 = 8,   // deg <= 253       one wavefront per row, 4 slots per lane
   CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
   CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..16 (class CLS_MW2 + nw - 2): one workgroup per row whose
@@ -73,7 +73,9 @@ enum BuildClass : int {
   CLS_STREAM_WIDE = 27,  // deg 65534..524287  and so
                     //                  does not end on its longest rows
   CLS_HUGE = 28,    // above            built tile by tile by the whole GPU
-  CLS_COUNT = 29
+  CLS_G32S = 29,    // deg 129..160     32 lanes, 5 slots per lane (the lower half of what CLS_G32X would hold;
+                    //                  3 slots per lane for rows of 33..48 entries gained nothing over CLS_G16)
+  CLS_COUNT = 30
 };
 
 // One listed row of a degree class: the build kernels read where the row lies from the list itself

@@ -11,7 +11,7 @@ TOL = 1e-6
 # degrees that straddle every dispatch class boundary of the build
 EDGE_DEGREES = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 16, 17, 22, 23, 24, 25, 28, 29, 30, 32, 33, 46, 47, 48,
                 49, 60, 61, 62, 63, 64, 65, 66, 67, 68, 94, 95, 96, 97, 124, 125, 126, 127, 190, 191, 192, 193, 253, 254, 255, 256, 257, 1021,
-                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 8189, 8190, 8191, 8192, 8193, 20000, 70001, 128, 129]
+                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 8189, 8190, 8191, 8192, 8193, 20000, 70001, 128, 129, 130, 144, 145, 159, 160, 161, 162, 34, 35, 36, 45]
 
 
 def build_and_compare(orc, xadj, adjncy, w, label):
