@@ -419,13 +419,23 @@ __device__ __forceinline__ unsigned long long group_ballot(bool p) {
   return N2V_G == 64 ? b : b & ((1ull << (N2V_G & 63)) - 1ull);
 }
 // Every lane of the group must call this together with the same row, n and key.
-__device__ __forceinline__ bool group_row_has(const uint32_t* __restrict__ row, uint32_t n, uint32_t key) {
+// The first round's probes depend on the row alone: group_first_probe loads them as soon as the row is known
+// (a step before the key is), and group_row_has takes the value.
+__device__ __forceinline__ uint32_t group_first_probe(const uint32_t* __restrict__ row, uint32_t n) {
+  const uint32_t gl = lane_id() & (N2V_G - 1);
+  if (n <= (uint32_t)N2V_G) return 0xFFFFFFFFu;
+  const uint32_t p = (gl + 1) * (n / (N2V_G + 1) + 1) - 1;
+  return p < n ? row[p] : 0xFFFFFFFFu;
+}
+__device__ __forceinline__ bool group_row_has(const uint32_t* __restrict__ row, uint32_t n, uint32_t key, uint32_t x0) {
   const uint32_t gl = lane_id() & (N2V_G - 1);
   uint32_t lo = 0, len = n;  // if the key is in the row it is in [lo, lo + len)
+  bool first_round = true;
   while (len > (uint32_t)N2V_G) {
     const uint32_t step = len / (N2V_G + 1) + 1, end = lo + len;
     const uint32_t p = lo + (gl + 1) * step - 1;           // probe gl: last element of part gl
-    const uint32_t x = p < end ? row[p] : 0xFFFFFFFFu;     // no vertex has this id
+    const uint32_t x = first_round ? x0 : (p < end ? row[p] : 0xFFFFFFFFu);  // no vertex has this id
+    first_round = false;
     const uint32_t c = (uint32_t)__popcll(group_ballot(x < key));  // parts that lie wholly below the key
     lo += c * step;
     len = min(step, end - lo);
@@ -446,6 +456,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_group_kernel(
     uint32_t v = seeds[i], prev = 0, prev_off = 0, prev_deg = 0;
     if (first) path[0] = v;
     for (; s < len && v < V; ++s) {
+      const uint32_t x0 = group_first_probe(adjncy + prev_off, prev_deg);  // in flight during the loads below
       u32x4 r = philox(seed, i, s, 0, DOM_WALK);
       if (stop_prob > 0.0f && u24(r.z) < stop_prob) break;
       const uint32_t off = xadj[v], deg = xadj[v + 1] - off;
@@ -463,7 +474,7 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_n2v_reject_group_kernel(
         }
         next = adjncy[off + cand];
         if (s == 0 || t >= 65536u) break;
-        const float f = next == prev ? fp : (group_row_has(adjncy + prev_off, prev_deg, next) ? 1.0f : fq);
+        const float f = next == prev ? fp : (group_row_has(adjncy + prev_off, prev_deg, next, x0) ? 1.0f : fq);
         if (u24(r.w) * fmax < f) break;
       }
       if (dead) break;
