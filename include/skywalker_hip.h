@@ -74,6 +74,9 @@ int sky_device_fill_u32(void* dst_device, uint32_t value, size_t count);
  * HBM traffic counters. */
 int sky_device_copy_u32(void* dst_device, const void* src_device, size_t count);
 int sky_device_synchronize(void);
+/* Free and total device memory of the current device as the HIP runtime reports them (hipMemGetInfo); either
+ * output may be NULL.  Lets a caller check that a call allocated nothing. */
+int sky_device_mem_info(size_t* free_bytes, size_t* total_bytes);
 int sky_device_name(char* buf, size_t buflen, int* compute_units);
 
 /* ---- graph residency: replaces gpu_graph::gpu_graph(Graph*, uint) (include/gpu_graph.cuh:68-117).
@@ -102,7 +105,12 @@ int sky_graph_free(sky_graph* g);
 int sky_alias_build_all(sky_graph* g, double* seconds);
 /* The same build from a weight array of the caller (E floats in device memory, CSR slot order) instead of the graph's
  * own weights, which are left as they are: for weights that a bias operator computes (include/skywalker_bias.h), as
- * the reference's constructors take them from gpu_graph::getBias (include/alias_table_new.cuh:1090-1091). */
+ * the reference's constructors take them from gpu_graph::getBias (include/alias_table_new.cuh:1090-1091).
+ * An array of exactly E floats is accepted.  The build kernels read whole 16-byte vectors that may reach up to 12
+ * bytes past the last weight: when the array's device allocation holds at least 16 readable bytes after the E floats
+ * (the library asks the HIP runtime for the allocation's extent) it is read where it lies; otherwise the call first
+ * copies it into a padded array that stays with the graph (E * 4 + 16 bytes more device memory, one device-to-device
+ * copy before the kernel region that `seconds` reports).  Allocate E * 4 + 16 bytes to avoid the copy. */
 int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, double* seconds);
 /* Copies the table to host as two arrays (any destination may be NULL). */
 int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t* valid);
@@ -165,11 +173,15 @@ int sky_sample_layout(const uint32_t* fanout, uint32_t hops, uint64_t* length_pe
 int sky_sample_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
                        uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device,
                        uint64_t* sampled, double* seconds);
-/* sky_sample_online draws WITH replacement, like sky_sample_offline and the reference's offline kernel
+/* By default sky_sample_online draws WITH replacement, like sky_sample_offline and the reference's offline kernel
  * (src/offline_sample.cu:109-133): a parent of more than fanout neighbours yields exactly fanout children, which may
  * repeat, and sample_lengths holds fanout.  The reference's OnlineGBSampleNew draws distinct neighbours by retrying
- * against a selected[] set and may return fewer than fanout (src/online_sample_new.cu:83-105); that rule is not
- * offered.  Online and offline results of this library are identical. */
+ * against a selected[] set and may return fewer than fanout (src/online_sample_new.cu:83-105): the option
+ * "sample_distinct" of sky_set_option (below) switches both sample calls to a rule of distinct children.  That rule
+ * is a deterministic variant, not the reference's law: here draw i of a parent tries up to 11 candidates in turn,
+ * there up to 11 rounds per parent run with 32 lanes drawing at once, so the expected number of children of a
+ * parent differs; the variant's own law is pinned by enumeration in the tests, its agreement with the reference's
+ * is unpinned.  Online and offline results of this library are identical under either setting. */
 int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
                       uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device, uint64_t* sampled,
                       double* seconds);

@@ -19,7 +19,7 @@ W_UNIFORM, W_UNIT, W_LOGNORMAL = 0, 1, 2
 
 EXPORTS = [
     "sky_last_error", "sky_version", "sky_device_malloc", "sky_device_free", "sky_memcpy_h2d", "sky_memcpy_d2h",
-    "sky_device_fill_u32", "sky_device_copy_u32", "sky_device_synchronize", "sky_device_name", "sky_graph_upload",
+    "sky_device_fill_u32", "sky_device_copy_u32", "sky_device_synchronize", "sky_device_mem_info", "sky_device_name", "sky_graph_upload",
     "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
     "sky_alias_build_all", "sky_alias_build_from_weights", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
     "sky_walk_offline_noalloc", "sky_walk_index_build",
@@ -68,6 +68,13 @@ def device_name():
 
 def synchronize():
     _ck(lib().sky_device_synchronize())
+
+
+def mem_info():
+    """(free, total) bytes of device memory as the HIP runtime reports them."""
+    f, t = C.c_size_t(0), C.c_size_t(0)
+    _ck(lib().sky_device_mem_info(C.byref(f), C.byref(t)))
+    return f.value, t.value
 
 
 class DeviceArray:
@@ -163,6 +170,12 @@ class Graph:
         """ConstructTable: returns the kernel-region seconds."""
         sec = C.c_double(0)
         _ck(lib().sky_alias_build_all(self.h, C.byref(sec)))
+        return sec.value
+
+    def build_tables_from_weights(self, weights):
+        """Tables from a caller's device array of E floats (a DeviceArray) instead of the graph's own weights."""
+        sec = C.c_double(0)
+        _ck(lib().sky_alias_build_from_weights(self.h, weights.ptr, C.byref(sec)))
         return sec.value
 
     def build_profile(self):

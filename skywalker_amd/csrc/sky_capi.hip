@@ -84,6 +84,14 @@ int sky_device_copy_u32(void* dst, const void* src, size_t count) {
   }
   return SKY_OK;
 }
+int sky_device_mem_info(size_t* free_bytes, size_t* total_bytes) {
+  SKY_TRY(ensure_device());
+  size_t f = 0, t = 0;
+  SKY_HIP(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return SKY_OK;
+}
 int sky_device_synchronize(void) {
   SKY_HIP(hipDeviceSynchronize());
   return SKY_OK;
@@ -118,6 +126,7 @@ int sky_graph_upload(const uint32_t* xadj, const uint32_t* adjncy, const float* 
   for (uint32_t i = 0; i < E; ++i)
     if (adjncy[i] >= V) return fail(SKY_ERR_ARG, "sky_graph_upload: neighbour id out of range");
   sky_graph* g = new sky_graph();
+  (void)hipGetDevice(&g->device);
   g->V = V;
   g->E = E;
   int rc = SKY_OK;
@@ -182,7 +191,7 @@ int sky_graph_device_ptrs(const sky_graph* g, const uint32_t** xadj, const uint3
 
 int sky_graph_free(sky_graph* g) {
   if (!g) return SKY_OK;
-  void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->table, g->valid, g->walk_index};
+  void* ptrs[] = {g->xadj, g->adjncy, g->adjwgt, g->table, g->valid, g->walk_index, g->wgt_copy};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   pool_release(g);
@@ -199,8 +208,37 @@ int sky_alias_build_all(sky_graph* g, double* seconds) {
 int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, double* seconds) {
   if (!g) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null graph");
   if (g->E && !weights_device) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null weights");
+  // The build kernels read whole 16-byte vectors that may reach up to 12 bytes past the last weight.  The
+  // caller's array is used where it lies only when its allocation is known to hold those bytes; otherwise the
+  // weights are copied into a padded array that stays with the graph.
+  const float* use = weights_device;
+  if (g->E) {
+    const size_t need = (size_t)g->E * 4 + 16;
+    void* abase = nullptr;
+    size_t asize = 0;
+    const hipError_t qe = hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t*>(&abase), &asize,
+                                                reinterpret_cast<hipDeviceptr_t>(const_cast<float*>(weights_device)));
+    bool padded = false;
+    if (qe == hipSuccess && abase) {
+      const size_t before = (size_t)(reinterpret_cast<const char*>(weights_device) - static_cast<const char*>(abase));
+      padded = before <= asize && asize - before >= need;
+    } else {
+      (void)hipGetLastError();  // a pointer the runtime does not know is not an error here: it is copied
+    }
+    if (!padded) {
+      if (g->wgt_copy_cap < g->E) {
+        if (g->wgt_copy) SKY_HIP(hipFree(g->wgt_copy));
+        g->wgt_copy = nullptr;
+        g->wgt_copy_cap = 0;
+        SKY_TRY(alloc_padded(&g->wgt_copy, (size_t)g->E));
+        g->wgt_copy_cap = g->E;
+      }
+      SKY_HIP(hipMemcpyAsync(g->wgt_copy, weights_device, (size_t)g->E * 4, hipMemcpyDeviceToDevice, g->stream));
+      use = g->wgt_copy;
+    }
+  }
   float* const own = g->adjwgt;
-  g->adjwgt = const_cast<float*>(weights_device);  // the build only reads it
+  g->adjwgt = const_cast<float*>(use);  // the build only reads it
   const int rc = build_all_tables(g, seconds);
   g->adjwgt = own;
   return rc;

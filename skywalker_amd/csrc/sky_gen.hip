@@ -115,6 +115,7 @@ int generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int
   if (weight_kind < SKY_W_UNIFORM || weight_kind > SKY_W_LOGNORMAL)
     return fail(SKY_ERR_ARG, "generate_rmat: unknown weight kind");
   sky_graph* g = new sky_graph();
+  (void)hipGetDevice(&g->device);
   g->V = (uint32_t)V;
   g->E = (uint32_t)E;
   hipStream_t st = g->stream;

@@ -6,11 +6,15 @@
 
 struct sky_graph {
   uint32_t V = 0, E = 0, max_degree = 0;
+  int device = 0;  // the device that was current when the graph was created: its arrays live there
   // CSR, device resident.  Arrays are allocated with 16 spare bytes so that kernels may
   // read whole aligned float4/uint4 quads that straddle the end.
   uint32_t* xadj = nullptr;    // [V+1]
   uint32_t* adjncy = nullptr;  // [E]
   float* adjwgt = nullptr;     // [E]
+  // padded copy of a caller's weight array (sky_alias_build_from_weights) whose allocation has no spare bytes
+  float* wgt_copy = nullptr;
+  size_t wgt_copy_cap = 0;
   // alias table: entry i belongs to CSR slot i; alias holds a row-local index
   sky::AliasEntry* table = nullptr;  // [E] {prob, alias}
   int8_t* valid = nullptr;    // [V]

@@ -318,6 +318,9 @@ int walk_offline_noalloc(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32
   int dev = 0;
   SKY_HIP(hipGetDevice(&dev));
   if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return fail(SKY_ERR_LIMIT, "sky_walk_offline_noalloc: device index beyond 63");
+  if (dev != g->device)  // the scratch array of the current device would be handed to kernels that read another device's graph
+    return fail(SKY_ERR_STATE, "sky_walk_offline_noalloc: the graph lives on device " + std::to_string(g->device) +
+                                   ", the current device is " + std::to_string(dev));
   if (!g_scratch_ptr[dev]) {  // once per device, with that device current: each GPU holds its own copy of the array
     unsigned long long* p = nullptr;
     SKY_HIP(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));

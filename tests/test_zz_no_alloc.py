@@ -29,6 +29,33 @@ def test_noalloc_walk_equals_walk_offline_twice_in_a_row(orc):
     g.free()
 
 
+def test_noalloc_walk_leaves_device_memory_as_it_found_it(orc):
+    # a graph whose pooled buffers are still empty: a call that allocated a counter, a list or an event pool would
+    # show up as a change of the free device memory the runtime reports
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 8, 6)
+    w = orc.gen_weights(orc.W_UNIFORM, 6, len(adjncy), 1.0, 100.0)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    N, length = 300001, 20  # outputs of 25 MB: far above the granularity of the report
+    seeds = g.gen_seeds(3, N)
+    paths = capi.DeviceArray(N * (length + 1), np.uint32, fill=capi.FILL)
+    lengths = capi.DeviceArray(N, np.uint32, fill=0)
+    sampled = capi.DeviceArray(1, np.uint64)
+    g.walk_offline_noalloc(seeds, length, 0.0, 3, paths, lengths, sampled)  # first call on this device: looks up the array
+    capi.synchronize()
+    free0, _ = capi.mem_info()
+    for _ in range(3):
+        g.walk_offline_noalloc(seeds, length, 0.0, 3, paths, lengths, sampled)
+    free1, _ = capi.mem_info()
+    capi.synchronize()
+    free2, _ = capi.mem_info()
+    assert free0 == free1 == free2
+    opaths, olen, osampled = orc.walk_offline(xadj, adjncy, *g.tables()[:2], seeds.to_host(), length, 0.0, 3)
+    assert np.array_equal(paths.to_host((N, length + 1)), opaths) and int(sampled.to_host()[0]) == osampled
+    g.free()
+
+
 def test_noalloc_walk_rejects_batches_beyond_its_scratch(orc):
     from skywalker_amd import capi
     xadj = np.array([0, 1, 2], np.uint32)
