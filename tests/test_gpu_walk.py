@@ -200,7 +200,7 @@ def test_read_once_gathers_give_the_same_paths(orc):
 
 
 def test_node2vec_rejection_one_walker_per_lane_for_large_batches(orc):
-    # up to 262,144 walkers take 16 lanes each (they search the previous row together); larger batches one lane each
+    # up to 262,144 walkers take 8 lanes each (they search the previous row together); larger batches one lane each
     from skywalker_amd import capi
     xadj, adjncy = orc.rmat_csr(12, 16, 35)
     w = orc.gen_weights(orc.W_LOGNORMAL, 35, len(adjncy), 0.0, 1.0)
