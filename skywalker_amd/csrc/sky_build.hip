@@ -101,18 +101,33 @@ __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const 
   if (PER % 2 == 1 && pos + PER - 1 < d) xs[PER - 1] = wgt[off + pos + PER - 1];
   double wd[PER];
   uint32_t live = 0;
-  WSum3 S{0.0, 0.0, 0.0};
+  // the sum of the row as a plain fp64 sum where that is exact (plain_sum_is_exact); a wavefront in which some
+  // group's is not falls back to the three-limb sum for all of its groups
+  double Sd = 0.0;
+  uint32_t mn = 0xFFFFFFFFu;
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
     const bool in = pos + k < d;
     if (in) live |= 1u << k;
-    wd[k] = (double)masked_weight(xs[k], in);
-    wsum3_add(S, wd[k]);
+    const float cw = masked_weight(xs[k], in);
+    wd[k] = (double)cw;
+    Sd += wd[k];
+    mn = min(mn, __float_as_uint(cw) - 1u);
   }
-  S = group_sum_wsum3<G>(S);
-  const bool row_ok = S.top + S.mid + S.low != 0.0;
-  Ledger L = make_ledger_small(d, wsum3_to_double(S));
+  Sd = group_sum_f64<G>(Sd);
+  mn = group_min_u32<G>(mn);
+  const bool plain = plain_sum_is_exact(Sd, mn);
+  if (__any(!plain)) {
+    WSum3 S{0.0, 0.0, 0.0};
+#pragma unroll
+    for (int k = 0; k < PER; ++k) wsum3_add(S, wd[k]);
+    S = group_sum_wsum3<G>(S);
+    if (!plain) Sd = S.top + S.mid + S.low != 0.0 ? wsum3_to_double(S) : 0.0;
+  }
+  const bool row_ok = Sd != 0.0;
+  Ledger L = make_ledger_small(d, Sd);
   if (!row_ok) L.scale = 0.0;
+  const double neg_fs = -L.fs;
 
   uint64_t dl[PER], sl[PER], sh[PER];
   float op[PER];
@@ -120,7 +135,7 @@ __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const 
   uint64_t ra = 0, rb = 0;
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
-    const Entry e = classify_small_unmasked(wd[k], L);
+    const Entry e = classify_small_fma(wd[k], L, neg_fs);
     dl[k] = (e.heavy || !((live >> k) & 1)) ? 0 : e.amount;
     ra += dl[k];
     rb += e.heavy ? (e.amount | GROUP_CNT) : 0;
@@ -403,7 +418,13 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
 // Neighbouring rows of different classes share their cache lines, and here the same wavefront touches them within a
 // few steps; no row list is written or read for these classes.  Also sets valid[] of the vertices it owns (rows of
 // 0..32 entries).  Workgroups are single wavefronts: nothing in here waits for another wavefront.
-constexpr int SMALL_Q = 128;  // queue capacity: less than one batch left over plus the 64 vertices of a step
+// Queue capacities (128, 96, 80, 72): less than one batch left over plus the 64 vertices of a step
+// (64 + 63, 64 + 31, 64 + 15, 64 + 7), rounded up.  A queue entry is the row's offset and, in 16 bits, its degree (6 bits) above the vertex's position in
+// the wavefront's range (10 bits): the vertex id itself is only needed for a row without weight, whose flag is
+// cleared.  6.5 KB of LDS per wavefront, so that six of them fit every SIMD (the kernel's registers allow six).
+constexpr uint32_t SMALL_RANGE = 1024;  // most vertices per wavefront
+constexpr uint32_t SMALL_QBASE[4] = {0, 128, 224, 304};
+constexpr uint32_t SMALL_QTOTAL = 376;
 __global__ __launch_bounds__(64) void small_rows_kernel(const uint32_t* __restrict__ xadj,
                                                         const float* __restrict__ wgt,
                                                         const uint32_t* __restrict__ src, uint32_t n,
@@ -411,8 +432,8 @@ __global__ __launch_bounds__(64) void small_rows_kernel(const uint32_t* __restri
                                                         int8_t* __restrict__ valid) {
   __shared__ uint64_t s_pre[2 * 64 * 4];
   __shared__ uint8_t s_hs[64 * 4];
-  __shared__ uint32_t q_off[4][SMALL_Q], q_v[4][SMALL_Q];
-  __shared__ uint8_t q_d[4][SMALL_Q];
+  __shared__ uint32_t q_off[SMALL_QTOTAL];
+  __shared__ uint16_t q_it[SMALL_QTOTAL];
   const uint32_t lane = threadIdx.x;
   const uint32_t lo = blockIdx.x * per_wave, hi = min(n, lo + per_wave);
   uint32_t cnt[4] = {0, 0, 0, 0};  // wave-uniform queue lengths: rows of 1..2, 3..8, 9..16, 17..32 entries
@@ -420,43 +441,48 @@ __global__ __launch_bounds__(64) void small_rows_kernel(const uint32_t* __restri
   // the last `rows` entries of queue q, one per group of G lanes; d = 0 for a group without a row.  `t` is the lane
   // number behind an empty asm statement: it keeps what depends on the lane number inside one batch (hoisted
   // out of the loop for all four row sizes at once, those values double the registers of the kernel).
-  auto take = [&](int q, uint32_t rows, uint32_t G, uint32_t& t, uint32_t& off, uint32_t& v, uint32_t& d) {
+  auto take = [&](int q, uint32_t rows, uint32_t G, uint32_t& t, uint32_t& off, uint32_t& it, uint32_t& d) {
     t = lane;
     asm volatile("" : "+v"(t));
     const uint32_t r = t / G;
-    off = v = d = 0;
+    off = it = d = 0;
     if (r < rows) {
-      const uint32_t k = cnt[q] - rows + r;
-      off = q_off[q][k];
-      v = q_v[q][k];
-      d = q_d[q][k];
+      const uint32_t k = SMALL_QBASE[q] + cnt[q] - rows + r;
+      off = q_off[k];
+      const uint32_t x = q_it[k];
+      it = x & (SMALL_RANGE - 1);
+      d = x >> 10;
     }
   };
+  auto clear_valid = [&](uint32_t it) {  // a row whose weights sum to zero (rare)
+    const uint32_t item = lo + it;
+    valid[src ? src[item] : item] = 0;
+  };
   auto build_tiny = [&](uint32_t rows) {
-    uint32_t t, off, v, d;
-    take(0, rows, 1, t, off, v, d);
-    if (d && !tiny_row(off, d, wgt, table)) valid[v] = 0;
+    uint32_t t, off, it, d;
+    take(0, rows, 1, t, off, it, d);
+    if (d && !tiny_row(off, d, wgt, table)) clear_valid(it);
     cnt[0] -= rows;
   };
   auto build_g2 = [&](uint32_t rows) {
-    uint32_t t, off, v, d;
-    take(1, rows, 2, t, off, v, d);
+    uint32_t t, off, it, d;
+    take(1, rows, 2, t, off, it, d);
     const bool ok = group_build_row<2, 4, 64>(off, d, wgt, table, s_pre, s_hs, t);
-    if ((t & 1) == 0 && !ok) valid[v] = 0;
+    if ((t & 1) == 0 && !ok) clear_valid(it);
     cnt[1] -= rows;
   };
   auto build_g4 = [&](uint32_t rows) {
-    uint32_t t, off, v, d;
-    take(2, rows, 4, t, off, v, d);
+    uint32_t t, off, it, d;
+    take(2, rows, 4, t, off, it, d);
     const bool ok = group_build_row<4, 4, 64>(off, d, wgt, table, s_pre, s_hs, t);
-    if ((t & 3) == 0 && !ok) valid[v] = 0;
+    if ((t & 3) == 0 && !ok) clear_valid(it);
     cnt[2] -= rows;
   };
   auto build_g8 = [&](uint32_t rows) {
-    uint32_t t, off, v, d;
-    take(3, rows, 8, t, off, v, d);
+    uint32_t t, off, it, d;
+    take(3, rows, 8, t, off, it, d);
     const bool ok = group_build_row<8, 4, 64>(off, d, wgt, table, s_pre, s_hs, t);
-    if ((t & 7) == 0 && !ok) valid[v] = 0;
+    if ((t & 7) == 0 && !ok) clear_valid(it);
     cnt[3] -= rows;
   };
 
@@ -481,14 +507,14 @@ __global__ __launch_bounds__(64) void small_rows_kernel(const uint32_t* __restri
       valid[v] = d != 0;  // a row without weight clears it when it is built
       q = d == 0 ? -1 : d <= 2 ? 0 : d <= 8 ? 1 : d <= 16 ? 2 : 3;
     }
+    const uint32_t packed = (d << 10) | (base - lo + lane);
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const unsigned long long m = __ballot(q == c);
       if (q == c) {
-        const uint32_t p = cnt[c] + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
-        q_off[c][p] = off;
-        q_v[c][p] = v;
-        q_d[c][p] = (uint8_t)d;
+        const uint32_t p = SMALL_QBASE[c] + cnt[c] + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+        q_off[p] = off;
+        q_it[p] = (uint16_t)packed;
       }
       cnt[c] += (uint32_t)__popcll(m);
     }
@@ -723,8 +749,8 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const RowRef* __restric
 constexpr uint64_t MERGE_CNT = 1ull << 52;
 constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
 
-template <int ROWT, int PER>
-__global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __restrict__ vlist,
+template <int ROWT, int PER, int MINW = 4>
+__global__ __launch_bounds__(ROWT, MINW) void build_merge_kernel(const RowRef* __restrict__ vlist,
                                                            const uint32_t* __restrict__ xadj,
                                                            const float* __restrict__ wgt,
                                                            AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
@@ -742,6 +768,8 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
   uint32_t* s_res = reinterpret_cast<uint32_t*>(smem + CAP + 2);  // [CAP + 2]
   uint16_t* s_hs = reinterpret_cast<uint16_t*>(s_res + CAP + 2);   // [CAP + 2] row-local slot of heavy h
   __shared__ WSum3 s_wsum[NW];
+  __shared__ double s_fsum[NW];
+  __shared__ uint32_t s_mn[NW];
   __shared__ uint64_t s_ex[3 * NW];
 
   const RowRef rr = vlist[blockIdx.x];
@@ -753,7 +781,9 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
 
   double wd[PER];
   uint32_t live = 0;  // bit j: slot pos0 + j belongs to the row
-  WSum3 sum{0.0, 0.0, 0.0};
+  // the sum of the row as a plain fp64 sum where that is exact (plain_sum_is_exact), else as three limbs
+  double rsum = 0.0;
+  uint32_t mn = 0xFFFFFFFFu;
   if (wave_on) {
 #pragma unroll
     for (int t = 0; t < PER / VEC; ++t) {
@@ -773,34 +803,61 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
         const uint32_t idx = pos + k;
         const bool in = idx - lead < d;  // one unsigned compare: slots before the row wrap around
         if (in) live |= 1u << (t * VEC + k);
-        wd[t * VEC + k] = (double)masked_weight(xs[k], in);
-        wsum3_add(sum, wd[t * VEC + k]);
+        const float cw = masked_weight(xs[k], in);
+        wd[t * VEC + k] = (double)cw;
+        rsum += wd[t * VEC + k];
+        mn = min(mn, __float_as_uint(cw) - 1u);
       }
     }
-    sum = group_sum_wsum3<64>(sum);
+    rsum = group_sum_f64<64>(rsum);
+    mn = wave_min_u32(mn);
   } else {
 #pragma unroll
     for (int j = 0; j < PER; ++j) wd[j] = 0.0;
   }
   if (NW > 1) {
-    if (lane == 0) s_wsum[wave] = sum;
+    if (lane == 0) {
+      s_fsum[wave] = rsum;
+      s_mn[wave] = mn;
+    }
     __syncthreads();
-    sum = s_wsum[0];
+    rsum = s_fsum[0];
+    mn = s_mn[0];
 #pragma unroll
     for (int i = 1; i < NW; ++i) {
-      sum.top += s_wsum[i].top;
-      sum.mid += s_wsum[i].mid;
-      sum.low += s_wsum[i].low;
+      rsum += s_fsum[i];
+      mn = min(mn, s_mn[i]);
     }
   }
-  if (sum.top + sum.mid + sum.low == 0.0) {
+  if (!plain_sum_is_exact(rsum, (uint32_t)__builtin_amdgcn_readfirstlane((int)mn))) {  // uniform over the workgroup
+    WSum3 sum{0.0, 0.0, 0.0};
+    if (wave_on) {
+#pragma unroll
+      for (int j = 0; j < PER; ++j) wsum3_add(sum, wd[j]);
+      sum = group_sum_wsum3<64>(sum);
+    }
+    if (NW > 1) {
+      if (lane == 0) s_wsum[wave] = sum;
+      __syncthreads();
+      sum = s_wsum[0];
+#pragma unroll
+      for (int i = 1; i < NW; ++i) {
+        sum.top += s_wsum[i].top;
+        sum.mid += s_wsum[i].mid;
+        sum.low += s_wsum[i].low;
+      }
+    }
+    rsum = sum.top + sum.mid + sum.low != 0.0 ? wsum3_to_double(sum) : 0.0;
+  }
+  if (rsum == 0.0) {
 #pragma unroll
     for (int j = 0; j < PER; ++j)
       if ((live >> j) & 1) table[base + pos0 + j] = AliasEntry{0.0f, SKY_INVALID};
     if (tid == 0) valid[v] = 0;
     return;
   }
-  const Ledger L = make_ledger_small(d, wsum3_to_double(sum));
+  const Ledger L = make_ledger_small(d, rsum);
+  const double neg_fs = -L.fs;
 
   float op[PER];
   uint32_t hcnt[PER];  // heavies up to and including this slot
@@ -811,7 +868,7 @@ __global__ __launch_bounds__(ROWT, 4) void build_merge_kernel(const RowRef* __re
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const bool in = (live >> j) & 1;
-      const Entry e = PACKED ? classify_small_unmasked(wd[j], L) : classify_fast(wd[j], in, L);
+      const Entry e = PACKED ? classify_small_fma(wd[j], L, neg_fs) : classify_fast(wd[j], in, L);
       dl[j] = (e.heavy || !in) ? 0 : e.amount;
       dh[j] = e.heavy ? (PACKED ? (e.amount | MERGE_CNT) : e.amount) : 0;
       op[j] = (float)e.p;
@@ -1284,7 +1341,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   const int listed_from = small_in_place ? CLS_G16 : CLS_G2;
   StreamFan fan(g, st);
   auto launch_small = [&](hipStream_t s) {
-    const uint32_t per_wave = std::max(256u, std::min(2048u, n / 16384u / 64u * 64u));
+    const uint32_t per_wave = std::max(256u, std::min(SMALL_RANGE, n / 16384u / 64u * 64u));
     hipLaunchKernelGGL(small_rows_kernel, dim3((n + per_wave - 1) / per_wave), dim3(64), 0, s, g->xadj, g->adjwgt, src, n,
                        per_wave, g->table, g->valid);
   };

@@ -19,6 +19,8 @@
 // the alias ranks of the lights and the slots of the heavies both grow along the row.  An emit pass
 // leaves alone what belongs to another window: lights whose alias lies outside this one, and heavies of
 // earlier windows, whose final entries are already written.  After the first pass the weights come from L2.
+#include <type_traits>
+
 #include "sky_build_common.h"
 #include "sky_graph.h"
 
@@ -28,7 +30,7 @@ constexpr int ST_T = 512;                 // threads per row
 constexpr int ST_PER = 8;                 // consecutive slots per thread and chunk
 constexpr int ST_CH = ST_T * ST_PER;      // slots per chunk
 constexpr int ST_NW = ST_T / 64;
-constexpr uint32_t ST_CAP = 5085;         // heavies per row kept in LDS (and one sentinel): two workgroups share a CU's 160 KB
+constexpr uint32_t ST_CAP = 5080;         // heavies per row kept in LDS (and one sentinel): two workgroups share a CU's 160 KB
 static_assert(STREAM_MAX_DEG + 3 < (1u << 20), "the three-limb sum is exact for rows of fewer than 2^20 entries");
 
 struct StreamRow {
@@ -54,6 +56,11 @@ __device__ __forceinline__ RawChunk fetch_chunk(const float* __restrict__ wgt, c
     if (pos < r.span) x.q[q] = *reinterpret_cast<const float4*>(wgt + r.base + pos);
   }
   return x;
+}
+// Makes the wavefront wait, here, until the chunk's loads have arrived.
+__device__ __forceinline__ void wait_for_chunk(const RawChunk& x) {
+#pragma unroll
+  for (int q = 0; q < ST_PER / 4; ++q) asm volatile("" ::"v"(x.q[q].x), "v"(x.q[q].y), "v"(x.q[q].z), "v"(x.q[q].w));
 }
 // Whether every slot of wavefront `wave` in chunk c lies inside the row: true for all but the row's first wavefront
 // (when the row starts after its 16-byte aligned base) and the one that holds its end.  Such a wavefront needs
@@ -171,10 +178,12 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
                                                             const float* __restrict__ wgt,
                                                             AliasEntry* __restrict__ table,
                                                             int8_t* __restrict__ valid) {
-  __shared__ uint64_t s_sh[ST_CAP + 1];    // surplus prefix of the window's h-th heavy, then a sentinel
-  __shared__ float s_prob[ST_CAP + 1];     // its residual probability, left by the light that reaches it
-  __shared__ uint32_t s_slot[ST_CAP + 1];  // its span slot; after them the slot lights beyond the window take
+  __shared__ uint64_t s_sh[ST_CAP + 2];    // surplus prefix of the window's h-th heavy, then two sentinels
+  __shared__ float s_prob[ST_CAP + 2];     // its residual probability, left by the light that reaches it
+  __shared__ uint32_t s_slot[ST_CAP + 2];  // its span slot; after them the slot lights beyond the window take
   __shared__ WSum3 s_w[ST_NW];
+  __shared__ double s_fsum[ST_NW];
+  __shared__ uint32_t s_mn[ST_NW];
   __shared__ uint64_t s_a[2][ST_NW];  // two sets of wavefront sums, used alternately
   __shared__ uint32_t s_c[2][ST_NW];
   __shared__ uint32_t s_next;  // slot of the first heavy after the window
@@ -187,32 +196,69 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   r.span = r.lead + rr.d;
   const uint32_t nch = (r.span + ST_CH - 1) / ST_CH;
 
-  // ---- pass A: exact sum
-  WSum3 sum{0.0, 0.0, 0.0};
+  // ---- pass A: the sum of the row, as a plain fp64 sum when that is exact (see plain_sum_is_exact)
+  double row_sum;
   RawChunk nx = fetch_chunk(wgt, r, 0, tid);  // every loop below requests chunk c + 1 before it works on chunk c
-  for (uint32_t c = 0; c < nch; ++c) {
-    const RawChunk cur = nx;
-    if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
-    if (!wave_in_row(r, c, wave)) continue;
-    float cw[ST_PER];
-    if (wave_inside_row(r, c, wave))
-      unpack_chunk<false>(cur, r, c, tid, cw);
-    else
-      unpack_chunk<true>(cur, r, c, tid, cw);
+  {
+    double fsum = 0.0;
+    uint32_t mn = 0xFFFFFFFFu;
+    for (uint32_t c = 0; c < nch; ++c) {
+      const RawChunk cur = nx;
+      if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
+      if (!wave_in_row(r, c, wave)) continue;
+      float cw[ST_PER];
+      if (wave_inside_row(r, c, wave))
+        unpack_chunk<false>(cur, r, c, tid, cw);
+      else
+        unpack_chunk<true>(cur, r, c, tid, cw);
 #pragma unroll
-    for (int j = 0; j < ST_PER; ++j) wsum3_add(sum, (double)cw[j]);
-  }
-  sum = group_sum_wsum3<64>(sum);
-  if (lane == 0) s_w[wave] = sum;
-  __syncthreads();
-  sum = s_w[0];
+      for (int j = 0; j < ST_PER; j += 2) {
+        fsum += (double)cw[j];
+        fsum += (double)cw[j + 1];
+        mn = min(mn, min(__float_as_uint(cw[j]) - 1u, __float_as_uint(cw[j + 1]) - 1u));
+      }
+    }
+    fsum = group_sum_f64<64>(fsum);
+    mn = wave_min_u32(mn);
+    if (lane == 0) {
+      s_fsum[wave] = fsum;
+      s_mn[wave] = mn;
+    }
+    __syncthreads();
+    fsum = s_fsum[0];
+    mn = s_mn[0];
 #pragma unroll
-  for (int i = 1; i < ST_NW; ++i) {
-    sum.top += s_w[i].top;
-    sum.mid += s_w[i].mid;
-    sum.low += s_w[i].low;
+    for (int i = 1; i < ST_NW; ++i) {
+      fsum += s_fsum[i];
+      mn = min(mn, s_mn[i]);
+    }
+    row_sum = fsum;
+    if (!plain_sum_is_exact(fsum, uniform_u32(mn))) {  // uniform: the three-limb sum, from a second pass over the row
+      WSum3 sum{0.0, 0.0, 0.0};
+      nx = fetch_chunk(wgt, r, 0, tid);
+      for (uint32_t c = 0; c < nch; ++c) {
+        const RawChunk cur = nx;
+        if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
+        if (!wave_in_row(r, c, wave)) continue;
+        float cw[ST_PER];
+        unpack_chunk<true>(cur, r, c, tid, cw);
+#pragma unroll
+        for (int j = 0; j < ST_PER; ++j) wsum3_add(sum, (double)cw[j]);
+      }
+      sum = group_sum_wsum3<64>(sum);
+      if (lane == 0) s_w[wave] = sum;
+      __syncthreads();
+      sum = s_w[0];
+#pragma unroll
+      for (int i = 1; i < ST_NW; ++i) {
+        sum.top += s_w[i].top;
+        sum.mid += s_w[i].mid;
+        sum.low += s_w[i].low;
+      }
+      row_sum = sum.top + sum.mid + sum.low == 0.0 ? 0.0 : wsum3_to_double(sum);
+    }
   }
-  if (sum.top + sum.mid + sum.low == 0.0) {
+  if (row_sum == 0.0) {
     for (uint32_t c = 0; c < nch; ++c)
 #pragma unroll
       for (int j = 0; j < ST_PER; ++j) {
@@ -222,7 +268,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     if (tid == 0) valid[rr.v] = 0;
     return;
   }
-  const Ledger L = make_ledger_small(rr.d, wsum3_to_double(sum));
+  const Ledger L = make_ledger_small(rr.d, row_sum);
 
   // Whether an entry is heavy is a monotone function of its clamped weight (p = fl(w * scale) and
   // t = fma(p, 2^F, -2^F) are monotone, heavy iff t >= 0.5), so one compare against the smallest heavy weight
@@ -256,6 +302,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     thr_bits = bits;
   }
   float* s_w32 = reinterpret_cast<float*>(s_sh);  // weight of heavy h in the low half of s_sh[h], until its prefix replaces it
+  const double neg_fs = -L.fs;
 
   // window state: collecting resumes at chunk cb (cnt_cb heavies lie before it), emitting at chunk cc
   // (def_cc deficits and hc_cc heavies lie before it)
@@ -343,9 +390,11 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     }
     const bool any_heavy = hb + nw != 0;
     const bool whole_row = hb == 0 && !more;  // the usual case: one window holds every heavy of the row
-    if (tid == 0) {  // after the list: a sentinel, and the slot that lights beyond the window's last heavy take
+    if (tid == 0) {  // after the list: two sentinels, and the slot that lights beyond the window's last heavy take
       s_sh[nw] = ~0ull;
+      s_sh[nw + 1] = ~0ull;
       s_slot[nw] = more ? next_slot : (nw ? s_slot[nw - 1] : 0u);
+      s_slot[nw + 1] = 0u;
     }
     __syncthreads();
 
@@ -364,41 +413,53 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       const RawChunk cur = nx;
       if (c + 1 < nch) nx = fetch_chunk(wgt, r, c + 1, tid);
       const bool on = wave_in_row(r, c, wave);  // a wavefront past the row's end only takes part in the scan
-      uint32_t live = 0;
+      const bool inside = wave_inside_row(r, c, wave);
+      uint32_t live = (1u << ST_PER) - 1u;
+      // op[j]: float(p) of a light, -1 of a heavy (the sign carries "heavy" to the walk below); dl[j]: the
+      // deficit of a light of the row, 0 for any other slot
       float op[ST_PER];
       uint64_t dl[ST_PER];
-      uint32_t heavy = 0;
+      uint32_t nheavy = 0;
       uint64_t run = 0;
-      if (on) {
+      auto classify_chunk = [&](auto edge) {
+        constexpr bool EDGE = decltype(edge)::value;
         float cw[ST_PER];
-        if (wave_inside_row(r, c, wave))
-          live = unpack_chunk<false>(cur, r, c, tid, cw);
-        else
-          live = unpack_chunk<true>(cur, r, c, tid, cw);
+        live = unpack_chunk<EDGE>(cur, r, c, tid, cw);
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
           // only the lights' amounts are used here: |t| <= 2^F, so the sum with 2^52 holds rint(|t|) in its low bits
           // (0 for a light with 0 < t < 0.5).  Heavy slots and slots outside the row come out as anything and are dropped.
           const double pj = (double)cw[j] * L.scale;
-          const double t = (pj - 1.0) * L.fs;
-          op[j] = (float)pj;
-          dl[j] = (uint64_t)__double_as_longlong(fabs(t) + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
-          if (__float_as_uint(cw[j]) >= thr_bits) heavy |= 1u << j;
+          const double t = fma(pj, L.fs, neg_fs);  // = (pj - 1) * 2^F rounded once: the product with 2^F is exact
+          const uint64_t d = (uint64_t)__double_as_longlong(fabs(t) + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
+          const bool lv = !EDGE || ((live >> j) & 1);
+          const bool hj = lv && __float_as_uint(cw[j]) >= thr_bits;
+          op[j] = hj ? -1.0f : (float)pj;
+          dl[j] = (lv && !hj) ? d : 0;
+          nheavy += hj ? 1u : 0u;
+          run += dl[j];
         }
-        heavy &= live;
-        const uint32_t light = live & ~heavy;
+      };
+      if (on) {
+        if (inside) classify_chunk(std::false_type{});
+        else classify_chunk(std::true_type{});
+      } else {
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
-          dl[j] = ((light >> j) & 1) ? dl[j] : 0;
-          run += dl[j];
+          op[j] = 0.0f;
+          dl[j] = 0;
         }
       }
       uint64_t ex_d, tot_d;
       uint32_t ex_c, tot_c;
-      stream_excl(run, (uint32_t)__popc(heavy), s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
+      stream_excl(run, nheavy, s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
+      const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
+      uint32_t oa[ST_PER];
+      uint32_t wr = 0;  // entries this window writes: its lights, and heavies as placeholders unless an earlier window owns them
       if (on) {
         // b = window heavies whose surplus prefix is <= the deficits before this thread's slots: one search;
-        // from there the thread's lights walk the list, each stopping at its own deficit prefix
+        // from there the thread's lights walk the list, each stopping at its own deficit prefix.  The list
+        // entry after the current one is requested a hit ahead, so that a hit does not wait for local memory.
         uint64_t sl = carry_d + ex_d;
         uint32_t b = 0;
         if (nw) {
@@ -407,38 +468,49 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
           count_le<1>(s_sh, nw, k1, o1);
           b = o1[0];
         }
-        uint64_t hv = s_sh[b];       // ~0 once the window is exhausted
-        uint32_t hslot = s_slot[b];  // then: the first heavy after the window, or the row's last heavy
-        const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
-        uint32_t oa[ST_PER];
-        uint32_t wr = 0;  // entries this window writes: its lights, and heavies as placeholders unless an earlier window owns them
+        uint64_t hv = s_sh[b], hvn = s_sh[b + 1];  // ~0 once the window is exhausted
+        // alias value of the current list entry (then: of the first heavy after the window, or the row's last heavy)
+        uint32_t hal = s_slot[b] - r.lead, haln = s_slot[b + 1] - r.lead;
+        const uint32_t self0 = pos0 - r.lead;
         uint32_t hrank = carry_c + ex_c;
         // One path for every slot: a heavy slot, or one outside the row, adds no deficit, so the list does not move.
 #pragma unroll
         for (int j = 0; j < ST_PER; ++j) {
-          const bool lv = (live >> j) & 1, hj = (heavy >> j) & 1;
-          // a light's alias is the first heavy whose surplus prefix exceeds sl: in this window iff
-          // sh_lo <= sl < sh_hi, or beyond every heavy of the row
-          const bool w = whole_row ? lv : hj ? hrank >= hb : lv && sl >= sh_lo && (sl < sh_hi || !more);
-          if (w) wr |= 1u << j;
-          oa[j] = (lv && !hj && any_heavy ? hslot : pos0 + (uint32_t)j) - r.lead;
-          op[j] = hj ? 1.0f : op[j];
-          hrank += hj ? 1u : 0u;
+          const bool lv = (live >> j) & 1, hj = op[j] < 0.0f;
+          if (!whole_row) {
+            // a light's alias is the first heavy whose surplus prefix exceeds sl: in this window iff
+            // sh_lo <= sl < sh_hi, or beyond every heavy of the row
+            const bool w = hj ? hrank >= hb : lv && sl >= sh_lo && (sl < sh_hi || !more);
+            if (w) wr |= 1u << j;
+            hrank += hj ? 1u : 0u;
+          }
+          oa[j] = (lv && !hj && any_heavy) ? hal : self0 + (uint32_t)j;
+          op[j] = fabsf(op[j]);
           // heavies of the window whose surplus prefix lies in (sl, sl + D]: this light finishes them
           sl += dl[j];
           if (hv <= sl) {
             do {
-              s_prob[b] = residual_prob(L.one + hv - sl, L);
+              s_prob[b] = residual_below(sl - hv);
               ++b;
-              hv = s_sh[b];
+              hv = hvn;
+              hal = haln;
+              hvn = s_sh[b + 1];
+              haln = s_slot[b + 1] - r.lead;
             } while (hv <= sl);
-            hslot = s_slot[b];
           }
         }
+        if (whole_row) wr = live;
+      }
+      // The weights of the next chunk, requested at the top of this iteration, are waited for here, before this
+      // chunk's stores are issued: loads and stores complete in one in-order count, so a wait for the load placed
+      // after the stores (at its first use in the next iteration) would wait for the stores as well.
+      wait_for_chunk(nx);
+      if (wr) {
+        AliasEntry* const t0 = table + r.base + pos0;
 #pragma unroll
         for (int q = 0; q < ST_PER / 4; ++q) {
           const uint32_t m = (wr >> (4 * q)) & 15u;
-          AliasEntry* t = table + r.base + pos0 + 4 * q;
+          AliasEntry* t = t0 + 4 * q;
           if (m == 15u) {
             const float p4[4] = {op[4 * q], op[4 * q + 1], op[4 * q + 2], op[4 * q + 3]};
             const uint32_t a4[4] = {oa[4 * q], oa[4 * q + 1], oa[4 * q + 2], oa[4 * q + 3]};

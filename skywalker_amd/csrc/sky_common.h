@@ -396,4 +396,60 @@ __device__ __forceinline__ WSum3 group_sum_wsum3(WSum3 s) {
   return s;
 }
 
+// Minimum over the wavefront; every lane receives it.
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+  v = min(v, dpp0<DPP_QUAD_XOR1, 0xF>(v));
+  v = min(v, dpp0<DPP_QUAD_XOR2, 0xF>(v));
+  v = min(v, dpp0<DPP_ROW_HALF_MIRROR, 0xF>(v));
+  v = min(v, dpp0<DPP_ROW_MIRROR, 0xF>(v));
+  v = min(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  v = min(v, (uint32_t)__shfl_xor((int)v, 32, 64));
+  return v;
+}
+
+// Residual probability of a heavy whose surplus prefix lies d units (d < 2^40) below the deficit prefix of the
+// light that finishes it: (2^40 - d) * 2^-40, the value residual_prob gives for 2^40 + SH - SL.  d below 2^52
+// becomes a double by the 2^52 trick; 1 - d * 2^-40 is a multiple of 2^-40 in (0, 1] and therefore exact.
+__device__ __forceinline__ float residual_below(uint64_t d) {
+  const double x = __longlong_as_double((long long)(d | 0x4330000000000000ull)) - 4503599627370496.0;
+  return (float)fma(x, -1.0 / 1099511627776.0, 1.0);
+}
+
+// The exact sum of a row without 128-bit work per entry.  Every clamped weight is a multiple of
+// u = 2^(e - 150), e the smallest exponent field among the nonzero ones; when e >= 86 no weight loses anything
+// to the floor of w * 2^64, and when the fp64 sum of the weights stays below 2^53 u every partial sum of
+// the (positive) terms is a multiple of u below 2^53 u, so every addition was exact in whatever order the lanes
+// added: the fp64 sum then equals double(S) of the 128-bit definition bit for bit.  (A sum that was rounded
+// somewhere is at least 2^53 u, because rounding is monotone and 2^53 u is representable: the test cannot pass
+// by accident.)  `mn` = min over the row of (weight bits - 1), unsigned: zero weights wrap to 2^32 - 1 and drop
+// out, a weight of the form 2^k counts with the exponent below its own, which only makes the test stricter.
+__device__ __forceinline__ bool plain_sum_is_exact(double sum, uint32_t mn) {
+  const int e = (int)(mn >> 23);  // 511 for a row without a nonzero weight
+  return e >= 86 && sum < ldexp(1.0, e - 97);
+}
+
+// Minimum of a 32-bit value over aligned groups of G lanes; every lane of the group receives it.
+template <int G>
+__device__ __forceinline__ uint32_t group_min_u32(uint32_t v) {
+  v = min(v, dpp0<DPP_QUAD_XOR1, 0xF>(v));
+  if (G >= 4) v = min(v, dpp0<DPP_QUAD_XOR2, 0xF>(v));
+  if (G >= 8) v = min(v, dpp0<DPP_ROW_HALF_MIRROR, 0xF>(v));
+  if (G >= 16) v = min(v, dpp0<DPP_ROW_MIRROR, 0xF>(v));
+  if (G >= 32) v = min(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  if (G >= 64) v = min(v, (uint32_t)__shfl_xor((int)v, 32, 64));
+  return v;
+}
+
+// classify_small_unmasked with one instruction less per step: t by one fused multiply-add (the product with 2^F
+// is exact, so the result is rounded once, as (p - 1) * 2^F is), the amount cut out of the 2^52 sum by a mask.
+__device__ __forceinline__ Entry classify_small_fma(double wd, const Ledger& L, double neg_fs) {
+  Entry e;
+  e.p = wd * L.scale;
+  const double t = fma(e.p, L.fs, neg_fs);
+  e.heavy = t >= 0.5;
+  const double a = fmax(fabs(t), e.heavy ? 1.0 : 0.0);  // |t| < 0.5 for a light with t > 0: rounds to the deficit 0
+  e.amount = (uint64_t)__double_as_longlong(a + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
+  return e;
+}
+
 }  // namespace sky
