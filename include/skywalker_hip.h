@@ -222,6 +222,12 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      "online_full_build" (default -1): how sky_walk_online serves a static bias on a graph without tables:
  *      0 builds, before every step, the rows the walkers stand on; 1 builds every row first and walks as
  *      sky_walk_offline does; -1 takes whichever is estimated to be faster.  The paths are the same.
+ *      "online_device_sized" (default 1): sky_sample_online and the step-by-step form of sky_walk_online build the
+ *      rows of a frontier without the host ever learning how many they are: the length of the list and the sizes of
+ *      its degree classes stay on the device, every build kernel finds its rows through them, and the call waits for
+ *      the device only once, at its end (a walk also learns that no walker is left through pinned host words that it
+ *      reads without waiting).  0 makes the host read the size of every frontier and size the launches exactly, which
+ *      waits twice per hop or step.  Same results.
  *      "walk_compact_every" (default 0): k > 0 makes sky_walk_offline run k steps per launch and hand the next
  *      launch the list of walkers that are still walking (the reference's walker queue,
  *      include/sampler_result.cuh:646-669), so that walkers that have stopped no longer hold a lane; 0 keeps every

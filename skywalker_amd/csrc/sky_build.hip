@@ -24,6 +24,9 @@
 // 64 to 512 threads per vertex with the row's prefix arrays in LDS (rows up to 4093 entries),
 // and the tile-parallel path of sky_build_tiled.hip for longer rows.
 #include <algorithm>
+#include <functional>
+#include <utility>
+#include <vector>
 
 #include "sky_build_common.h"
 #include "sky_graph.h"
@@ -219,18 +222,41 @@ __device__ __forceinline__ bool group_build_row(uint32_t off, uint32_t d, const 
   return row_ok || d == 0;
 }
 
-template <int G, int PER>
+// Where a class kernel finds its rows.  A build whose class sizes the host knows passes the class's segment of the
+// row list and its length, and launches exactly the workgroups the rows need (dev null).  A build whose sizes only
+// the device knows (the rows of a frontier that the host never waits for) passes the whole list and the counter
+// block of the binning pass: the class's rows start after those of the classes before it, and a grid of fixed
+// size strides over them.
+__device__ __forceinline__ void class_segment(const uint32_t* __restrict__ dev, int cls, int ncls, uint32_t& start,
+                                              uint32_t& count) {
+  if (!dev) return;
+  uint32_t st = 0;
+  for (int c = 0; c < cls; ++c) st += dev[c];
+  uint32_t n = 0;
+  for (int c = cls; c < cls + ncls; ++c) n += dev[c];
+  start = st;
+  count = n;
+}
+
+template <int G, int PER, bool DEV = false>
 __global__ __launch_bounds__(256) void build_group_kernel(const RowRef* __restrict__ vlist, uint32_t count,
+                                                          const uint32_t* __restrict__ dev, int cls,
                                                           const float* __restrict__ wgt,
                                                           AliasEntry* __restrict__ table,
                                                           int8_t* __restrict__ valid) {
   __shared__ uint64_t s_pre[2 * 256 * PER];
   __shared__ uint8_t s_hs[256 * PER];
-  const uint32_t grp = (blockIdx.x * 256u + threadIdx.x) / G;
-  RowRef rr{0, 0, 0, 0};
-  if (grp < count) rr = vlist[grp];
-  const bool ok = group_build_row<G, PER>(rr.off, rr.d, wgt, table, s_pre, s_hs);
-  if ((threadIdx.x & (G - 1)) == 0 && !ok) valid[rr.v] = 0;  // the binning pass has set it
+  uint32_t start = 0;
+  if (DEV) class_segment(dev, cls, 1, start, count);
+  constexpr uint32_t ROWS = 256 / G;  // rows per workgroup and round
+  // DEV false: one round per workgroup, and the loop is none
+  for (uint32_t b = blockIdx.x; DEV ? b * ROWS < count : b == blockIdx.x; b += DEV ? gridDim.x : 1u) {
+    const uint32_t grp = b * ROWS + threadIdx.x / G;
+    RowRef rr{0, 0, 0, 0};
+    if (grp < count) rr = vlist[start + grp];
+    const bool ok = group_build_row<G, PER>(rr.off, rr.d, wgt, table, s_pre, s_hs);
+    if ((threadIdx.x & (G - 1)) == 0 && !ok) valid[rr.v] = 0;  // the binning pass has set it
+  }
 }
 
 // ---------------------------------------------------------------- binning
@@ -244,6 +270,7 @@ constexpr int BIN_ITEMS = 4;      // vertices per thread and step
 
 __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restrict__ xadj,
                                                         const uint32_t* __restrict__ src, uint32_t n,
+                                                        const uint32_t* __restrict__ n_dev,
                                                         uint32_t per_block, int listed_from,
                                                         uint32_t* __restrict__ blk_cnt,
                                                         unsigned long long* __restrict__ class_edges) {
@@ -254,6 +281,7 @@ __global__ __launch_bounds__(256) void bin_count_kernel(const uint32_t* __restri
     s_edges[threadIdx.x] = 0;
   }
   __syncthreads();
+  if (n_dev) n = min(n, *n_dev);  // the host passed an upper bound
   const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
   uint32_t tiny_edges = 0;  // rows of 1..2 entries, the commonest kind of a power-law graph, stay out of the LDS atomics
   // four vertices per thread and step: their loads are in flight together (one at a time, the loop waits a
@@ -355,6 +383,7 @@ __device__ __forceinline__ bool tiny_row(uint32_t off, uint32_t d, const float* 
 __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __restrict__ xadj,
                                                           const float* __restrict__ wgt,
                                                           const uint32_t* __restrict__ src, uint32_t n,
+                                                          const uint32_t* __restrict__ n_dev,
                                                           uint32_t per_block, int listed_from,
                                                           const uint32_t* __restrict__ counts,
                                                           const uint32_t* __restrict__ blk_off,
@@ -371,6 +400,7 @@ __global__ __launch_bounds__(256) void bin_scatter_kernel(const uint32_t* __rest
   }
   __syncthreads();
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (n_dev) n = min(n, *n_dev);
   const uint32_t lo = blockIdx.x * per_block, hi = min(n, lo + per_block);
   for (uint32_t chunk = lo; chunk < hi; chunk += 256u * BIN_ITEMS) {
     uint32_t nt = 0;  // wave-uniform: rows in this wavefront's list
@@ -749,9 +779,9 @@ __global__ __launch_bounds__(ROWT) void build_lds_kernel(const RowRef* __restric
 constexpr uint64_t MERGE_CNT = 1ull << 52;
 constexpr uint32_t MERGE_SELF = 0x80000000u;  // "prob 1, alias self" in the per-heavy result word
 
-template <int ROWT, int PER, int MINW = 4>
-__global__ __launch_bounds__(ROWT, MINW) void build_merge_kernel(const RowRef* __restrict__ vlist,
-                                                           const uint32_t* __restrict__ xadj,
+template <int ROWT, int PER, int MINW = 4, int DEV = 0>  // DEV 1: segment from the device, one row per workgroup; 2: striding grid
+__global__ __launch_bounds__(ROWT, MINW) void build_merge_kernel(const RowRef* __restrict__ vlist, uint32_t count,
+                                                           const uint32_t* __restrict__ dev, int cls,
                                                            const float* __restrict__ wgt,
                                                            AliasEntry* __restrict__ table, int8_t* __restrict__ valid) {
   // PER consecutive slots per thread, counted from the row's 16-byte aligned start; a thread moves them as
@@ -772,7 +802,13 @@ __global__ __launch_bounds__(ROWT, MINW) void build_merge_kernel(const RowRef* _
   __shared__ uint32_t s_mn[NW];
   __shared__ uint64_t s_ex[3 * NW];
 
-  const RowRef rr = vlist[blockIdx.x];
+  uint32_t start = 0;
+  if (DEV) class_segment(dev, cls, 1, start, count);
+  if (DEV == 1 && blockIdx.x >= count) return;
+  // DEV 0 and 1: one row per workgroup, and the loop is none
+  for (uint32_t row = blockIdx.x; DEV == 2 ? row < count : row == blockIdx.x; row += DEV == 2 ? gridDim.x : 1u) {
+  if (DEV == 2 && row != blockIdx.x) __syncthreads();  // the arrays in LDS are about to be rewritten
+  const RowRef rr = vlist[start + row];
   const uint32_t v = rr.v, off = rr.off, d = rr.d;
   const uint32_t base = off & ~3u, lead = off - base, span = lead + d;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -854,7 +890,7 @@ __global__ __launch_bounds__(ROWT, MINW) void build_merge_kernel(const RowRef* _
     for (int j = 0; j < PER; ++j)
       if ((live >> j) & 1) table[base + pos0 + j] = AliasEntry{0.0f, SKY_INVALID};
     if (tid == 0) valid[v] = 0;
-    return;
+    continue;
   }
   const Ledger L = make_ledger_small(d, rsum);
   const double neg_fs = -L.fs;
@@ -975,6 +1011,7 @@ __global__ __launch_bounds__(ROWT, MINW) void build_merge_kernel(const RowRef* _
       }
     }
   }
+  }  // rows of this workgroup
 }
 
 // ---------------------------------------------------------------- rows beyond LDS: global scratch
@@ -1315,6 +1352,11 @@ int prepare_build_scratch(uint32_t max_rows) {
     SKY_TRY(enable_big_lds(build_merge_kernel<768, 6>, (768 * 6 + 2) * 14));
     SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
 #undef SKY_BIG
+#define SKY_BIG(NW) SKY_TRY(enable_big_lds((build_merge_kernel<64 * NW, 8, 4, 1>), (64 * NW * 8 + 2) * 14))
+    SKY_TRY(enable_big_lds((build_merge_kernel<512, 10, 4, 1>), (512 * 10 + 2) * 14));
+    SKY_TRY(enable_big_lds((build_merge_kernel<768, 6, 4, 1>), (768 * 6 + 2) * 14));
+    SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
+#undef SKY_BIG
     sc.lds_enabled = true;
   }
   return SKY_OK;
@@ -1356,11 +1398,13 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t step = 256u * BIN_ITEMS;
     const uint32_t per_block = ((n + BIN_BLOCKS - 1) / BIN_BLOCKS + step - 1) / step * step;
     const uint32_t blocks = (n + per_block - 1) / per_block;
-    hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n, per_block, listed_from,
-                       sc.blk_cnt, reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
+    hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n, (const uint32_t*)nullptr,
+                       per_block, listed_from, sc.blk_cnt,
+                       reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
     hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(256), 0, st, sc.blk_cnt, blocks, sc.counters);
-    hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n, per_block,
-                       listed_from, sc.counters, sc.blk_cnt, sc.vlist, g->table, g->valid);
+    hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n,
+                       (const uint32_t*)nullptr, per_block, listed_from, sc.counters, sc.blk_cnt, sc.vlist, g->table,
+                       g->valid);
     // The class sizes decide the launches that follow.  Those of all vertices depend on xadj alone and are kept
     // with the graph after the first time; any other list of rows is waited for.
     const bool all_rows = src == nullptr && n == g->V;
@@ -1404,7 +1448,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     if (cnt) {
       const uint32_t per_block = 256 / G;
       hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, fan.next(), vlist + starts[cls],
-                         cnt, g->adjwgt, g->table, g->valid);
+                         cnt, (const uint32_t*)nullptr, 0, g->adjwgt, g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
@@ -1429,8 +1473,8 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const size_t bytes = ((size_t)rowt * per + 2) * 14;
-      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(), vlist + starts[cls], g->xadj, g->adjwgt,
-                         g->table, g->valid);
+      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(), vlist + starts[cls], cnt,
+                         (const uint32_t*)nullptr, 0, g->adjwgt, g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
@@ -1533,6 +1577,151 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
   }
   return fan.join();
+}
+
+// ---------------------------------------------------------------- builds that never wait for the device
+// The rows of a frontier: how many there are, and how many fall into each degree class, is known on the device
+// only.  The binning kernels take the length of the list from a device word, every class kernel finds its segment
+// of the row list through the counter block (class_segment) and strides over it with a grid of fixed size.  Which
+// classes can hold a row at all depends on the graph alone: a census of all vertices, taken once per graph, lets
+// the host skip the launches of the classes the graph does not populate.
+// Most workgroups of a launch, by workgroup size: enough to fill every CU several times over (a class that
+// turns out small leaves most of them with nothing to do, which costs microseconds).
+constexpr uint32_t DEV_GRID_STREAM = 512;
+constexpr uint32_t dev_grid_cap(int threads) { return threads <= 64 ? 16384u : threads <= 256 ? 8192u : 2048u; }
+
+bool build_rows_dev_possible(const sky_graph* g) { return g_row_merge && tiled_max_tiles() == (1u << 22); }
+
+int ensure_class_census(sky_graph* g) {
+  if (g->bin_known || g->V == 0) return SKY_OK;
+  hipStream_t st = g->stream;
+  SKY_TRY(prepare_build_scratch(1));
+  BuildScratch& sc = g_scratch;
+  struct {
+    uint32_t counts[2 * CLS_COUNT];
+    unsigned long long edges[CLS_COUNT];
+  } host = {};
+  const uint32_t n = g->V, step = 256u * BIN_ITEMS;
+  const uint32_t per_block = ((n + BIN_BLOCKS - 1) / BIN_BLOCKS + step - 1) / step * step;
+  const uint32_t blocks = (n + per_block - 1) / per_block;
+  SKY_HIP(hipMemsetAsync(sc.counters, 0, COUNTER_BYTES, st));
+  hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, (const uint32_t*)nullptr, n,
+                     (const uint32_t*)nullptr, per_block, (int)CLS_G2, sc.blk_cnt,
+                     reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
+  hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(256), 0, st, sc.blk_cnt, blocks, sc.counters);
+  SKY_HIP(hipMemcpyAsync(&host, sc.counters, COUNTER_BYTES, hipMemcpyDeviceToHost, st));
+  SKY_HIP(hipStreamSynchronize(st));
+  for (int c = 0; c < CLS_COUNT; ++c) {
+    g->bin_counts[c] = host.counts[c];
+    g->bin_edges[c] = host.edges[c];
+  }
+  g->bin_known = true;
+  g->bin_listed_from = CLS_G2;
+  return SKY_OK;
+}
+
+int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uint32_t n_upper) {
+  if (n_upper == 0) return SKY_OK;
+  if (!build_rows_dev_possible(g) || !g->bin_known)
+    return fail(SKY_ERR_STATE, "build_rows_dev: needs the class census and rows the streaming kernel takes");
+  hipStream_t st = g->stream;
+  g->has_walk_index = false;
+  BuildScratch& sc = g_scratch;
+  const uint32_t step = 256u * BIN_ITEMS;
+  const uint32_t per_block = ((n_upper + BIN_BLOCKS - 1) / BIN_BLOCKS + step - 1) / step * step;
+  const uint32_t blocks = (n_upper + per_block - 1) / per_block;
+  SKY_HIP(hipMemsetAsync(sc.counters, 0, COUNTER_BYTES, st));
+  hipLaunchKernelGGL(bin_count_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, src, n_upper, n_dev, per_block,
+                     (int)CLS_G2, sc.blk_cnt, reinterpret_cast<unsigned long long*>(sc.counters + 2 * CLS_COUNT));
+  hipLaunchKernelGGL(bin_offsets_kernel, dim3(CLS_COUNT), dim3(256), 0, st, sc.blk_cnt, blocks, sc.counters);
+  hipLaunchKernelGGL(bin_scatter_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjwgt, src, n_upper, n_dev,
+                     per_block, (int)CLS_G2, sc.counters, sc.blk_cnt, sc.vlist, g->table, g->valid);
+  // a class of the graph holds bin_counts[c] rows at most (bin_edges tells whether it holds any: the counts of the
+  // census leave out the classes that a large full build does not list)
+  auto rows_of = [&](int cls) -> uint32_t {
+    if (g->bin_edges[cls] == 0) return 0;
+    const uint32_t in_graph = g->bin_listed_from <= cls ? g->bin_counts[cls] : n_upper;
+    return std::min(n_upper, std::max(1u, in_graph));
+  };
+  const uint32_t* const dev = sc.counters;
+  const RowRef* const vlist = sc.vlist;
+  // the class kernels are independent of one another: they go out in turn over the graph's stream and its side streams
+  StreamFan fan(g, st);
+  if (g_build_streams && n_upper >= 4096) SKY_TRY(fan.start());
+  // Rows of 8190 entries and more first, because theirs is the longest chain of launches.  The classes STREAM,
+  // STREAM_LAST, STREAM_WIDE, HUGE lie back to back.  What the graph holds of them decides, as in a build of all
+  // rows, which go to the streaming kernel (one workgroup per row) and which are built tile by tile by the whole
+  // GPU: the two longest classes always are (a frontier holds a few such rows at most, and one workgroup would need
+  // a millisecond for one), the other two when the graph has too few of their rows to fill the GPU with one
+  // workgroup each.
+  static_assert(CLS_STREAM_LAST == CLS_STREAM + 1 && CLS_STREAM_WIDE == CLS_STREAM + 2 && CLS_HUGE == CLS_STREAM + 3,
+                "the lists of the long rows lie back to back");
+  const bool narrow_tiled = g->bin_edges[CLS_STREAM] + g->bin_edges[CLS_STREAM_LAST] <= g_stream_min_edges;
+  const uint32_t stream_rows = narrow_tiled ? 0 : rows_of(CLS_STREAM) + rows_of(CLS_STREAM_LAST);
+  const int t_first = narrow_tiled ? CLS_STREAM : CLS_STREAM_WIDE;
+  uint32_t tiled_rows = 0;
+  uint64_t tiled_edges = 0;
+  for (int c = t_first; c <= CLS_HUGE; ++c) {
+    tiled_rows += rows_of(c);
+    tiled_edges += g->bin_edges[c];
+  }
+  if (tiled_rows) {
+    StreamSwap sw(g, fan.next());
+    SKY_TRY(build_rows_tiled_dev(g, vlist, dev, t_first, CLS_HUGE - t_first + 1, tiled_rows, tiled_edges));
+  }
+  // the streaming kernel fills the LDS of every CU it reaches: the tile-parallel path, whose first kernels are small,
+  // is enqueued before it
+  if (stream_rows) {
+    StreamSwap sw(g, fan.next());
+    SKY_TRY(build_rows_stream_dev(g, vlist, dev, 2, std::min(DEV_GRID_STREAM, stream_rows)));
+  }
+  auto grp = [&](int cls, auto kernel, int G) {
+    const uint32_t rows = rows_of(cls);
+    if (!rows) return;
+    const uint32_t per = 256 / G;
+    hipLaunchKernelGGL(kernel, dim3(std::min(dev_grid_cap(256), (rows + per - 1) / per)), dim3(256), 0, fan.next(), vlist,
+                       0u, dev, cls, g->adjwgt, g->table, g->valid);
+  };
+  auto mrg = [&](int cls, auto kernel, int rowt, int per) {
+    const uint32_t rows = rows_of(cls);
+    if (!rows) return;
+    const size_t bytes = ((size_t)rowt * per + 2) * 14;
+    // one wavefront per row: a striding grid; larger workgroups: one per row the class can hold (the code of a
+    // loop over rows costs these kernels registers they do not have)
+    hipLaunchKernelGGL(kernel, dim3(rowt <= 64 ? std::min(dev_grid_cap(rowt), rows) : rows), dim3(rowt), bytes, fan.next(),
+                       vlist, 0u, dev, cls, g->adjwgt, g->table, g->valid);
+  };
+  // The class kernels go out in the order of the classes' sizes in the graph, the largest first: a frontier mirrors
+  // the graph, and the streams should not end on a long kernel that started last.
+  std::vector<std::pair<unsigned long long, std::function<void()>>> queue;
+#define SKY_Q(CLS, CALL) queue.emplace_back(g->bin_edges[CLS], [&] { CALL; })
+  SKY_Q(CLS_G2, grp(CLS_G2, (build_group_kernel<2, 4, true>), 2));
+  SKY_Q(CLS_G4, grp(CLS_G4, (build_group_kernel<4, 4, true>), 4));
+  SKY_Q(CLS_G8, grp(CLS_G8, (build_group_kernel<8, 4, true>), 8));
+  SKY_Q(CLS_G16, grp(CLS_G16, (build_group_kernel<16, 4, true>), 16));
+  SKY_Q(CLS_G32, grp(CLS_G32, (build_group_kernel<32, 4, true>), 32));
+  SKY_Q(CLS_G32S, grp(CLS_G32S, (build_group_kernel<32, 5, true>), 32));
+  SKY_Q(CLS_G32X, grp(CLS_G32X, (build_group_kernel<32, 6, true>), 32));
+  SKY_Q(CLS_LDS_W1, mrg(CLS_LDS_W1, (build_merge_kernel<64, 4, 4, 2>), 64, 4));
+  SKY_Q(CLS_LDS_W2, mrg(CLS_LDS_W2, (build_merge_kernel<64, 8, 4, 2>), 64, 8));
+#define SKY_MW(NW) SKY_Q(CLS_MW2 + NW - 2, mrg(CLS_MW2 + NW - 2, (build_merge_kernel<64 * NW, 8, 4, 1>), 64 * NW, 8))
+  SKY_MW(2);
+  SKY_Q(CLS_MW2 + 1, mrg(CLS_MW2 + 1, (build_merge_kernel<256, 6, 4, 1>), 256, 6));
+  SKY_MW(4);
+  SKY_Q(CLS_MW2 + 3, mrg(CLS_MW2 + 3, (build_merge_kernel<256, 10, 4, 1>), 256, 10));
+  SKY_Q(CLS_MW2 + 4, mrg(CLS_MW2 + 4, (build_merge_kernel<512, 6, 4, 1>), 512, 6));
+  SKY_Q(CLS_MW2 + 5, mrg(CLS_MW2 + 5, (build_merge_kernel<256, 14, 4, 1>), 256, 14));
+  SKY_MW(8);
+  SKY_Q(CLS_MW2 + 7, mrg(CLS_MW2 + 7, (build_merge_kernel<768, 6, 4, 1>), 768, 6));
+  SKY_Q(CLS_MW2 + 8, mrg(CLS_MW2 + 8, (build_merge_kernel<512, 10, 4, 1>), 512, 10));
+  SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
+#undef SKY_MW
+#undef SKY_Q
+  std::stable_sort(queue.begin(), queue.end(), [](const auto& a, const auto& b) { return a.first > b.first; });
+  for (auto& q : queue) q.second();
+  SKY_TRY(fan.join());
+  SKY_HIP(hipGetLastError());
+  return SKY_OK;
 }
 
 int build_all_tables(sky_graph* g, double* seconds) {

@@ -173,8 +173,10 @@ __device__ __forceinline__ uint64_t uniform_u64(uint64_t x) {
   return ((uint64_t)uniform_u32((uint32_t)(x >> 32)) << 32) | uniform_u32((uint32_t)x);
 }
 
+template <bool DEV>
 __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __restrict__ first_list, uint32_t n_first,
-                                                            const RowRef* __restrict__ vlist,
+                                                            const RowRef* __restrict__ vlist, uint32_t n_rows,
+                                                            const uint32_t* __restrict__ dev, int dev_ncls,
                                                             const float* __restrict__ wgt,
                                                             AliasEntry* __restrict__ table,
                                                             int8_t* __restrict__ valid) {
@@ -187,9 +189,20 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   __shared__ uint64_t s_a[2][ST_NW];  // two sets of wavefront sums, used alternately
   __shared__ uint32_t s_c[2][ST_NW];
   __shared__ uint32_t s_next;  // slot of the first heavy after the window
-  // the first n_first workgroups take the rows of first_list (the longest ones), the others those of vlist
-  const RowRef rr = blockIdx.x < n_first ? first_list[blockIdx.x] : vlist[blockIdx.x - n_first];
+  // Class sizes known to the host (dev null): one workgroup per row, the first n_first take the rows of first_list
+  // (the longest ones), the others those of vlist.  Sizes known to the device alone: the rows of the first dev_ncls
+  // streaming classes lie back to back in vlist, after those of the classes before them, and the grid strides over them.
+  uint32_t start = 0, count = n_first + n_rows;
+  if (DEV) {
+    for (int c = 0; c < CLS_STREAM; ++c) start += dev[c];
+    count = 0;
+    for (int c = CLS_STREAM; c < CLS_STREAM + dev_ncls; ++c) count += dev[c];
+  }
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  // DEV false: one row per workgroup, and the loop is none
+  for (uint32_t row = blockIdx.x; DEV ? row < count : row == blockIdx.x; row += DEV ? gridDim.x : 1u) {
+  if (DEV && row != blockIdx.x) __syncthreads();  // the window and the sums in LDS are about to be rewritten
+  const RowRef rr = DEV ? vlist[start + row] : (row < n_first ? first_list[row] : vlist[row - n_first]);
   StreamRow r;
   r.base = rr.off & ~3u;
   r.lead = rr.off - r.base;
@@ -266,7 +279,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
         if (idx >= r.lead && idx < r.span) table[r.base + idx] = AliasEntry{0.0f, SKY_INVALID};
       }
     if (tid == 0) valid[rr.v] = 0;
-    return;
+    continue;
   }
   const Ledger L = make_ledger_small(rr.d, row_sum);
 
@@ -544,14 +557,24 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
     hc_cc = last_hc;
     __syncthreads();  // the lists are rewritten by the next window, whose stores must not overtake this sweep's
   }
+  }  // rows of this workgroup
 }
 
 // Builds the n_first rows of `first_list` and the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each) in one
 // launch that starts with the former.
 int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n) {
   if (n + n_first == 0) return SKY_OK;
-  hipLaunchKernelGGL(build_stream_kernel, dim3(n + n_first), dim3(ST_T), 0, g->stream, first_list, n_first, rows_list,
-                     g->adjwgt, g->table, g->valid);
+  hipLaunchKernelGGL(build_stream_kernel<false>, dim3(n + n_first), dim3(ST_T), 0, g->stream, first_list, n_first, rows_list, n,
+                     (const uint32_t*)nullptr, 0, g->adjwgt, g->table, g->valid);
+  return SKY_OK;
+}
+
+// The rows of the first ncls streaming classes of a list whose class sizes only the device knows (`dev`: the counter
+// block of the binning pass): `grid` workgroups stride over them.
+int build_rows_stream_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int ncls, uint32_t grid) {
+  if (grid == 0) return SKY_OK;
+  hipLaunchKernelGGL(build_stream_kernel<true>, dim3(grid), dim3(ST_T), 0, g->stream, (const RowRef*)nullptr, 0u, vlist, 0u, dev,
+                     ncls, g->adjwgt, g->table, g->valid);
   return SKY_OK;
 }
 

@@ -88,7 +88,12 @@ struct TiledCounters {
 
 // Geometry of every row; each block reserves a run of tile ids (and of prefix-array slots) for its
 // rows with one atomic.  Tile numbering therefore depends on scheduling; no result does.
+// `dev` (may be null): the counter block of a binning pass whose class sizes the host does not know.  The rows are
+// then those of the classes cls .. cls + ncls - 1, which lie back to back in vlist after the rows of the classes
+// before them; `count` is an upper bound, and the rows between the true number and the bound are recorded as rows
+// without tiles, which every later kernel passes over.
 __global__ __launch_bounds__(256) void tiled_rows_kernel(const RowRef* __restrict__ vlist, uint32_t count,
+                                                         const uint32_t* __restrict__ dev, int cls, int ncls,
                                                          const uint32_t* __restrict__ xadj, uint32_t max_tiles,
                                                          TiledRow* __restrict__ rows,
                                                          TiledCounters* __restrict__ ctr) {
@@ -96,6 +101,14 @@ __global__ __launch_bounds__(256) void tiled_rows_kernel(const RowRef* __restric
   __shared__ unsigned long long s_base;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t r = blockIdx.x * 256u + tid;
+  const uint32_t bound = count;
+  if (dev) {
+    uint32_t st = 0, n = 0;
+    for (int c = 0; c < cls; ++c) st += dev[c];
+    for (int c = cls; c < cls + ncls; ++c) n += dev[c];
+    vlist += st;
+    count = min(count, n);
+  }
   TiledRow row = {};
   uint32_t nt = 0;
   bool skip = false;
@@ -129,6 +142,8 @@ __global__ __launch_bounds__(256) void tiled_rows_kernel(const RowRef* __restric
     row.tile0 = (uint32_t)s_base + before + inc - nt;
     row.bofs = row.tile0 + (uint32_t)(s_base >> 32) + tid;  // every row owns ntiles + 1 prefix slots
     rows[r] = row;
+  } else if (r < bound) {
+    rows[r] = row;  // no tiles
   }
 }
 
@@ -626,8 +641,9 @@ void set_tiled_max_tiles(uint32_t n) { g_tiled_max_tiles = std::min<uint32_t>(st
 // entries of the listed rows when the caller knows it (0 otherwise): the tile grids are then sized by
 // the bound edges / TILE + 2 n, with empty records for the tiles that do not exist, and the host does
 // not wait for the device to count them.
-int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
-                     uint64_t edges) {
+// dev non-null: see tiled_rows_kernel; n and edges are then upper bounds, and the call never waits for the device.
+static int build_rows_tiled_any(sky_graph* g, const RowRef* rows_list, uint32_t n, const uint32_t* dev, int cls, int ncls,
+                                uint32_t* skipped, EventTimer* tm, uint64_t edges) {
   hipStream_t st = g->stream;
   TiledScratch& sc = g_tiled;
   *skipped = 0;
@@ -641,7 +657,7 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
   }
   if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, sizeof(TiledCounters)));
   SKY_HIP(hipMemsetAsync(sc.totals, 0, sizeof(TiledCounters), st));
-  hipLaunchKernelGGL(tiled_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, st, rows_list, n, g->xadj,
+  hipLaunchKernelGGL(tiled_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, st, rows_list, n, dev, cls, ncls, g->xadj,
                      g_tiled_max_tiles, sc.rows, sc.totals);
   const bool bounded = edges != 0 && g_tiled_max_tiles == TILED_MAX_TILES && edges / TILE + 2ull * n < (1ull << 31);
   uint32_t ntiles, nslots;
@@ -696,6 +712,19 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
                      sc.BH, sc.nfh, sc.ranges, g->table, g->valid);
   if (tm) SKY_TRY(tm->mark("tiled_emit", edges));
   return SKY_OK;
+}
+
+int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
+                     uint64_t edges) {
+  return build_rows_tiled_any(g, rows_list, n, nullptr, 0, 0, skipped, tm, edges);
+}
+
+int build_rows_tiled_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int cls, int ncls, uint32_t n_upper,
+                         uint64_t edges_upper) {
+  if (g_tiled_max_tiles != TILED_MAX_TILES || edges_upper == 0 || edges_upper / TILE + 2ull * n_upper >= (1ull << 31))
+    return fail(SKY_ERR_STATE, "build_rows_tiled_dev: the number of tiles has no usable bound");
+  uint32_t skipped = 0;
+  return build_rows_tiled_any(g, vlist, n_upper, dev, cls, ncls, &skipped, nullptr, edges_upper);
 }
 
 }  // namespace sky

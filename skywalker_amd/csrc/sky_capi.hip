@@ -195,6 +195,7 @@ int sky_graph_free(sky_graph* g) {
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   pool_release(g);
+  if (g->live_report) (void)hipHostFree(g->live_report);
   delete g;
   return SKY_OK;
 }
@@ -448,6 +449,10 @@ int sky_set_option(const char* name, long value) {
   if (!strcmp(name, "walk_compact_every")) {
     if (value < 0) return fail(SKY_ERR_ARG, "sky_set_option: walk_compact_every must be >= 0");
     set_walk_compact_every((uint32_t)value);
+    return SKY_OK;
+  }
+  if (!strcmp(name, "online_device_sized")) {
+    set_online_device_sized(value != 0);
     return SKY_OK;
   }
   if (!strcmp(name, "online_full_build")) {

@@ -41,6 +41,10 @@ struct sky_graph {
   };
   PoolBuf pool[POOL_SLOTS];
   hipEvent_t ev[2] = {nullptr, nullptr};
+  // Pinned host words into which the device reports, step by step, how many walkers of an online walk still walk;
+  // the host reads them without waiting (they lag behind the enqueued steps) to stop enqueuing once none does.
+  uint32_t* live_report = nullptr;
+  size_t live_report_cap = 0;
   // Side streams (default priority) over which a small build spreads its class kernels, the event they wait for
   // and the events the graph's stream waits for afterwards; created on first use.
   static constexpr int SIDE_STREAMS = 3;
@@ -115,15 +119,26 @@ int build_all_tables(sky_graph* g, double* seconds);
 constexpr uint32_t TILED_TILE = 1024;  // slots per tile of the tile-parallel path
 int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t* skipped, EventTimer* tm,
                      uint64_t edges);
+int build_rows_tiled_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int cls, int ncls, uint32_t n_upper,
+                         uint64_t edges_upper);
 void set_tiled_max_tiles(uint32_t n);
 constexpr uint32_t STREAM_MAX_DEG = 524287;  // longest row of the streaming classes (one workgroup takes 1.5 ms for it)
 int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n);
+int build_rows_stream_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int ncls, uint32_t grid);
+// Builds the rows listed in src[0 .. *n_dev) (n_dev: a device word the host never reads; n_upper: what it cannot
+// exceed) without waiting for the device at any point.  Needs the graph's class census and a longest row the
+// streaming kernel takes (build_rows_dev_possible).
+bool build_rows_dev_possible(const sky_graph* g);
+int ensure_class_census(sky_graph* g);
+int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uint32_t n_upper);
 void set_row_merge(bool on);
 void set_stream_min_edges(uint64_t n);
 void set_stream_wide_min_edges(uint64_t n);
 void set_build_streams(bool on);
 void set_small_in_place(int mode);
 void set_sample_distinct(bool on);
+void set_online_device_sized(bool on);
+extern bool g_online_device_sized;
 void set_walk_read_once(int mode);
 void set_build_profile(bool on);
 void set_online_full_build(int mode);

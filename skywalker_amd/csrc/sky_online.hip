@@ -129,8 +129,24 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
   unsigned long long* d_sampled = nullptr;
   uint32_t *bitmap = nullptr, *list = nullptr, *d_cnt = nullptr;
   const uint32_t words = (g->V + 31) / 32;
+  // Without a row too long for the streaming kernel, no step waits for the device: the size of a step's list stays
+  // there (build_rows_dev), and whether any walker still walks comes back through pinned host words that the host
+  // reads as they arrive, some steps behind what it has enqueued; the steps enqueued past the last walker's end find
+  // nothing to do.
+  const bool dev_sized = build_rows_dev_possible(g) && g_online_device_sized;
   auto body = [&]() -> int {
     SKY_TRY(ensure_table_storage(g));
+    if (dev_sized) {
+      SKY_TRY(ensure_class_census(g));
+      if (g->live_report_cap < len) {
+        if (g->live_report) SKY_HIP(hipHostFree(g->live_report));
+        g->live_report = nullptr;
+        g->live_report_cap = 0;
+        SKY_HIP(hipHostMalloc((void**)&g->live_report, (size_t)len * 4, hipHostMallocDefault));
+        g->live_report_cap = len;
+      }
+      for (uint32_t s = 0; s < len; ++s) g->live_report[s] = 0xFFFFFFFFu;  // "not reported yet"
+    }
     SKY_TRY(prepare_build_scratch(std::min(N, g->V)));
     SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
     d_cnt = reinterpret_cast<uint32_t*>(d_sampled + 1);
@@ -147,11 +163,19 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
         SKY_HIP(hipMemsetAsync(d_cnt, 0, 8, st));
         hipLaunchKernelGGL(walk_collect_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, N, len, s, stop_prob, seed,
                            paths, lengths, bitmap, list, d_cnt);
-        uint32_t cnt[2] = {0, 0};
-        SKY_HIP(hipMemcpyAsync(cnt, d_cnt, 8, hipMemcpyDeviceToHost, st));
-        SKY_HIP(hipStreamSynchronize(st));
-        if (cnt[1] == 0) break;  // every walker has stopped
-        SKY_TRY(build_rows(g, list, cnt[0], nullptr));
+        if (dev_sized) {
+          SKY_HIP(hipMemcpyAsync(&g->live_report[s], d_cnt + 1, 4, hipMemcpyDeviceToHost, st));
+          bool ended = false;
+          for (uint32_t k = 0; k < s && !ended; ++k) ended = *(volatile uint32_t*)&g->live_report[k] == 0;
+          if (ended) break;  // a step that has run found no walker left
+          SKY_TRY(build_rows_dev(g, list, d_cnt, std::min(N, g->V)));
+        } else {
+          uint32_t cnt[2] = {0, 0};
+          SKY_HIP(hipMemcpyAsync(cnt, d_cnt, 8, hipMemcpyDeviceToHost, st));
+          SKY_HIP(hipStreamSynchronize(st));
+          if (cnt[1] == 0) break;  // every walker has stopped
+          SKY_TRY(build_rows(g, list, cnt[0], nullptr));
+        }
         hipLaunchKernelGGL(walk_step_kernel, dim3(blocks), dim3(256), 0, st, g->xadj, g->adjncy, g->table, N,
                            len, s, seed, paths, lengths);
       }

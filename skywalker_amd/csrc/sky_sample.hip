@@ -146,14 +146,20 @@ __global__ __launch_bounds__(256) void sum_u32_kernel(const uint32_t* __restrict
 }
 
 // Collects the distinct vertices of the filled slots of hop h whose table has not been built
-// during this call: first setter of the vertex's bit appends it (one counter update per wavefront).
-__global__ __launch_bounds__(256) void frontier_collect_kernel(const uint32_t* __restrict__ data,
-                                                               const uint32_t* __restrict__ sl, uint64_t total,
-                                                               uint32_t V, HopGeom g, uint32_t* __restrict__ bitmap,
-                                                               uint32_t* __restrict__ list,
-                                                               uint32_t* __restrict__ count) {
-  const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-  bool fresh = false;
+// during this call: first setter of the vertex's bit appends it.  One counter update per workgroup of 1024
+// lanes: every append of a launch goes through one word, and a word serves its atomics one after another
+// (one update per wavefront made this kernel as long as the build it feeds).
+constexpr int COLLECT_T = 1024;
+__global__ __launch_bounds__(COLLECT_T) void frontier_collect_kernel(const uint32_t* __restrict__ data,
+                                                                     const uint32_t* __restrict__ sl, uint64_t total,
+                                                                     uint32_t V, HopGeom g, uint32_t* __restrict__ bitmap,
+                                                                     uint32_t* __restrict__ list,
+                                                                     uint32_t* __restrict__ count) {
+  __shared__ uint32_t s_n[COLLECT_T / 64];
+  __shared__ uint32_t s_base;
+  const uint64_t tid = (uint64_t)blockIdx.x * COLLECT_T + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  bool fresh = false, live = false;
   uint32_t v = 0;
   if (tid < total) {
     uint64_t si, s;
@@ -167,19 +173,38 @@ __global__ __launch_bounds__(256) void frontier_collect_kernel(const uint32_t* _
     }
     if (slot_filled(g, sl, si, s)) {
       v = data[si * g.lps + g.off + s];
-      if (v < V) {
+      live = v < V;
+    }
+  }
+  // The draws of a hop land on a few well-connected vertices again and again: the lanes of the wavefront that hold
+  // the same vertex send one atomic between them (the lanes take turns by distinct vertex, at most 64 short rounds).
+  {
+    unsigned long long todo = __ballot(live);
+    while (todo) {
+      const int first = __ffsll((long long)todo) - 1;
+      const uint32_t v0 = (uint32_t)__shfl((int)v, first, 64);
+      const unsigned long long same = __ballot(live && v == v0);
+      if (lane == first) {
         const uint32_t bit = 1u << (v & 31);
         fresh = !(atomicOr(&bitmap[v >> 5], bit) & bit);
       }
+      todo &= ~same;
     }
   }
   const unsigned long long m = __ballot(fresh);
-  if (m) {
-    const int lane = threadIdx.x & 63, first = __ffsll((long long)m) - 1;
-    uint32_t base = 0;
-    if (lane == first) base = atomicAdd(count, (uint32_t)__popcll(m));
-    base = (uint32_t)__shfl((int)base, first, 64);
-    if (fresh) list[base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = v;
+  if (lane == 0) s_n[wave] = (uint32_t)__popcll(m);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t n = 0;
+#pragma unroll
+    for (int w = 0; w < COLLECT_T / 64; ++w) n += s_n[w];
+    s_base = n ? atomicAdd(count, n) : 0u;
+  }
+  __syncthreads();
+  if (fresh) {
+    uint32_t base = s_base;
+    for (int w = 0; w < wave; ++w) base += s_n[w];
+    list[base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = v;
   }
 }
 
@@ -191,6 +216,8 @@ __global__ __launch_bounds__(256) void sample_init_kernel(const uint32_t* __rest
 
 static bool g_sample_distinct = false;
 void set_sample_distinct(bool on) { g_sample_distinct = on; }
+bool g_online_device_sized = true;  // option "online_device_sized": 0 makes the online modes wait for every frontier size
+void set_online_device_sized(bool on) { g_online_device_sized = on; }
 
 int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
                 uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds) {
@@ -202,6 +229,9 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
       if (fanout[h] > DISTINCT_MAX_K) return fail(SKY_ERR_LIMIT, "sample: distinct children need fanouts of at most 64");
   }
   if (g->has_tables) online = false;  // every row is already there: nothing to build on the way
+  // Rows longer than the streaming kernel takes need the tile-parallel path, whose launches the host sizes: a graph
+  // with such a row waits for the size of every frontier, any other graph never waits inside the call.
+  const bool dev_sized = online && build_rows_dev_possible(g) && g_online_device_sized;
   std::vector<uint64_t> width(hops), off(hops), loff(hops, 0);
   uint64_t lps = 0, slen = 0, wd = 1;
   for (uint32_t h = 0; h < hops; ++h) {
@@ -226,6 +256,7 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
     if (N && slen) SKY_HIP(hipMemsetAsync(sample_lengths, 0, (size_t)N * slen * 4, st));
     if (online) {
       SKY_TRY(ensure_table_storage(g));
+      if (dev_sized) SKY_TRY(ensure_class_census(g));  // once per graph
       SKY_TRY(prepare_build_scratch(g->V));
       SKY_TRY(pool_get(g, sky_graph::POOL_BITMAP, (size_t)words * 4, (void**)&bitmap));
       SKY_TRY(pool_get(g, sky_graph::POOL_LIST, (size_t)g->V * 4, (void**)&list));
@@ -249,12 +280,19 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
       if (online) {
         const uint64_t slots = (uint64_t)N * hg.width;
         SKY_HIP(hipMemsetAsync(d_count, 0, 4, st));
-        hipLaunchKernelGGL(frontier_collect_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, st, data,
-                           sample_lengths, slots, g->V, hg, bitmap, list, d_count);
-        uint32_t cnt = 0;
-        SKY_HIP(hipMemcpyAsync(&cnt, d_count, 4, hipMemcpyDeviceToHost, st));
-        SKY_HIP(hipStreamSynchronize(st));
-        SKY_TRY(build_rows(g, list, cnt, nullptr));
+        hipLaunchKernelGGL(frontier_collect_kernel, dim3((uint32_t)((slots + COLLECT_T - 1) / COLLECT_T)), dim3(COLLECT_T),
+                           0, st, data, sample_lengths, slots, g->V, hg, bitmap, list, d_count);
+        if (dev_sized) {
+          // the length of the list stays on the device: the kernels of the build find it there, and the host goes on
+          // to enqueue the hop without waiting (the reference's sampler never leaves the device either,
+          // src/online_sample_new.cu:191-270)
+          SKY_TRY(build_rows_dev(g, list, d_count, (uint32_t)std::min<uint64_t>(slots, g->V)));
+        } else {
+          uint32_t cnt = 0;
+          SKY_HIP(hipMemcpyAsync(&cnt, d_count, 4, hipMemcpyDeviceToHost, st));
+          SKY_HIP(hipStreamSynchronize(st));
+          SKY_TRY(build_rows(g, list, cnt, nullptr));
+        }
       }
       const uint64_t total = (uint64_t)N * hg.width * hg.k;
       if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");

@@ -14,15 +14,22 @@ def test_layout_closed_form():
     assert capi.sample_layout([1, 20, 20]) == (421, 21)
 
 
+@pytest.mark.parametrize("device_sized", [1, 0])
 @pytest.mark.parametrize("fanout", [[1, 25, 10], [1, 3, 2, 2], [1, 5]])
-def test_offline_and_online_match_oracle(orc, fanout):
+def test_offline_and_online_match_oracle(orc, fanout, device_sized):
+    # device_sized 1 (the default): the size of every frontier stays on the device and the host never waits inside
+    # the call; 0: the host reads it before it launches the build of the frontier's rows
     from skywalker_amd import capi
     xadj, adjncy = orc.rmat_csr(13, 8, 21)
     w = orc.gen_weights(orc.W_LOGNORMAL, 21, len(adjncy), 0.0, 1.0)
     seeds = orc.gen_seeds(4, 1 << 13, 1500)
     lps, slen = capi.sample_layout(fanout)
     g = capi.Graph.upload(xadj, adjncy, w)
-    d_on, sl_on, s_on, _ = g.sample_online(seeds, fanout, 17)
+    capi.set_option("online_device_sized", device_sized)
+    try:
+        d_on, sl_on, s_on, _ = g.sample_online(seeds, fanout, 17)
+    finally:
+        capi.set_option("online_device_sized", 1)
     on = (d_on.to_host((1500, lps)), sl_on.to_host((1500, slen)))
     g.build_tables()
     prob, alias, valid = g.tables()
@@ -144,3 +151,27 @@ def test_seeds_that_do_not_exist_have_no_children(orc):
     for got, s in ((on, s_on), (off, s_off)):
         assert np.array_equal(got[0], odata) and np.array_equal(got[1], osl) and s == osampled
     assert np.all(osl[seeds >= V] == 0)
+
+
+def test_online_sampling_builds_rows_of_every_class_without_waiting(orc):
+    # frontiers whose rows fall into every degree class up to the streaming kernel's, their sizes known to the
+    # device alone; a second call on the same graph finds the class census in place
+    from helpers import graph_from_degrees
+    from skywalker_amd import capi
+    rng = np.random.default_rng(77)
+    degs = [0, 1, 2, 3, 8, 9, 16, 17, 32, 33, 64, 65, 128, 129, 160, 161, 192, 193, 253, 254, 509, 510, 1021, 1022]
+    degs += [512 * nw - 3 for nw in range(3, 17)] + [8190, 9000, 25000, 70000, 300000]
+    degs += list(rng.integers(0, 300, 600))
+    rng.shuffle(degs)
+    xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal")
+    V = len(xadj) - 1
+    fanout = [1, 4, 3]
+    lps, slen = capi.sample_layout(fanout)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    for rep, n in enumerate((V, 50)):
+        seeds = np.arange(n, dtype=np.uint32) if rep == 0 else rng.integers(0, V, n).astype(np.uint32)
+        d_on, sl_on, s_on, _ = g.sample_online(seeds, fanout, 31 + rep)
+        odata, osl, osampled = orc.sample_online(xadj, adjncy, w, seeds, fanout, 31 + rep)
+        assert np.array_equal(d_on.to_host((n, lps)), odata) and np.array_equal(sl_on.to_host((n, slen)), osl)
+        assert s_on == osampled
+    g.free()

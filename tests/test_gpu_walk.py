@@ -90,10 +90,14 @@ def test_walk_does_not_depend_on_batch_composition(orc):
     assert np.array_equal(full[:1000], part)
 
 
-@pytest.mark.parametrize("mode", [0, 1, -1])
+@pytest.mark.parametrize("mode", [0, 1, -1, 2])
 def test_online_static_walk_equals_offline_and_oracle(orc, mode):
-    # mode 0: rows built step by step as walkers reach them; 1: every row first; -1: the library chooses
+    # mode 0: rows built step by step as walkers reach them; 1: every row first; -1: the library chooses;
+    # 2: step by step with the host waiting for the size of every step's row list (option online_device_sized 0)
     from skywalker_amd import capi
+    if mode == 2:
+        capi.set_option("online_device_sized", 0)
+        mode = 0
     xadj, adjncy = orc.rmat_csr(13, 8, 6)
     w = orc.gen_weights(orc.W_UNIFORM, 6, len(adjncy), 1.0, 100.0)
     seeds = orc.gen_seeds(3, 1 << 13, 2000)
@@ -103,6 +107,7 @@ def test_online_static_walk_equals_offline_and_oracle(orc, mode):
         p_on, l_on, s_on, _ = g.walk_online(capi.BIAS_STATIC, 1.0, 1.0, seeds, 30, 0.1, 5)
     finally:
         capi.set_option("online_full_build", -1)
+        capi.set_option("online_device_sized", 1)
     on = (p_on.to_host((2000, 31)), l_on.to_host())
     g.build_tables()
     p_off, l_off, s_off, _ = g.walk_offline(seeds, 30, 0.1, 5)
