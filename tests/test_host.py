@@ -338,3 +338,54 @@ def test_cli_degree_bias_plugin(tmp_path, orc):
             assert [int(x) for x in lines[i + 1].split()] == paths[j, :min(lengths[j], 13)].tolist()
     rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--input", p, "--biasplugin", "/nonexistent.so"])
     assert rc == 1 and "cannot load bias plug-in" in err
+
+
+def _walk_lines(out, lengths, paths, n, width):
+    lines = out.splitlines()
+    for j in range(n):
+        i = lines.index("%drd path len %d " % (j, lengths[j]))
+        assert [int(x) for x in lines[i + 1].split()] == paths[j, :min(lengths[j], width)].tolist()
+
+
+@pytest.mark.gpu
+def test_cli_degree_as_weight(tmp_path, orc):
+    # --dw: every edge of a row weighs the row's out-degree (include/graph.cuh:299-310), whatever the file holds
+    xadj, adjncy = orc.rmat_csr(11, 8, 31)
+    stored = (orc.gen_weights(orc.W_UNIFORM, 31, len(adjncy), 1.0, 100.0)).astype(np.uint32)
+    p = str(tmp_path / "rmat11.w.gr")
+    write_gr(p, xadj, adjncy, stored)
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--bias=1", "--ol=0", "--dw", "--input", p, "-n", "300",
+                        "--d", "16", "--printresult", "--seed", "6"])
+    assert rc == 0, err
+    w = np.repeat(np.diff(xadj).astype(np.float32), np.diff(xadj))
+    prob, alias, valid = orc.alias_build(xadj, w)
+    assert (prob[alias != 0xFFFFFFFF] == 1.0).all()  # equal weights inside a row: every slot keeps its bucket
+    paths, lengths, sampled = orc.walk_offline(xadj, adjncy, prob, alias, np.arange(300, dtype=np.uint32), 16, 0.0, 6)
+    _walk_lines(out, lengths, paths, 3, 17)
+    # and it is not the walk on the stored weights
+    sprob, salias, _ = orc.alias_build(xadj, stored.astype(np.float32))
+    spaths, _, _ = orc.walk_offline(xadj, adjncy, sprob, salias, np.arange(300, dtype=np.uint32), 16, 0.0, 6)
+    assert not np.array_equal(spaths, paths)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("weighted_file", [True, False])
+def test_cli_random_weights(tmp_path, orc, weighted_file):
+    # --randomweight --weightrange=R: weight i = float(rand()) / float(RAND_MAX / R) after srand(0)
+    # (include/graph.cuh:210-219), for a file with weights and for one without
+    import ctypes
+    xadj, adjncy = orc.rmat_csr(11, 8, 32)
+    p = str(tmp_path / "rmat11.gr")
+    write_gr(p, xadj, adjncy, np.ones(len(adjncy), np.uint32) if weighted_file else None)
+    R = 7
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--deepwalk", "--bias=1", "--ol=0", "--randomweight",
+                        "--weightrange=%d" % R, "--input", p, "-n", "300", "--d", "16", "--printresult", "--seed", "8"])
+    assert rc == 0, err
+    assert "generating random weight" in out
+    libc = ctypes.CDLL("libc.so.6")
+    libc.srand(0)
+    RAND_MAX = 2147483647
+    w = (np.array([libc.rand() for _ in range(len(adjncy))], np.float32) / np.float32(RAND_MAX // R)).astype(np.float32)
+    prob, alias, valid = orc.alias_build(xadj, w)
+    paths, lengths, sampled = orc.walk_offline(xadj, adjncy, prob, alias, np.arange(300, dtype=np.uint32), 16, 0.0, 8)
+    _walk_lines(out, lengths, paths, 3, 17)
