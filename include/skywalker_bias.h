@@ -85,6 +85,14 @@ int sky_bias_walk_online(sky_graph* g, float p, float q, const uint32_t* seeds_d
                          float stop_prob, uint64_t philox_seed, uint32_t* paths_device, uint32_t* lengths_device,
                          uint64_t* sampled, double* seconds);
 
+/* OnlineGBSampleNew under the operator (src/online_sample_new.cu:459-547; its constructors ask getBias for every
+ * weight of every frontier row, include/alias_table_new.cuh:1090-1091): hop by hop, the operator is evaluated for
+ * the rows of the distinct frontier vertices alone (walker state with has_last 0), their tables are built from those
+ * weights by libskywalker_hip, and the hop is drawn; arguments as sky_sample_online. */
+int sky_bias_sample_online(sky_graph* g, float p, float q, const uint32_t* seeds_device, uint32_t N,
+                           const uint32_t* fanout, uint32_t hops, uint64_t philox_seed, uint32_t* data_device,
+                           uint32_t* sample_lengths_device, uint64_t* sampled, double* seconds);
+
 #ifdef __cplusplus
 }
 #endif

@@ -186,6 +186,30 @@ int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, co
                       uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device, uint64_t* sampled,
                       double* seconds);
 
+/* ---- sky_sample_online taken apart hop by hop, for callers that compute the weights of the rows a hop builds
+ *      themselves: a bias operator (include/skywalker_bias.h).  The reference's online sampler builds every frontier
+ *      row through a constructor that asks gpu_graph::getBias for each weight
+ *      (include/alias_table_new.cuh:1090-1091, called from src/online_sample_new.cu:3-70); here the operator lives in
+ *      another library, so the sampler hands out the frontier and takes the weights back:
+ *        begin     outputs cleared, start vertices in place; the graph's tables count as not built
+ *        frontier  the distinct parents of `hop` (0 .. hops - 2) whose rows this session has not built: their vertex
+ *                  ids in *list_device, their number in the device word *count_device (the host is not told it),
+ *                  at most *upper of them
+ *        hop       builds those rows from weights_device (E floats in CSR slot order, of which only the slots of
+ *                  the listed rows are read; one allocation with 16 readable bytes after them; NULL: the graph's own
+ *                  weights), then draws the children of `hop`
+ *        end       sampled edges and kernel-region seconds; frees the session
+ *      Calls come in that order, frontier and hop once per hop, on one host thread.  Results are those of
+ *      sky_sample_online on a graph whose weights are the ones supplied. ---- */
+typedef struct sky_sample_session sky_sample_session;
+int sky_sample_session_begin(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                             uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device,
+                             sky_sample_session** out);
+int sky_sample_session_frontier(sky_sample_session* s, uint32_t hop, const uint32_t** list_device,
+                                const uint32_t** count_device, uint32_t* upper);
+int sky_sample_session_hop(sky_sample_session* s, uint32_t hop, const float* weights_device);
+int sky_sample_session_end(sky_sample_session* s, uint64_t* sampled, double* seconds);
+
 /* ---- self-test hook: runs Philox4x32-10 on the device for n (counter, key) pairs.
  *      ctr_host[4n], key_host[2n] -> out_host[4n]. ---- */
 int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint32_t n, uint32_t* out_host);

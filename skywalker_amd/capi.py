@@ -23,7 +23,8 @@ EXPORTS = [
     "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
     "sky_alias_build_all", "sky_alias_build_from_weights", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
     "sky_walk_offline_noalloc", "sky_walk_index_build",
-    "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_philox_selftest",
+    "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_sample_session_begin", "sky_sample_session_frontier", "sky_sample_session_hop",
+    "sky_sample_session_end", "sky_philox_selftest",
     "sky_last_build_profile", "sky_set_option",
 ]
 
@@ -304,6 +305,19 @@ class BiasPlugin:
                                                C.c_uint32(length), C.c_float(stop_prob), C.c_uint64(seed), paths.ptr,
                                                lengths.ptr, C.byref(sampled), C.byref(sec)))
         return paths, lengths, sampled.value, sec.value
+
+    def sample_online(self, g, p, q, seeds, fanout, seed):
+        seeds_d = seeds if isinstance(seeds, DeviceArray) else DeviceArray.from_host(np.asarray(seeds, np.uint32))
+        N = seeds_d.count
+        fan = np.asarray(fanout, np.uint32)
+        lps, slen = sample_layout(fan)
+        data = DeviceArray(N * lps, np.uint32, fill=FILL)
+        sl = DeviceArray(N * slen, np.uint32, fill=0)
+        sampled, sec = C.c_uint64(0), C.c_double(0)
+        self._ck(self.lib.sky_bias_sample_online(g.h, C.c_float(p), C.c_float(q), seeds_d.ptr, C.c_uint32(N), _p(fan),
+                                                 C.c_uint32(len(fan)), C.c_uint64(seed), data.ptr, sl.ptr,
+                                                 C.byref(sampled), C.byref(sec)))
+        return data, sl, sampled.value, sec.value
 
 
 def set_option(name, value):

@@ -6,6 +6,7 @@
 //                         build of libskywalker_hip runs on that array (ConstructTable, src/createTable.cu:119-179)
 //   sky_bias_walk_online  one workgroup per (walker, step) draws from the table of the current vertex under the
 //                         walker's state without building it (OnlineWalkShMem, src/online_walk.cu:97-132)
+#include <algorithm>
 #include <string>
 
 #include "../../include/skywalker_bias.h"
@@ -61,6 +62,24 @@ __global__ __launch_bounds__(256) void bias_weights_kernel(View g, float p, floa
   for (uint32_t k = 0; k < 64u; ++k) {  // the wavefront's 64 vertices in turn, its lanes side by side in the row
     const uint32_t v = wave * 64u + k;
     if (v >= g.V) break;
+    sky_row_view row{g.xadj, g.adjncy, g.adjwgt, g.V, v, g.xadj[v], g.xadj[v + 1] - g.xadj[v]};
+    for (uint32_t s = lane; s < row.deg; s += 64u) out[row.off + s] = sky_get_bias(&row, s, g.adjncy[row.off + s], &st);
+  }
+}
+
+// The operator's weights of the rows listed in list[0 .. *count): one wavefront per row at a time, its lanes side
+// by side in the row; the grid strides over the list, whose length only the device knows.
+__global__ __launch_bounds__(256) void bias_frontier_weights_kernel(View g, float p, float q,
+                                                                    const uint32_t* __restrict__ list,
+                                                                    const uint32_t* __restrict__ count,
+                                                                    float* __restrict__ out) {
+  sky_walker_state st{};
+  st.p = p;
+  st.q = q;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t n = *count, waves = gridDim.x * 4u;
+  for (uint32_t i = (blockIdx.x * 256u + threadIdx.x) >> 6; i < n; i += waves) {
+    const uint32_t v = list[i];
     sky_row_view row{g.xadj, g.adjncy, g.adjwgt, g.V, v, g.xadj[v], g.xadj[v + 1] - g.xadj[v]};
     for (uint32_t s = lane; s < row.deg; s += 64u) out[row.off + s] = sky_get_bias(&row, s, g.adjncy[row.off + s], &st);
   }
@@ -158,6 +177,42 @@ int sky_bias_build_all(sky_graph* g, float p, float q, double* seconds) {
   rc = body();
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
+  (void)sky_device_free(w);
+  return rc;
+}
+
+int sky_bias_sample_online(sky_graph* g, float p, float q, const uint32_t* seeds, uint32_t N, const uint32_t* fanout,
+                           uint32_t hops, uint64_t philox_seed, uint32_t* data, uint32_t* sample_lengths,
+                           uint64_t* sampled, double* seconds) {
+  if (!g) {
+    g_err = "sky_bias_sample_online: null graph";
+    return SKY_ERR_ARG;
+  }
+  View v{};
+  BIAS_TRY(view_of(g, &v));
+  float* w = nullptr;  // weights of the rows built so far, in their CSR slots; every other slot is never read
+  BIAS_TRY(sky_device_malloc((size_t)v.E * 4 + 16, (void**)&w));
+  sky_sample_session* s = nullptr;
+  auto body = [&]() -> int {
+    BIAS_TRY(sky_sample_session_begin(g, seeds, N, fanout, hops, philox_seed, data, sample_lengths, &s));
+    for (uint32_t h = 0; h + 1 < hops; ++h) {
+      const uint32_t *list = nullptr, *count = nullptr;
+      uint32_t upper = 0;
+      BIAS_TRY(sky_sample_session_frontier(s, h, &list, &count, &upper));
+      if (upper) {
+        const uint32_t blocks = std::min<uint32_t>((upper + 3) / 4, 8192u);
+        hipLaunchKernelGGL(bias_frontier_weights_kernel, dim3(blocks), dim3(256), 0, nullptr, v, p, q, list, count, w);
+        BIAS_HIP(hipGetLastError());
+      }
+      BIAS_TRY(sky_sample_session_hop(s, h, w));
+    }
+    return SKY_OK;
+  };
+  int rc = body();
+  if (s) {
+    const int rc_end = sky_sample_session_end(s, sampled, seconds);
+    if (rc == SKY_OK) rc = rc_end;
+  }
   (void)sky_device_free(w);
   return rc;
 }

@@ -206,6 +206,19 @@ int sky_alias_build_all(sky_graph* g, double* seconds) {
   return build_all_tables(g, seconds);
 }
 
+// Whether `bytes + 16` bytes are known to be readable from p on: the build kernels read whole 16-byte vectors.
+static bool padded_allocation(const void* p, size_t bytes) {
+  void* abase = nullptr;
+  size_t asize = 0;
+  if (hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t*>(&abase), &asize,
+                            reinterpret_cast<hipDeviceptr_t>(const_cast<void*>(p))) != hipSuccess || !abase) {
+    (void)hipGetLastError();
+    return false;
+  }
+  const size_t before = (size_t)(static_cast<const char*>(p) - static_cast<const char*>(abase));
+  return before <= asize && asize - before >= bytes + 16;
+}
+
 int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, double* seconds) {
   if (!g) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null graph");
   if (g->E && !weights_device) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null weights");
@@ -214,18 +227,7 @@ int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, doub
   // weights are copied into a padded array that stays with the graph.
   const float* use = weights_device;
   if (g->E) {
-    const size_t need = (size_t)g->E * 4 + 16;
-    void* abase = nullptr;
-    size_t asize = 0;
-    const hipError_t qe = hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t*>(&abase), &asize,
-                                                reinterpret_cast<hipDeviceptr_t>(const_cast<float*>(weights_device)));
-    bool padded = false;
-    if (qe == hipSuccess && abase) {
-      const size_t before = (size_t)(reinterpret_cast<const char*>(weights_device) - static_cast<const char*>(abase));
-      padded = before <= asize && asize - before >= need;
-    } else {
-      (void)hipGetLastError();  // a pointer the runtime does not know is not an error here: it is copied
-    }
+    const bool padded = padded_allocation(weights_device, (size_t)g->E * 4);
     if (!padded) {
       if (g->wgt_copy_cap < g->E) {
         if (g->wgt_copy) SKY_HIP(hipFree(g->wgt_copy));
@@ -381,6 +383,43 @@ static int sample_common(const char* who, bool online, sky_graph* g, const uint3
   SKY_TRY(sky_sample_layout(fanout, hops, &lps, &slen));
   if (!online && !g->has_tables) return fail(SKY_ERR_STATE, std::string(who) + ": alias tables have not been built");
   return sample_khop(g, online, seeds, N, fanout, hops, seed, data, sl, sampled, seconds);
+}
+
+struct sky_sample_session {
+  sky::SampleSession* s;
+  sky_graph* g;
+};
+
+int sky_sample_session_begin(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                             uint64_t philox_seed, uint32_t* data_device, uint32_t* sample_lengths_device,
+                             sky_sample_session** out) {
+  if (!g || !out) return fail(SKY_ERR_ARG, "sky_sample_session_begin: null pointer");
+  if (N && (!seeds_device || !data_device || !sample_lengths_device))
+    return fail(SKY_ERR_ARG, "sky_sample_session_begin: null pointer");
+  uint64_t lps = 0, slen = 0;
+  SKY_TRY(sky_sample_layout(fanout, hops, &lps, &slen));
+  g->has_tables = false;  // the rows are rebuilt from the caller's weights, hop by hop
+  sky::SampleSession* s = nullptr;
+  SKY_TRY(sample_session_begin(g, seeds_device, N, fanout, hops, philox_seed, data_device, sample_lengths_device, &s));
+  *out = new sky_sample_session{s, g};
+  return SKY_OK;
+}
+int sky_sample_session_frontier(sky_sample_session* s, uint32_t hop, const uint32_t** list_device,
+                                const uint32_t** count_device, uint32_t* upper) {
+  if (!s) return fail(SKY_ERR_ARG, "sky_sample_session_frontier: null session");
+  return sample_session_frontier(s->s, hop, list_device, count_device, upper);
+}
+int sky_sample_session_hop(sky_sample_session* s, uint32_t hop, const float* weights_device) {
+  if (!s) return fail(SKY_ERR_ARG, "sky_sample_session_hop: null session");
+  if (weights_device && s->g->E && !padded_allocation(weights_device, (size_t)s->g->E * 4))
+    return fail(SKY_ERR_ARG, "sky_sample_session_hop: the weight array needs E * 4 + 16 readable bytes in one allocation");
+  return sample_session_hop(s->s, hop, weights_device);
+}
+int sky_sample_session_end(sky_sample_session* s, uint64_t* sampled, double* seconds) {
+  if (!s) return fail(SKY_ERR_ARG, "sky_sample_session_end: null session");
+  const int rc = sample_session_end(s->s, sampled, seconds);
+  delete s;
+  return rc;
 }
 
 int sky_sample_offline(sky_graph* g, const uint32_t* seeds_device, uint32_t N, const uint32_t* fanout, uint32_t hops,

@@ -157,6 +157,12 @@ int walk_node2vec_reject(sky_graph* g, float p, float q, const uint32_t* seeds, 
                          double* seconds);
 int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
                 uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds);
+struct SampleSession;
+int sample_session_begin(sky_graph* g, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                         uint64_t seed, uint32_t* data, uint32_t* sample_lengths, SampleSession** out);
+int sample_session_frontier(SampleSession* s, uint32_t hop, const uint32_t** list, const uint32_t** count, uint32_t* upper);
+int sample_session_hop(SampleSession* s, uint32_t hop, const float* weights);
+int sample_session_end(SampleSession* s, uint64_t* sampled, double* seconds);
 int generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int weight_kind, float wa, float wb,
                   uint64_t weight_seed, sky_graph** out);
 int gen_seeds(uint64_t seed, uint32_t V, uint32_t N, uint32_t* seeds_device);

@@ -12,6 +12,9 @@
 //
 // Online mode builds the table of every distinct frontier vertex, once, through the same
 // kernels as the offline build (into the graph's table storage), then samples the hop.
+#include <algorithm>
+#include <vector>
+
 #include "sky_graph.h"
 
 namespace sky {
@@ -219,37 +222,79 @@ void set_sample_distinct(bool on) { g_sample_distinct = on; }
 bool g_online_device_sized = true;  // option "online_device_sized": 0 makes the online modes wait for every frontier size
 void set_online_device_sized(bool on) { g_online_device_sized = on; }
 
-int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
-                uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds) {
-  hipStream_t st = g->stream;
-  const bool distinct = g_sample_distinct;
-  if (distinct) {
-    if (hops > 256) return fail(SKY_ERR_LIMIT, "sample: distinct children need at most 256 hops");
-    for (uint32_t h = 1; h < hops; ++h)
-      if (fanout[h] > DISTINCT_MAX_K) return fail(SKY_ERR_LIMIT, "sample: distinct children need fanouts of at most 64");
-  }
-  if (g->has_tables) online = false;  // every row is already there: nothing to build on the way
-  // Rows longer than the streaming kernel takes need the tile-parallel path, whose launches the host sizes: a graph
-  // with such a row waits for the size of every frontier, any other graph never waits inside the call.
-  const bool dev_sized = online && build_rows_dev_possible(g) && g_online_device_sized;
-  std::vector<uint64_t> width(hops), off(hops), loff(hops, 0);
-  uint64_t lps = 0, slen = 0, wd = 1;
-  for (uint32_t h = 0; h < hops; ++h) {
-    wd *= fanout[h];
-    width[h] = wd;
-    off[h] = lps;
-    lps += wd;
-    if (h + 1 < hops) {
-      loff[h] = slen;
-      slen += wd;
-    }
-  }
-  if ((uint64_t)N * lps > (1ull << 40)) return fail(SKY_ERR_LIMIT, "sample: output too large");
-
+// One call of the k-hop sampler, taken apart hop by hop: begin (outputs cleared, start vertices in place), then for
+// every hop frontier (online: the distinct parents whose rows are not built yet), build (online: their rows) and
+// draw, then end (count, time).  sample_khop runs the steps in turn; sky_sample_session_* hands them to callers that
+// supply the weights of a frontier's rows themselves.
+struct SampleSession {
+  sky_graph* g = nullptr;
+  bool online = false, dev_sized = false, distinct = false;
+  const uint32_t* seeds = nullptr;
+  uint32_t N = 0, hops = 0;
+  uint64_t seed = 0;
+  uint32_t *data = nullptr, *sample_lengths = nullptr;
+  std::vector<uint32_t> fanout;
+  std::vector<uint64_t> width, off, loff;
+  uint64_t lps = 0, slen = 0;
   unsigned long long* d_sampled = nullptr;
   uint32_t *bitmap = nullptr, *list = nullptr, *d_count = nullptr;
-  const uint32_t words = (g->V + 31) / 32;
-  auto body = [&]() -> int {
+  uint32_t frontier_upper = 0;   // most rows the last frontier can hold
+  uint32_t frontier_count = 0;   // its size, when the host has read it (dev_sized false)
+  EventTimer tm;
+  explicit SampleSession(sky_graph* g_) : g(g_), tm(g_) {}
+
+  HopGeom geom(uint32_t h) const {
+    HopGeom hg;
+    hg.h = h;
+    hg.k = fanout[h + 1];
+    hg.fan_h = fanout[h];
+    hg.width = width[h];
+    hg.off = off[h];
+    hg.off_next = off[h + 1];
+    hg.loff = loff[h];
+    hg.loff_prev = h ? loff[h - 1] : 0;
+    hg.lps = lps;
+    hg.slen = slen;
+    return hg;
+  }
+
+  int begin(bool online_, const uint32_t* seeds_, uint32_t N_, const uint32_t* fanout_, uint32_t hops_, uint64_t seed_,
+            uint32_t* data_, uint32_t* sl_) {
+    hipStream_t st = g->stream;
+    online = online_;
+    seeds = seeds_;
+    N = N_;
+    hops = hops_;
+    seed = seed_;
+    data = data_;
+    sample_lengths = sl_;
+    distinct = g_sample_distinct;
+    fanout.assign(fanout_, fanout_ + hops);
+    if (distinct) {
+      if (hops > 256) return fail(SKY_ERR_LIMIT, "sample: distinct children need at most 256 hops");
+      for (uint32_t h = 1; h < hops; ++h)
+        if (fanout[h] > DISTINCT_MAX_K) return fail(SKY_ERR_LIMIT, "sample: distinct children need fanouts of at most 64");
+    }
+    if (g->has_tables) online = false;  // every row is already there: nothing to build on the way
+    // Without the option the host reads the size of every frontier and sizes the launches of its build exactly;
+    // with it (the default) nothing inside the call waits for the device.
+    dev_sized = online && build_rows_dev_possible(g) && g_online_device_sized;
+    width.assign(hops, 0);
+    off.assign(hops, 0);
+    loff.assign(hops, 0);
+    uint64_t wd = 1;
+    for (uint32_t h = 0; h < hops; ++h) {
+      wd *= fanout[h];
+      width[h] = wd;
+      off[h] = lps;
+      lps += wd;
+      if (h + 1 < hops) {
+        loff[h] = slen;
+        slen += wd;
+      }
+    }
+    if ((uint64_t)N * lps > (1ull << 40)) return fail(SKY_ERR_LIMIT, "sample: output too large");
+    const uint32_t words = (g->V + 31) / 32;
     SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
     d_count = reinterpret_cast<uint32_t*>(d_sampled + 1);
     SKY_HIP(hipMemsetAsync(d_sampled, 0, 8, st));
@@ -261,52 +306,63 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
       SKY_TRY(pool_get(g, sky_graph::POOL_BITMAP, (size_t)words * 4, (void**)&bitmap));
       SKY_TRY(pool_get(g, sky_graph::POOL_LIST, (size_t)g->V * 4, (void**)&list));
     }
-    EventTimer tm(g);
     SKY_TRY(tm.mark("start", 0));
     if (online) SKY_HIP(hipMemsetAsync(bitmap, 0, (size_t)words * 4, st));
     if (N) hipLaunchKernelGGL(sample_init_kernel, dim3((N + 255) / 256), dim3(256), 0, st, seeds, N, lps, data);
-    for (uint32_t h = 0; h + 1 < hops && N; ++h) {
-      HopGeom hg;
-      hg.h = h;
-      hg.k = fanout[h + 1];
-      hg.fan_h = fanout[h];
-      hg.width = width[h];
-      hg.off = off[h];
-      hg.off_next = off[h + 1];
-      hg.loff = loff[h];
-      hg.loff_prev = h ? loff[h - 1] : 0;
-      hg.lps = lps;
-      hg.slen = slen;
-      if (online) {
-        const uint64_t slots = (uint64_t)N * hg.width;
-        SKY_HIP(hipMemsetAsync(d_count, 0, 4, st));
-        hipLaunchKernelGGL(frontier_collect_kernel, dim3((uint32_t)((slots + COLLECT_T - 1) / COLLECT_T)), dim3(COLLECT_T),
-                           0, st, data, sample_lengths, slots, g->V, hg, bitmap, list, d_count);
-        if (dev_sized) {
-          // the length of the list stays on the device: the kernels of the build find it there, and the host goes on
-          // to enqueue the hop without waiting (the reference's sampler never leaves the device either,
-          // src/online_sample_new.cu:191-270)
-          SKY_TRY(build_rows_dev(g, list, d_count, (uint32_t)std::min<uint64_t>(slots, g->V)));
-        } else {
-          uint32_t cnt = 0;
-          SKY_HIP(hipMemcpyAsync(&cnt, d_count, 4, hipMemcpyDeviceToHost, st));
-          SKY_HIP(hipStreamSynchronize(st));
-          SKY_TRY(build_rows(g, list, cnt, nullptr));
-        }
-      }
-      const uint64_t total = (uint64_t)N * hg.width * hg.k;
-      if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");
-      if (distinct) {
-        const uint64_t slots = (uint64_t)N * hg.width;
-        hipLaunchKernelGGL(sample_hop_distinct_kernel, dim3((uint32_t)((slots + DISTINCT_T - 1) / DISTINCT_T)),
-                           dim3(DISTINCT_T), 0, st, g->xadj, g->adjncy, g->table, g->valid, slots, g->V, hg, seed, data,
-                           sample_lengths);
-        continue;
-      }
-      hipLaunchKernelGGL(sample_hop_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, g->xadj,
-                         g->adjncy, g->table, g->valid, total, g->V, hg, seed, total <= 0xFFFFFFFFull, data,
-                         sample_lengths);
+    return SKY_OK;
+  }
+
+  // Online: the distinct parents of hop h whose rows this call has not built yet, into `list`; their number stays in
+  // the device word d_count (and is read by the host only when the build needs it there).
+  int frontier(uint32_t h) {
+    frontier_upper = frontier_count = 0;
+    if (!online || !N) return SKY_OK;
+    hipStream_t st = g->stream;
+    const HopGeom hg = geom(h);
+    const uint64_t slots = (uint64_t)N * hg.width;
+    SKY_HIP(hipMemsetAsync(d_count, 0, 4, st));
+    hipLaunchKernelGGL(frontier_collect_kernel, dim3((uint32_t)((slots + COLLECT_T - 1) / COLLECT_T)), dim3(COLLECT_T), 0,
+                       st, data, sample_lengths, slots, g->V, hg, bitmap, list, d_count);
+    frontier_upper = (uint32_t)std::min<uint64_t>(slots, g->V);
+    if (!dev_sized) {
+      SKY_HIP(hipMemcpyAsync(&frontier_count, d_count, 4, hipMemcpyDeviceToHost, st));
+      SKY_HIP(hipStreamSynchronize(st));
     }
+    return SKY_OK;
+  }
+
+  // Online: the rows of the last frontier, from `weights` (null: the graph's own).  The length of the list stays
+  // on the device where it can: the kernels of the build find it there, and the host goes on to enqueue the hop
+  // without waiting (the reference's sampler never leaves the device either, src/online_sample_new.cu:191-270).
+  int build(const float* weights) {
+    if (!online || !N || !frontier_upper) return SKY_OK;
+    float* const own = g->adjwgt;
+    if (weights) g->adjwgt = const_cast<float*>(weights);  // the build only reads it
+    const int rc = dev_sized ? build_rows_dev(g, list, d_count, frontier_upper) : build_rows(g, list, frontier_count, nullptr);
+    g->adjwgt = own;
+    return rc;
+  }
+
+  int draw(uint32_t h) {
+    if (!N) return SKY_OK;
+    hipStream_t st = g->stream;
+    const HopGeom hg = geom(h);
+    const uint64_t total = (uint64_t)N * hg.width * hg.k;
+    if (total > 0xFFFFFFFFull * 256ull) return fail(SKY_ERR_LIMIT, "sample: hop too large for one launch");
+    if (distinct) {
+      const uint64_t slots = (uint64_t)N * hg.width;
+      hipLaunchKernelGGL(sample_hop_distinct_kernel, dim3((uint32_t)((slots + DISTINCT_T - 1) / DISTINCT_T)),
+                         dim3(DISTINCT_T), 0, st, g->xadj, g->adjncy, g->table, g->valid, slots, g->V, hg, seed, data,
+                         sample_lengths);
+      return SKY_OK;
+    }
+    hipLaunchKernelGGL(sample_hop_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st, g->xadj, g->adjncy,
+                       g->table, g->valid, total, g->V, hg, seed, total <= 0xFFFFFFFFull, data, sample_lengths);
+    return SKY_OK;
+  }
+
+  int end(uint64_t* sampled, double* seconds) {
+    hipStream_t st = g->stream;
     if (N && slen) {
       const uint64_t n = (uint64_t)N * slen;
       hipLaunchKernelGGL(sum_u32_kernel, dim3((uint32_t)std::min<uint64_t>((n + 255) / 256, 1024)), dim3(256), 0, st,
@@ -318,8 +374,52 @@ int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, co
     SKY_HIP(hipMemcpy(&hcount, d_sampled, 8, hipMemcpyDeviceToHost));
     if (sampled) *sampled = hcount;
     return SKY_OK;
-  };
-  return body();
+  }
+};
+
+int sample_khop(sky_graph* g, bool online, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                uint64_t seed, uint32_t* data, uint32_t* sample_lengths, uint64_t* sampled, double* seconds) {
+  SampleSession s(g);
+  SKY_TRY(s.begin(online, seeds, N, fanout, hops, seed, data, sample_lengths));
+  for (uint32_t h = 0; h + 1 < hops; ++h) {
+    SKY_TRY(s.frontier(h));
+    SKY_TRY(s.build(nullptr));
+    SKY_TRY(s.draw(h));
+  }
+  return s.end(sampled, seconds);
 }
+
+// The same steps behind the C interface (sky_sample_session_*).
+int sample_session_begin(sky_graph* g, const uint32_t* seeds, uint32_t N, const uint32_t* fanout, uint32_t hops,
+                         uint64_t seed, uint32_t* data, uint32_t* sample_lengths, SampleSession** out) {
+  SampleSession* s = new SampleSession(g);
+  const int rc = s->begin(true, seeds, N, fanout, hops, seed, data, sample_lengths);
+  if (rc != SKY_OK) {
+    delete s;
+    return rc;
+  }
+  *out = s;
+  return SKY_OK;
+}
+int sample_session_frontier(SampleSession* s, uint32_t hop, const uint32_t** list, const uint32_t** count,
+                            uint32_t* upper) {
+  if (hop + 1 >= s->hops) return fail(SKY_ERR_ARG, "sky_sample_session_frontier: no such hop");
+  SKY_TRY(s->frontier(hop));
+  if (list) *list = s->list;
+  if (count) *count = s->d_count;
+  if (upper) *upper = s->frontier_upper;
+  return SKY_OK;
+}
+int sample_session_hop(SampleSession* s, uint32_t hop, const float* weights) {
+  if (hop + 1 >= s->hops) return fail(SKY_ERR_ARG, "sky_sample_session_hop: no such hop");
+  SKY_TRY(s->build(weights));
+  return s->draw(hop);
+}
+int sample_session_end(SampleSession* s, uint64_t* sampled, double* seconds) {
+  const int rc = s->end(sampled, seconds);
+  delete s;
+  return rc;
+}
+bool sample_session_online(const SampleSession* s) { return s->online; }
 
 }  // namespace sky

@@ -34,6 +34,7 @@ struct BiasPluginLib {
   decltype(&sky_bias_last_error) last_error = nullptr;
   decltype(&sky_bias_build_all) build_all = nullptr;
   decltype(&sky_bias_walk_online) walk_online = nullptr;
+  decltype(&sky_bias_sample_online) sample_online = nullptr;
   bool Load(const std::string& path) {
     handle = dlopen(path.c_str(), RTLD_NOW | RTLD_GLOBAL);
     if (!handle) {
@@ -44,7 +45,8 @@ struct BiasPluginLib {
     last_error = (decltype(last_error))dlsym(handle, "sky_bias_last_error");
     build_all = (decltype(build_all))dlsym(handle, "sky_bias_build_all");
     walk_online = (decltype(walk_online))dlsym(handle, "sky_bias_walk_online");
-    if (!name || !last_error || !build_all || !walk_online) {
+    sample_online = (decltype(sample_online))dlsym(handle, "sky_bias_sample_online");
+    if (!name || !last_error || !build_all || !walk_online || !sample_online) {
       fprintf(stderr, "%s does not export the entry points of include/skywalker_bias.h\n", path.c_str());
       return false;
     }
@@ -356,7 +358,11 @@ inline float sample_common(Sampler_new& sampler, bool online, const char* who) {
   double sec = 0;
   uint64_t sampled = 0;
   const uint* seeds = (const uint*)sampler.result.seed_buf.ptr;
-  if (online) {
+  if (online && BiasPlugin().handle) {
+    SKY_PLUGIN_CALL(BiasPlugin().sample_online(sampler.ggraph.handle, (float)FLAGS_p, (float)FLAGS_q, seeds, sampler.num_seed,
+                                               sampler.result.hops_h.data(), sampler.result.hop_num, (uint64_t)FLAGS_seed,
+                                               sampler.result.data, sampler.result.sample_lengths, &sampled, &sec));
+  } else if (online) {
     SKY_RT_CALL(sky_sample_online(sampler.ggraph.handle, seeds, sampler.num_seed, sampler.result.hops_h.data(),
                                   sampler.result.hop_num, (uint64_t)FLAGS_seed, sampler.result.data,
                                   sampler.result.sample_lengths, &sampled, &sec));

@@ -29,7 +29,8 @@ def test_plugin_libraries_export_the_operator_entry_points():
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     host = text[text.index('extern "C"'):]
     names = sorted(set(re.findall(r"\b(sky_bias_[a-z0-9_]+)\s*\(", host)))
-    assert names == ["sky_bias_build_all", "sky_bias_last_error", "sky_bias_name", "sky_bias_walk_online"]
+    assert names == ["sky_bias_build_all", "sky_bias_last_error", "sky_bias_name", "sky_bias_sample_online",
+                     "sky_bias_walk_online"]
     for plug in build.PLUGINS:
         lib = ctypes.CDLL(build.plugin_path(plug))
         for n in names:

@@ -76,3 +76,47 @@ def test_static_plugin_is_the_edge_weight(orc):
     assert np.array_equal(paths.to_host((1000, 31)), opaths) and np.array_equal(lengths.to_host(), olengths)
     assert sampled == osampled
     g.free()
+
+
+@pytest.mark.parametrize("device_sized", [1, 0])
+def test_degree_plugin_online_sampling(orc, device_sized):
+    # the operator inside online k-hop sampling: hop by hop, evaluated for the distinct frontier rows alone, their
+    # tables built from those weights = the oracle's online sampler on the weights the operator stands for
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(13, 8, 47)
+    w = orc.gen_weights(orc.W_UNIFORM, 47, len(adjncy), 1.0, 100.0)  # ignored by the operator
+    wd = degree_weights(xadj, adjncy)
+    seeds = orc.gen_seeds(5, len(xadj) - 1, 1200)
+    fanout = [1, 6, 4]
+    lps, slen = capi.sample_layout(fanout)
+    plug = capi.BiasPlugin("degree")
+    g = capi.Graph.upload(xadj, adjncy, w)
+    capi.set_option("online_device_sized", device_sized)
+    try:
+        data, sl, sampled, _ = plug.sample_online(g, 1.0, 1.0, seeds, fanout, 13)
+    finally:
+        capi.set_option("online_device_sized", 1)
+    odata, osl, osampled = orc.sample_online(xadj, adjncy, wd, seeds, fanout, 13)
+    assert np.array_equal(sl.to_host((1200, slen)), osl) and np.array_equal(data.to_host((1200, lps)), odata)
+    assert sampled == osampled
+    # and it differs from sampling on the graph's own weights, which stay as they are
+    d2, _, _, _ = g.sample_online(seeds, fanout, 13)
+    assert not np.array_equal(d2.to_host((1200, lps)), odata)
+    assert np.array_equal(g.download()[2], w)
+    g.free()
+
+
+def test_static_plugin_online_sampling_equals_the_built_in(orc):
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 8, 48)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 48, len(adjncy), 0.0, 1.0)
+    seeds = orc.gen_seeds(6, len(xadj) - 1, 800)
+    fanout = [1, 5, 3]
+    lps, slen = capi.sample_layout(fanout)
+    plug = capi.BiasPlugin("static")
+    g = capi.Graph.upload(xadj, adjncy, w)
+    data, sl, sampled, _ = plug.sample_online(g, 1.0, 1.0, seeds, fanout, 14)
+    ref = g.sample_online(seeds, fanout, 14)
+    g.free()
+    assert np.array_equal(data.to_host(), ref[0].to_host()) and np.array_equal(sl.to_host(), ref[1].to_host())
+    assert sampled == ref[2]

@@ -389,3 +389,29 @@ def test_cli_random_weights(tmp_path, orc, weighted_file):
     prob, alias, valid = orc.alias_build(xadj, w)
     paths, lengths, sampled = orc.walk_offline(xadj, adjncy, prob, alias, np.arange(300, dtype=np.uint32), 16, 0.0, 8)
     _walk_lines(out, lengths, paths, 3, 17)
+
+
+@pytest.mark.gpu
+def test_cli_degree_bias_plugin_in_online_sampling(tmp_path, orc):
+    # --sage --ol=1 --biasplugin: the operator is asked for the weights of every frontier row the sampler builds
+    # (include/alias_table_new.cuh:1090-1091 via src/online_sample_new.cu:3-70)
+    xadj, adjncy = orc.rmat_csr(11, 8, 29)
+    p = str(tmp_path / "ds.gr")
+    write_gr(p, xadj, adjncy, np.ones(len(adjncy), np.uint32))
+    deg = np.diff(xadj.astype(np.int64))
+    wd = deg[adjncy].astype(np.float32)
+    plug = os.path.join(ROOT, "skywalker_amd", "libskywalker_bias_degree.so")
+    rc, out, err = run([os.path.join(HOST, "skywalker"), "--sage", "--bias=1", "--ol=1", "--input", p, "-n", "300",
+                        "--printresult", "--seed", "4", "--biasplugin", plug])
+    assert rc == 0, err
+    data, sl, sampled = orc.sample_online(xadj, adjncy, wd, np.arange(300, dtype=np.uint32), [1, 25, 10], 4)
+    blocks = out.split("th sample src: ")[1:]
+    assert len(blocks) == 4
+    for j, blk in enumerate(blocks):
+        m = re.match(r"(\d+), 1-hop len: (\d+)", blk)
+        assert int(m.group(1)) == j and int(m.group(2)) == sl[j, 0]
+        hop1 = [int(x) for x in blk.split("1-hop : ")[1].splitlines()[0].split()]
+        assert hop1 == data[j, 1:1 + sl[j, 0]].tolist()
+        for i in range(sl[j, 0]):
+            line = blk.split("\t %d th 2-hop [%d]: " % (i, data[j, 1 + i]))[1].splitlines()[0]
+            assert [int(x) for x in line.split()] == data[j, 26 + 10 * i:26 + 10 * i + min(sl[j, 1 + i], 30)].tolist()
