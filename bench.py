@@ -30,7 +30,33 @@ CONFIGS = {
     "c4": dict(scale=24, ef=16, wkind="uniform", wa=1.0, wb=100.0, seed=4, walkers=40000, length=80, ppr=False,
                mode="node2vec", p=2.0, q=0.5),
     "c5": dict(scale=26, ef=28, wkind="lognormal", wa=0.0, wb=2.0, seed=5, walkers=1000000, length=80, ppr=True),
+    # graphs the build was not tuned on (builder-run): another R-MAT shape of the same edge count, and a graph whose
+    # rows fill every degree class of the build with the same number of entries
+    "rmat25": dict(scale=25, ef=56, wkind="lognormal", wa=0.0, wb=2.0, seed=6, walkers=1000000, length=80, ppr=False),
+    "classes": dict(degrees="classes", per_class=50_000_000, wkind="lognormal", wa=0.0, wb=2.0, seed=7, walkers=1000000,
+                    length=80, ppr=False),
 }
+# degree ranges of the build's classes (skywalker_amd/csrc/sky_build.hip, degree_class)
+CLASS_RANGES = ([(1, 2), (3, 8), (9, 16), (17, 32), (33, 64), (65, 128), (129, 160), (161, 192), (193, 253), (254, 509)] +
+                [(512 * (nw - 1) - 2, 512 * nw - 3) for nw in range(2, 11)] +
+                [(5118, 24576), (24577, 65533), (65534, 524287), (524288, 1200000)])
+
+
+def class_degrees(per_class, seed):
+    """Row lengths that put about per_class entries into every degree class, in random order."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    parts = []
+    for lo, hi in CLASS_RANGES:
+        n = max(1, int(per_class / ((lo + hi) / 2)))
+        parts.append(rng.integers(lo, hi + 1, n, dtype=np.int64))
+    degs = np.concatenate(parts)
+    rng.shuffle(degs)
+    xadj = np.zeros(len(degs) + 1, np.uint32)
+    total = np.cumsum(degs)
+    assert total[-1] < 0xFFFFFFFF
+    xadj[1:] = total
+    return xadj
 # algorithmic bytes per edge of one launch: read w (4) and write prob + alias (8); the two tiled passes that only
 # read the weights count 4; xadj / valid are per vertex and small
 BYTES_PER_EDGE = {"tiled_sum": 4, "tiled_totals": 4}
@@ -47,7 +73,7 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
 KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
                   for g in (2, 4, 8, 16, 32) for x in ("", "x")})
 KERNEL_OF.update({"g32s": "build_group_kernel<32,5>"})
-KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,8>" % (64 * nw) for nw in range(2, 17)})
+KERNEL_OF.update({"mw%d" % nw: "build_merge_kernel<%d,8>" % (64 * nw) for nw in range(2, 11)})
 KERNEL_OF.update({"mw3": "build_merge_kernel<256,6>", "mw5": "build_merge_kernel<256,10>", "mw6": "build_merge_kernel<512,6>",
                   "mw7": "build_merge_kernel<256,14>", "mw9": "build_merge_kernel<768,6>", "mw10": "build_merge_kernel<512,10>"})
 
@@ -281,7 +307,13 @@ def main():
     wk = {"uniform": capi.W_UNIFORM, "unit": capi.W_UNIT, "lognormal": capi.W_LOGNORMAL}[cfg["wkind"]]
     name, cus = capi.device_name()
     t_gen = time.perf_counter()
-    g = capi.Graph.rmat(cfg["scale"], cfg["ef"], cfg["seed"], wk, cfg["wa"], cfg["wb"], cfg["seed"])
+    if cfg.get("degrees") == "classes":
+        g = capi.Graph.from_degrees(class_degrees(cfg["per_class"], cfg["seed"]), cfg["seed"], wk, cfg["wa"], cfg["wb"],
+                                    cfg["seed"])
+        shape = "rows of every degree class of the build, about %d entries per class, neighbours uniform" % cfg["per_class"]
+    else:
+        g = capi.Graph.rmat(cfg["scale"], cfg["ef"], cfg["seed"], wk, cfg["wa"], cfg["wb"], cfg["seed"])
+        shape = "R-MAT scale %d ef %d" % (cfg["scale"], cfg["ef"])
     t_gen = time.perf_counter() - t_gen
     V, E, N, L = g.V, g.E, cfg["walkers"], cfg["length"]
     seeds = g.gen_seeds(cfg["seed"], N)
@@ -375,9 +407,9 @@ def main():
         "value": work / (ms_per_step * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f64", "arithmetic": ARITHMETIC, "data": "synthetic",
-        "config": {"workload": "%s: R-MAT scale %d ef %d (%d V, %d E), %s weights; offline alias build of all vertices "
+        "config": {"workload": "%s: %s (%d V, %d E), %s weights; offline alias build of all vertices "
                                "+ biased DeepWalk L=%d from %d start vertices%s" %
-                               (args.config, cfg["scale"], cfg["ef"], V, E, cfg["wkind"], L, N,
+                               (args.config, shape, V, E, cfg["wkind"], L, N,
                                 " + PPR(0.15, max 100)" if cfg["ppr"] else ""),
                    "device": name, "compute_units": cus, "graph_generation_s": t_gen},
         "build": {"edges_per_s": E / build_s, "ms": build_s * 1e3, "algorithmic_bytes": build_bytes,

@@ -89,6 +89,13 @@ int sky_graph_upload(const uint32_t* xadj, const uint32_t* adjncy, const float* 
  * parameters (wa, wb) = (lo, hi) for UNIFORM, ignored for UNIT, (mu, sigma) for LOGNORMAL. */
 int sky_graph_generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int weight_kind, float wa,
                             float wb, uint64_t weight_seed, sky_graph** out);
+/* Synthetic graph with the row lengths the caller chooses: xadj[V+1] is a host array (row offsets), every neighbour id
+ * is drawn uniformly over [0, V) and every weight as in sky_graph_generate_rmat, both on the device, so that a graph of
+ * a billion edges needs no host arrays of that size.  No counterpart in the reference.  Rows are NOT sorted by
+ * neighbour id: fine for table builds, first-order walks and sampling, not for node2vec.  Made for measuring the
+ * build on degree distributions that an R-MAT generator does not produce. */
+int sky_graph_generate_from_degrees(const uint32_t* xadj, uint32_t V, uint64_t graph_seed, int weight_kind, float wa,
+                                    float wb, uint64_t weight_seed, sky_graph** out);
 int sky_graph_info(const sky_graph* g, uint32_t* V, uint32_t* E, uint32_t* max_degree);
 /* Copies to host; any destination may be NULL. */
 int sky_graph_download(const sky_graph* g, uint32_t* xadj, uint32_t* adjncy, float* adjwgt);
@@ -217,14 +224,14 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
 /* ---- tuning knobs (no counterpart in the reference).  "tiled_max_tiles": rows too long for one workgroup are
  *      built tile by tile (1024 entries per tile) up to this many tiles (default: no limit); longer rows
  *      fall to a kernel in which one workgroup walks the whole row.  Tests lower it to exercise that kernel.
- *      "row_merge" (default 1): rows of 62..8189 entries pair lights and heavies by a merge of their prefix
+ *      "row_merge" (default 1): rows of 62..5117 entries pair lights and heavies by a merge of their prefix
  *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table.
- *      "stream_min_edges" (default 4000000): rows of 8190..524287 entries have a kernel of their own (one workgroup
+ *      "stream_min_edges" (default 4000000): rows of 5118..524287 entries have a kernel of their own (one workgroup
  *      streams a row); when a build holds no more than this many entries in such rows, too few to fill the GPU
  *      with one workgroup each, they go to the tile-parallel path instead.  Tests set 0.
  *      "stream_wide_min_edges" (default 134217216): the rows of more than 65533 entries among them keep a workgroup
  *      busy for up to 1.5 ms; they join that kernel only when the build holds at least this many entries in rows
- *      of 8190..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
+ *      of 5118..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
  *      "walk_read_once" (default -1): 1 makes the walks load a step's table entry and neighbour id as read-once
  *      data, which keeps the row offsets of the well-connected vertices in L2 on a graph whose tables are far larger
  *      than the caches; 0 loads them as ordinary data (better when the tables fit the caches); -1 decides by the size of

@@ -20,7 +20,7 @@ W_UNIFORM, W_UNIT, W_LOGNORMAL = 0, 1, 2
 EXPORTS = [
     "sky_last_error", "sky_version", "sky_device_malloc", "sky_device_free", "sky_memcpy_h2d", "sky_memcpy_d2h",
     "sky_device_fill_u32", "sky_device_copy_u32", "sky_device_synchronize", "sky_device_mem_info", "sky_device_name", "sky_graph_upload",
-    "sky_graph_generate_rmat", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
+    "sky_graph_generate_rmat", "sky_graph_generate_from_degrees", "sky_graph_info", "sky_graph_download", "sky_graph_device_ptrs", "sky_graph_free",
     "sky_alias_build_all", "sky_alias_build_from_weights", "sky_alias_download", "sky_alias_upload", "sky_gen_seeds", "sky_walk_offline",
     "sky_walk_offline_noalloc", "sky_walk_index_build",
     "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_sample_session_begin", "sky_sample_session_frontier", "sky_sample_session_hop",
@@ -153,6 +153,16 @@ class Graph:
         _ck(lib().sky_graph_generate_rmat(C.c_uint32(scale), C.c_uint32(edge_factor), C.c_uint64(graph_seed),
                                           C.c_int(weight_kind), C.c_float(wa), C.c_float(wb),
                                           C.c_uint64(weight_seed), C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def from_degrees(cls, xadj, graph_seed, weight_kind, wa, wb, weight_seed):
+        """Rows of the given lengths, neighbours uniform over the vertices, weights of the given law (device side)."""
+        xadj = np.ascontiguousarray(xadj, np.uint32)
+        h = C.c_void_p()
+        _ck(lib().sky_graph_generate_from_degrees(_p(xadj), C.c_uint32(len(xadj) - 1), C.c_uint64(graph_seed),
+                                                  C.c_int(weight_kind), C.c_float(wa), C.c_float(wb),
+                                                  C.c_uint64(weight_seed), C.byref(h)))
         return cls(h)
 
     def download(self, weights=True):

@@ -47,7 +47,10 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
-  if (nw <= 16) return CLS_MW2 + (int)nw - 2;
+  // Longer rows stream through one workgroup: the arrays of a row of more than 5117 entries leave room for one
+  // workgroup per CU only (14 bytes of LDS per slot), and wavefronts that all wait at the same barriers ran such
+  // rows at 1.6 TB/s where the streaming kernel reaches 2.5.
+  if (nw <= MERGE_MAX_NW) return CLS_MW2 + (int)nw - 2;
   if (d > STREAM_MAX_DEG) return CLS_HUGE;
   if (d > 65533u) return CLS_STREAM_WIDE;
   return d > 24576u ? CLS_STREAM : CLS_STREAM_LAST;
@@ -1347,16 +1350,10 @@ int prepare_build_scratch(uint32_t max_rows) {
   if (!sc.blk_cnt) SKY_HIP(hipMalloc((void**)&sc.blk_cnt, (size_t)BIN_BLOCKS * CLS_COUNT * 4));
   if (!sc.lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
-#define SKY_BIG(NW) SKY_TRY(enable_big_lds(build_merge_kernel<64 * NW, 8>, (64 * NW * 8 + 2) * 14))
     SKY_TRY(enable_big_lds(build_merge_kernel<512, 10>, (512 * 10 + 2) * 14));
     SKY_TRY(enable_big_lds(build_merge_kernel<768, 6>, (768 * 6 + 2) * 14));
-    SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
-#undef SKY_BIG
-#define SKY_BIG(NW) SKY_TRY(enable_big_lds((build_merge_kernel<64 * NW, 8, 4, 1>), (64 * NW * 8 + 2) * 14))
     SKY_TRY(enable_big_lds((build_merge_kernel<512, 10, 4, 1>), (512 * 10 + 2) * 14));
     SKY_TRY(enable_big_lds((build_merge_kernel<768, 6, 4, 1>), (768 * 6 + 2) * 14));
-    SKY_BIG(11); SKY_BIG(12); SKY_BIG(13); SKY_BIG(14); SKY_BIG(15); SKY_BIG(16);
-#undef SKY_BIG
     sc.lds_enabled = true;
   }
   return SKY_OK;
@@ -1478,8 +1475,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
-  static const char* const mw_name[15] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9",
-                                          "mw10", "mw11", "mw12", "mw13", "mw14", "mw15", "mw16"};
+  static const char* const mw_name[9] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9", "mw10"};
   if (g_row_merge) {
     SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 4>, 64, 4, "lds_w1"));
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 8>, 64, 8, "lds_w2"));
@@ -1498,17 +1494,16 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     SKY_MW(8);
     SKY_TRY(mrg(CLS_MW2 + 7, build_merge_kernel<768, 6>, 768, 6, mw_name[7]));
     SKY_TRY(mrg(CLS_MW2 + 8, build_merge_kernel<512, 10>, 512, 10, mw_name[8]));
-    SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
 #undef SKY_MW
   } else {
     SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
     SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
-    for (int nw = 2; nw <= 16; ++nw) {
+    for (int nw = 2; nw <= MERGE_MAX_NW; ++nw) {
       const int cls = CLS_MW2 + nw - 2;
       if (nw <= 2) SKY_TRY(lds(cls, build_lds_kernel<128, 2>, 128, 2, mw_name[nw - 2]));
       else if (nw <= 4) SKY_TRY(lds(cls, build_lds_kernel<256, 2>, 256, 2, mw_name[nw - 2]));
       else if (nw <= 8) SKY_TRY(lds(cls, build_lds_kernel<512, 2>, 512, 2, mw_name[nw - 2]));
-      else {  // this variant has no kernel for rows of 4094..8189 entries: tile-parallel path
+      else {  // this variant has no kernel for rows of 4094..5117 entries: tile-parallel path
         if (counts[cls]) {
           uint32_t skipped = 0;
           SKY_TRY(fan.join());  // the tile-parallel path's scratch serves one call at a time
@@ -1520,7 +1515,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
   }
 
-  // Rows of 8190..STREAM_MAX_DEG entries: one workgroup streams a row.  A small streaming class is not worth its
+  // Rows of 5118..STREAM_MAX_DEG entries: one workgroup streams a row.  A small streaming class is not worth its
   // own launch (too few workgroups to fill the GPU): its rows then go to the tile-parallel path together with the
   // HUGE class.  The rows above 65533 entries keep one workgroup busy for up to 1.5 ms; they join the launch (and
   // start first) only when it holds enough other rows to run that long anyway, else they are built tile by tile.
@@ -1648,7 +1643,7 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   // the class kernels are independent of one another: they go out in turn over the graph's stream and its side streams
   StreamFan fan(g, st);
   if (g_build_streams && n_upper >= 4096) SKY_TRY(fan.start());
-  // Rows of 8190 entries and more first, because theirs is the longest chain of launches.  The classes STREAM,
+  // Rows of 5118 entries and more first, because theirs is the longest chain of launches.  The classes STREAM,
   // STREAM_LAST, STREAM_WIDE, HUGE lie back to back.  What the graph holds of them decides, as in a build of all
   // rows, which go to the streaming kernel (one workgroup per row) and which are built tile by tile by the whole
   // GPU: the two longest classes always are (a frontier holds a few such rows at most, and one workgroup would need
@@ -1714,7 +1709,6 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   SKY_MW(8);
   SKY_Q(CLS_MW2 + 7, mrg(CLS_MW2 + 7, (build_merge_kernel<768, 6, 4, 1>), 768, 6));
   SKY_Q(CLS_MW2 + 8, mrg(CLS_MW2 + 8, (build_merge_kernel<512, 10, 4, 1>), 512, 10));
-  SKY_MW(11); SKY_MW(12); SKY_MW(13); SKY_MW(14); SKY_MW(15); SKY_MW(16);
 #undef SKY_MW
 #undef SKY_Q
   std::stable_sort(queue.begin(), queue.end(), [](const auto& a, const auto& b) { return a.first > b.first; });

@@ -1,4 +1,4 @@
-// Alias tables of rows of 8190..524287 entries: one workgroup streams the row and keeps a window of
+// Alias tables of rows of 5118..524287 entries: one workgroup streams the row and keeps a window of
 // the row's heavies in LDS.
 //
 // The table is the same pure function of the weights as everywhere else (see sky_build.hip).
@@ -560,7 +560,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   }  // rows of this workgroup
 }
 
-// Builds the n_first rows of `first_list` and the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each) in one
+// Builds the n_first rows of `first_list` and the n rows of `rows_list` (5118..STREAM_MAX_DEG entries each) in one
 // launch that starts with the former.
 int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n) {
   if (n + n_first == 0) return SKY_OK;

@@ -162,6 +162,12 @@ int sky_graph_generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph
   return generate_rmat(scale, edge_factor, graph_seed, weight_kind, wa, wb, weight_seed, out);
 }
 
+int sky_graph_generate_from_degrees(const uint32_t* xadj, uint32_t V, uint64_t graph_seed, int weight_kind, float wa,
+                                    float wb, uint64_t weight_seed, sky_graph** out) {
+  SKY_TRY(ensure_device());
+  return generate_from_degrees(xadj, V, graph_seed, weight_kind, wa, wb, weight_seed, out);
+}
+
 int sky_graph_info(const sky_graph* g, uint32_t* V, uint32_t* E, uint32_t* max_degree) {
   if (!g) return fail(SKY_ERR_ARG, "sky_graph_info: null graph");
   if (V) *V = g->V;

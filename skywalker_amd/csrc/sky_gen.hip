@@ -168,6 +168,53 @@ int generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int
   return SKY_OK;
 }
 
+// Neighbour ids uniform over [0, V), one Philox counter per slot (domain of the R-MAT generator, third counter
+// word 1 so that no counter is shared with it).  Rows come out unsorted.
+__global__ __launch_bounds__(256) void random_adjncy_kernel(uint64_t seed, uint32_t V, uint64_t E,
+                                                            uint32_t* __restrict__ adjncy) {
+  const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+  if (i >= E) return;
+  adjncy[i] = __umulhi(philox(seed, (uint32_t)i, (uint32_t)(i >> 32), 1, DOM_RMAT).x, V);
+}
+
+int generate_from_degrees(const uint32_t* xadj_host, uint32_t V, uint64_t graph_seed, int weight_kind, float wa, float wb,
+                          uint64_t weight_seed, sky_graph** out) {
+  if (!out || !xadj_host) return fail(SKY_ERR_ARG, "generate_from_degrees: null pointer");
+  if (weight_kind < SKY_W_UNIFORM || weight_kind > SKY_W_LOGNORMAL)
+    return fail(SKY_ERR_ARG, "generate_from_degrees: unknown weight kind");
+  if (xadj_host[0] != 0) return fail(SKY_ERR_ARG, "generate_from_degrees: xadj[0] != 0");
+  for (uint32_t v = 0; v < V; ++v)
+    if (xadj_host[v] > xadj_host[v + 1]) return fail(SKY_ERR_ARG, "generate_from_degrees: xadj is not monotone");
+  const uint64_t E = xadj_host[V];
+  if (E && V == 0) return fail(SKY_ERR_ARG, "generate_from_degrees: edges without vertices");
+  sky_graph* g = new sky_graph();
+  (void)hipGetDevice(&g->device);
+  g->V = V;
+  g->E = (uint32_t)E;
+  hipStream_t st = g->stream;
+  auto body = [&]() -> int {
+    SKY_TRY(alloc_padded(&g->xadj, (size_t)V + 1));
+    SKY_TRY(alloc_padded(&g->adjncy, (size_t)E));
+    SKY_TRY(alloc_padded(&g->adjwgt, (size_t)E));
+    SKY_HIP(hipMemcpy(g->xadj, xadj_host, ((size_t)V + 1) * 4, hipMemcpyHostToDevice));
+    if (E) {
+      const uint32_t eblocks = (uint32_t)((E + 255) / 256);
+      hipLaunchKernelGGL(random_adjncy_kernel, dim3(eblocks), dim3(256), 0, st, graph_seed, V, E, g->adjncy);
+      hipLaunchKernelGGL(weights_kernel, dim3(eblocks), dim3(256), 0, st, weight_kind, weight_seed, E, wa, wb, g->adjwgt);
+    }
+    SKY_HIP(hipStreamSynchronize(st));
+    SKY_HIP(hipGetLastError());
+    return compute_max_degree(g);
+  };
+  const int rc = body();
+  if (rc != SKY_OK) {
+    sky_graph_free(g);
+    return rc;
+  }
+  *out = g;
+  return SKY_OK;
+}
+
 int gen_seeds(uint64_t seed, uint32_t V, uint32_t N, uint32_t* seeds_device) {
   if (N) hipLaunchKernelGGL(seeds_kernel, dim3((N + 255) / 256), dim3(256), 0, nullptr, seed, V, N, seeds_device);
   SKY_HIP(hipStreamSynchronize(nullptr));

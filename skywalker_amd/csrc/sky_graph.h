@@ -74,10 +74,10 @@ enum BuildClass : int {
   CLS_G32X = 7,     // deg 161..192     32 lanes, 6 slots per lane
   CLS_LDS_W1 = 8,   // deg <= 253       one wavefront per row, 4 slots per lane
   CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
-  CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..16 (class CLS_MW2 + nw - 2): one workgroup per row whose
-  CLS_MW16 = 24,    //                  threads cover 512 * nw slots
+  CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..10 (class CLS_MW2 + nw - 2, up to 18): one workgroup per row whose
+                    //                  threads cover 512 * nw slots (the numbers 19..24 are not used)
   CLS_STREAM = 25,       // deg 24577..65533   one workgroup streams the row, a window of its heavies stays in LDS.
-  CLS_STREAM_LAST = 26,  // deg 8190..24576    Three classes built by one launch that takes the longest rows first
+  CLS_STREAM_LAST = 26,  // deg 5118..24576    Three classes built by one launch that takes the longest rows first
   CLS_STREAM_WIDE = 27,  // deg 65534..524287  and so
                     //                  does not end on its longest rows
   CLS_HUGE = 28,    // above            built tile by tile by the whole GPU
@@ -122,6 +122,7 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
 int build_rows_tiled_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int cls, int ncls, uint32_t n_upper,
                          uint64_t edges_upper);
 void set_tiled_max_tiles(uint32_t n);
+constexpr int MERGE_MAX_NW = 10;  // rows of at most 512 * 10 - 3 = 5117 entries pair by merge in LDS
 constexpr uint32_t STREAM_MAX_DEG = 524287;  // longest row of the streaming classes (one workgroup takes 1.5 ms for it)
 int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n);
 int build_rows_stream_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int ncls, uint32_t grid);
@@ -165,6 +166,8 @@ int sample_session_hop(SampleSession* s, uint32_t hop, const float* weights);
 int sample_session_end(SampleSession* s, uint64_t* sampled, double* seconds);
 int generate_rmat(uint32_t scale, uint32_t edge_factor, uint64_t graph_seed, int weight_kind, float wa, float wb,
                   uint64_t weight_seed, sky_graph** out);
+int generate_from_degrees(const uint32_t* xadj_host, uint32_t V, uint64_t graph_seed, int weight_kind, float wa, float wb,
+                          uint64_t weight_seed, sky_graph** out);
 int gen_seeds(uint64_t seed, uint32_t V, uint32_t N, uint32_t* seeds_device);
 int philox_selftest(const uint32_t* ctr, const uint32_t* key, uint32_t n, uint32_t* out);
 int compute_max_degree(sky_graph* g);

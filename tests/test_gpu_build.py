@@ -11,7 +11,7 @@ TOL = 1e-6
 # degrees that straddle every dispatch class boundary of the build
 EDGE_DEGREES = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 16, 17, 22, 23, 24, 25, 28, 29, 30, 32, 33, 46, 47, 48,
                 49, 60, 61, 62, 63, 64, 65, 66, 67, 68, 94, 95, 96, 97, 124, 125, 126, 127, 190, 191, 192, 193, 253, 254, 255, 256, 257, 1021,
-                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 8189, 8190, 8191, 8192, 8193, 20000, 70001, 128, 129, 130, 144, 145, 159, 160, 161, 162, 34, 35, 36, 45]
+                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 5116, 5117, 5118, 5119, 5120, 5121, 8189, 8190, 8191, 8192, 8193, 20000, 70001, 128, 129, 130, 144, 145, 159, 160, 161, 162, 34, 35, 36, 45]
 
 
 def build_and_compare(orc, xadj, adjncy, w, label):
@@ -19,9 +19,9 @@ def build_and_compare(orc, xadj, adjncy, w, label):
     print("case", label, "V", len(xadj) - 1, "E", len(w), flush=True)
     oprob, oalias, ovalid = orc.alias_build(xadj, w)
     deg = np.diff(xadj)
-    # rows of 8190..524287 entries: once through their own kernel, once (the default for so few of them)
+    # rows of 5118..524287 entries: once through their own kernel, once (the default for so few of them)
     # through the tile-parallel path
-    routes = (0, 4000000) if ((deg >= 8190) & (deg <= 524287)).any() else (4000000,)
+    routes = (0, 4000000) if ((deg >= 5118) & (deg <= 524287)).any() else (4000000,)
     # rows of at most 32 entries: by degree class (the default below 2^25 rows), and by the kernel that walks the
     # vertices in order
     for stream_min_edges, small_in_place in [(r, 0) for r in routes] + [(routes[0], 1)]:
@@ -80,7 +80,7 @@ def test_unaligned_row_starts(orc):
     # rows of every residue mod 4 in front of each LDS-class row
     rng = np.random.default_rng(5)
     degs = []
-    for d in (70, 254, 700, 1021, 3000, 4093, 8000, 8189, 9000):
+    for d in (70, 254, 700, 1021, 3000, 4093, 5117, 5118, 8000, 8189, 9000):
         for pad in (1, 2, 3, 5):
             degs += [pad, d]
     xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal")
@@ -197,7 +197,7 @@ def test_streaming_kernel_for_rows_with_too_many_tiles(orc):
 
 def test_search_variant_of_the_row_kernels_gives_the_same_table(orc):
     # "row_merge" = 0 selects the kernels that do one binary search per entry (rows of 62..4093 entries) and
-    # sends rows of 4094..8189 entries down the tile-parallel path
+    # sends rows of 4094..5117 entries down the tile-parallel path (longer ones stream or go tile by tile anyway)
     from skywalker_amd import capi
     rng = np.random.default_rng(23)
     degs = [70, 126, 254, 300, 509, 510, 1021, 1500, 2046, 3000, 4093, 4094, 5000, 8189, 8190, 3, 0, 1]
@@ -212,11 +212,11 @@ def test_search_variant_of_the_row_kernels_gives_the_same_table(orc):
 
 @pytest.mark.parametrize("dist", ["lognormal2", "uniform", "nearequal", "sparse", "fewlights", "fewheavies"])
 def test_rows_streamed_by_one_workgroup(orc, dist):
-    # rows of 8190..524287 entries: a window of 5085 heavies kept in LDS ("fewlights" and "uniform" have rows with
+    # rows of 5118..524287 entries: a window of 5080 heavies kept in LDS ("fewlights" and "uniform" have rows with
     # many windows, "nearequal" rows without a heavy); 524288 is the first degree of the tile-parallel class
     from helpers import weights
     rng = np.random.default_rng(31)
-    degs = [8190, 8191, 7, 8193, 12288, 2, 12289, 16385, 1, 30000, 65533, 65534, 0, 9001, 150001, 524287, 524288]
+    degs = [5118, 5119, 6000, 8190, 8191, 7, 8193, 12288, 2, 12289, 16385, 1, 30000, 65533, 65534, 0, 9001, 150001, 524287, 524288]
     xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=4096)
     if dist == "fewlights":
         w = np.where(rng.random(len(w)) < 0.01, 0.01, 1.01).astype(np.float32)
@@ -310,8 +310,8 @@ def test_random_mixtures_of_every_class(orc, seed):
     from helpers import weights
     rng = np.random.default_rng(1000 + seed)
     ends = [0, 1, 2, 3, 5, 6, 8, 9, 13, 14, 16, 17, 29, 30, 32, 33, 61, 62, 64, 65, 125, 126, 128, 129, 191, 192, 193, 253, 254,
-            509, 8190, 24576, 24577, 65533, 65534]
-    for nw in range(2, 17):
+            509, 5117, 5118, 8190, 24576, 24577, 65533, 65534]
+    for nw in range(2, 11):
         ends += [512 * (nw - 1) - 2, 512 * nw - 3]
     degs = ends + list(rng.integers(0, 70, 3000)) + list(rng.integers(60, 600, 600)) + \
         list(rng.integers(500, 8300, 260)) + list(rng.integers(8000, 66000, 12)) + list(rng.integers(66000, 400000, 2))

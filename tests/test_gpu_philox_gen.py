@@ -69,3 +69,27 @@ def test_seeds(orc):
     g.free()
     assert np.array_equal(s, orc.gen_seeds(99, 1 << 10, 5000))
     assert s.max() < (1 << 10)
+
+
+def test_graph_from_degrees(orc):
+    # rows of chosen lengths, neighbours and weights drawn on the device: the build of such a graph = the oracle's on
+    # the arrays it downloads, and the generator repeats itself for the same seeds
+    from skywalker_amd import capi
+    rng = np.random.default_rng(3)
+    degs = np.concatenate([rng.integers(0, 40, 3000), rng.integers(100, 3000, 60), [9000, 70000]])
+    rng.shuffle(degs)
+    xadj = np.zeros(len(degs) + 1, np.uint32)
+    xadj[1:] = np.cumsum(degs)
+    g = capi.Graph.from_degrees(xadj, 11, capi.W_LOGNORMAL, 0.0, 2.0, 12)
+    assert g.V == len(degs) and g.E == int(xadj[-1]) and g.max_degree == 70000
+    hx, hadj, hw = g.download()
+    assert np.array_equal(hx, xadj) and hadj.max() < g.V and len(np.unique(hadj)) > g.V // 2
+    assert np.allclose(hw, orc.gen_weights(orc.W_LOGNORMAL, 12, g.E, 0.0, 2.0), rtol=1e-4)  # device expf, logf, cosf
+    g.build_tables()
+    prob, alias, valid = g.tables()
+    oprob, oalias, ovalid = orc.alias_build(hx, hw)
+    assert np.array_equal(prob, oprob) and np.array_equal(alias, oalias) and np.array_equal(valid, ovalid)
+    g2 = capi.Graph.from_degrees(xadj, 11, capi.W_LOGNORMAL, 0.0, 2.0, 12)
+    assert np.array_equal(g2.download()[1], hadj)
+    g.free()
+    g2.free()
