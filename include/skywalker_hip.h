@@ -12,9 +12,8 @@
  *     the last failure on the calling thread is available from sky_last_error().
  *   - a sky_graph owns the device-resident CSR and, after sky_alias_build_all, the
  *     alias tables.  One host thread per sky_graph; calls are synchronous.  The scratch memory of the table
- *     build and the options of sky_set_option belong to the process, not to a graph: calls that build tables
- *     (sky_alias_build_all, sky_walk_online, sky_sample_online) must not overlap, whatever graphs they are for,
- *     like the reference's entry functions, which share the default stream.
+ *     builds belongs to the graph (allocated on first use, freed with it), and so can the tuning knobs
+ *     (sky_graph_set_option).  Every graph works on the null stream, like the reference's entry functions.
  *   - "device pointer" arguments are HIP device addresses on the current device
  *     (from sky_device_malloc, or any other allocator of the same process).
  *   - `seconds` outputs report the kernel region only (launch to completion,
@@ -264,6 +263,11 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      include/sampler_result.cuh:646-669), so that walkers that have stopped no longer hold a lane; 0 keeps every
  *      walker on its lane for the whole walk in one launch.  The paths are the same. ---- */
 int sky_set_option(const char* name, long value);
+/* The same knobs for one graph: sky_graph_set_option gives the graph a value of its own, which the calls on that graph
+ * use instead of the process-wide one that sky_set_option sets; sky_graph_unset_option returns the graph to the
+ * process-wide value.  Two graphs of one process can so be built and walked under different settings. */
+int sky_graph_set_option(sky_graph* g, const char* name, long value);
+int sky_graph_unset_option(sky_graph* g, const char* name);
 
 /* ---- per-kernel timing of the last sky_alias_build_all on this graph, for roofline reporting:
  *      names[i] is a static string, ms[i] its HIP-event duration.  Returns the number of entries: one

@@ -25,7 +25,7 @@ EXPORTS = [
     "sky_walk_offline_noalloc", "sky_walk_index_build",
     "sky_walk_online", "sky_sample_layout", "sky_sample_offline", "sky_sample_online", "sky_sample_session_begin", "sky_sample_session_frontier", "sky_sample_session_hop",
     "sky_sample_session_end", "sky_philox_selftest",
-    "sky_last_build_profile", "sky_set_option",
+    "sky_last_build_profile", "sky_set_option", "sky_graph_set_option", "sky_graph_unset_option",
 ]
 
 
@@ -270,6 +270,13 @@ class Graph:
     def sample_online(self, seeds, fanout, seed, out=None):
         """OnlineGBSampleNew."""
         return self._sample(lib().sky_sample_online, seeds, fanout, seed, out)
+
+    def set_option(self, name, value):
+        """A tuning knob for this graph alone (None: back to the process-wide value)."""
+        if value is None:
+            _ck(lib().sky_graph_unset_option(self.h, name.encode()))
+        else:
+            _ck(lib().sky_graph_set_option(self.h, name.encode(), C.c_long(value)))
 
     def free(self):
         if self.h:

@@ -1172,10 +1172,8 @@ struct BuildScratch {
   uint64_t* huge_scratch = nullptr;
   uint32_t vcap = 0, huge_cap = 0;
   uint64_t huge_scratch_cap = 0;
-  bool lds_enabled = false;
 };
-BuildScratch g_scratch;  // reused across builds; one build at a time per process
-bool g_row_merge = true;   // rows of 62..4093 entries: pairing by merge (else one binary search per entry)
+bool g_lds_enabled = false;  // the kernels' LDS limits are raised once per process
 
 template <class K>
 int enable_big_lds(K kernel, size_t bytes) {
@@ -1184,18 +1182,23 @@ int enable_big_lds(K kernel, size_t bytes) {
   return SKY_OK;
 }
 
+// The graph's build scratch, created on first use.
+BuildScratch& scratch_of(sky_graph* g) {
+  if (!g->build_scratch) g->build_scratch = new BuildScratch();
+  return *static_cast<BuildScratch*>(g->build_scratch);
+}
+
 }  // namespace
-static uint64_t g_stream_min_edges = 4000000;
-static uint64_t g_stream_wide_min_edges = 512ull * (STREAM_MAX_DEG / 2);  // 512 workgroups run at a time
-void set_stream_wide_min_edges(uint64_t n) { g_stream_wide_min_edges = n; }
-static bool g_build_profile = false;
-void set_build_profile(bool on) { g_build_profile = on; }
-static bool g_build_streams = true;
-void set_build_streams(bool on) { g_build_streams = on; }
-static int g_small_in_place = -1;  // -1: builds of at least 2^25 rows, 0: never, 1: always
-void set_small_in_place(int mode) { g_small_in_place = mode; }
-void set_stream_min_edges(uint64_t n) { g_stream_min_edges = n; }
-void set_row_merge(bool on) { g_row_merge = on; }
+
+void free_build_scratch(sky_graph* g) {
+  if (!g->build_scratch) return;
+  BuildScratch* sc = static_cast<BuildScratch*>(g->build_scratch);
+  void* ptrs[] = {sc->vlist, sc->counters, sc->blk_cnt, sc->huge_off, sc->huge_scratch};
+  for (void* p : ptrs)
+    if (p) (void)hipFree(p);
+  delete sc;
+  g->build_scratch = nullptr;
+}
 
 EventTimer::EventTimer(sky_graph* g) : stream(g->stream), pooled(g->ev), npooled(2) {}
 
@@ -1337,8 +1340,8 @@ int ensure_table_storage(sky_graph* g) {
   return SKY_OK;
 }
 
-int prepare_build_scratch(uint32_t max_rows) {
-  BuildScratch& sc = g_scratch;
+int prepare_build_scratch(sky_graph* g, uint32_t max_rows) {
+  BuildScratch& sc = scratch_of(g);
   if (sc.vcap < max_rows) {
     if (sc.vlist) SKY_HIP(hipFree(sc.vlist));
     sc.vlist = nullptr;
@@ -1348,13 +1351,13 @@ int prepare_build_scratch(uint32_t max_rows) {
   }
   if (!sc.counters) SKY_HIP(hipMalloc((void**)&sc.counters, COUNTER_BYTES));
   if (!sc.blk_cnt) SKY_HIP(hipMalloc((void**)&sc.blk_cnt, (size_t)BIN_BLOCKS * CLS_COUNT * 4));
-  if (!sc.lds_enabled) {
+  if (!g_lds_enabled) {
     SKY_TRY(enable_big_lds(build_lds_kernel<512, 2>, 512 * 4 * 2 * 16));
     SKY_TRY(enable_big_lds(build_merge_kernel<512, 10>, (512 * 10 + 2) * 14));
     SKY_TRY(enable_big_lds(build_merge_kernel<768, 6>, (768 * 6 + 2) * 14));
     SKY_TRY(enable_big_lds((build_merge_kernel<512, 10, 4, 1>), (512 * 10 + 2) * 14));
     SKY_TRY(enable_big_lds((build_merge_kernel<768, 6, 4, 1>), (768 * 6 + 2) * 14));
-    sc.lds_enabled = true;
+    g_lds_enabled = true;
   }
   return SKY_OK;
 }
@@ -1364,7 +1367,7 @@ int prepare_build_scratch(uint32_t max_rows) {
 int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   hipStream_t st = g->stream;
   g->has_walk_index = false;  // the table entries it was made from are about to change
-  BuildScratch& sc = g_scratch;
+  BuildScratch& sc = scratch_of(g);
   uint32_t counts[CLS_COUNT] = {0}, starts[CLS_COUNT] = {0};
   struct {
     uint32_t counts[2 * CLS_COUNT];
@@ -1376,7 +1379,8 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   // scale-26 graph), but it does not depend on the binning pass: on a side stream it runs beside the binning and
   // the kernels of the long rows (it waits on memory, they on the vector ALU): 10.2 -> 9.95 ms for the whole build.
   // Smaller builds, whose class kernels already overlap, gain nothing (scale 24: 3 % slower).
-  const bool small_in_place = g_small_in_place < 0 ? n >= (1u << 25) : g_small_in_place != 0;
+  const long long sip = option(g, OPT_SMALL_IN_PLACE);
+  const bool small_in_place = sip < 0 ? n >= (1u << 25) : sip != 0;
   const int listed_from = small_in_place ? CLS_G16 : CLS_G2;
   StreamFan fan(g, st);
   auto launch_small = [&](hipStream_t s) {
@@ -1438,7 +1442,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   RowRef* const vlist = sc.vlist;
   uint64_t call_edges = 0;
   for (int c = 0; c < CLS_COUNT; ++c) call_edges += host.edges[c];
-  if (!tm && g_build_streams && call_edges >= FAN_MIN_EDGES && call_edges < FAN_MAX_EDGES) SKY_TRY(fan.start());
+  if (!tm && option(g, OPT_BUILD_STREAMS) && call_edges >= FAN_MIN_EDGES && call_edges < FAN_MAX_EDGES) SKY_TRY(fan.start());
 
   auto grp = [&](int cls, auto kernel, int G, const char* name) -> int {
     const uint32_t cnt = counts[cls];
@@ -1476,7 +1480,8 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
   static const char* const mw_name[9] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9", "mw10"};
-  if (g_row_merge) {
+  const bool row_merge = option(g, OPT_ROW_MERGE) != 0;
+  if (row_merge) {
     SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 4>, 64, 4, "lds_w1"));
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 8>, 64, 8, "lds_w2"));
 #define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 8>, 64 * NW, 8, mw_name[NW - 2]))
@@ -1523,8 +1528,8 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   const uint32_t narrow_rows = counts[CLS_STREAM] + counts[CLS_STREAM_LAST];
   const uint64_t narrow_edges = host.edges[CLS_STREAM] + host.edges[CLS_STREAM_LAST];
   const uint64_t all_stream_edges = narrow_edges + host.edges[CLS_STREAM_WIDE];
-  const bool stream_to_tiled = !g_row_merge || all_stream_edges <= g_stream_min_edges;
-  const bool wide_streamed = !stream_to_tiled && all_stream_edges >= g_stream_wide_min_edges;
+  const bool stream_to_tiled = !row_merge || all_stream_edges <= (uint64_t)option(g, OPT_STREAM_MIN_EDGES);
+  const bool wide_streamed = !stream_to_tiled && all_stream_edges >= (uint64_t)option(g, OPT_STREAM_WIDE_MIN_EDGES);
   const uint32_t wide_rows = wide_streamed ? counts[CLS_STREAM_WIDE] : 0;
   if (!stream_to_tiled && narrow_rows + wide_rows) {
     StreamSwap sw(g, fan.next());
@@ -1545,7 +1550,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     SKY_TRY(fan.join());
     if (skipped) {  // rows with more tiles than the tile-parallel path takes: one workgroup streams each
-      const uint32_t max_tiles = tiled_max_tiles();
+      const uint32_t max_tiles = tiled_max_tiles(g);
       if (sc.huge_cap < cnt) {
         if (sc.huge_off) SKY_HIP(hipFree(sc.huge_off));
         sc.huge_off = nullptr;
@@ -1585,13 +1590,13 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
 constexpr uint32_t DEV_GRID_STREAM = 512;
 constexpr uint32_t dev_grid_cap(int threads) { return threads <= 64 ? 16384u : threads <= 256 ? 8192u : 2048u; }
 
-bool build_rows_dev_possible(const sky_graph* g) { return g_row_merge && tiled_max_tiles() == (1u << 22); }
+bool build_rows_dev_possible(const sky_graph* g) { return option(g, OPT_ROW_MERGE) != 0 && tiled_max_tiles(g) == (1u << 22); }
 
 int ensure_class_census(sky_graph* g) {
   if (g->bin_known || g->V == 0) return SKY_OK;
   hipStream_t st = g->stream;
-  SKY_TRY(prepare_build_scratch(1));
-  BuildScratch& sc = g_scratch;
+  SKY_TRY(prepare_build_scratch(g, 1));
+  BuildScratch& sc = scratch_of(g);
   struct {
     uint32_t counts[2 * CLS_COUNT];
     unsigned long long edges[CLS_COUNT];
@@ -1621,7 +1626,7 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
     return fail(SKY_ERR_STATE, "build_rows_dev: needs the class census and rows the streaming kernel takes");
   hipStream_t st = g->stream;
   g->has_walk_index = false;
-  BuildScratch& sc = g_scratch;
+  BuildScratch& sc = scratch_of(g);
   const uint32_t step = 256u * BIN_ITEMS;
   const uint32_t per_block = ((n_upper + BIN_BLOCKS - 1) / BIN_BLOCKS + step - 1) / step * step;
   const uint32_t blocks = (n_upper + per_block - 1) / per_block;
@@ -1642,7 +1647,7 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   const RowRef* const vlist = sc.vlist;
   // the class kernels are independent of one another: they go out in turn over the graph's stream and its side streams
   StreamFan fan(g, st);
-  if (g_build_streams && n_upper >= 4096) SKY_TRY(fan.start());
+  if (option(g, OPT_BUILD_STREAMS) && n_upper >= 4096) SKY_TRY(fan.start());
   // Rows of 5118 entries and more first, because theirs is the longest chain of launches.  The classes STREAM,
   // STREAM_LAST, STREAM_WIDE, HUGE lie back to back.  What the graph holds of them decides, as in a build of all
   // rows, which go to the streaming kernel (one workgroup per row) and which are built tile by tile by the whole
@@ -1651,7 +1656,7 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   // workgroup each.
   static_assert(CLS_STREAM_LAST == CLS_STREAM + 1 && CLS_STREAM_WIDE == CLS_STREAM + 2 && CLS_HUGE == CLS_STREAM + 3,
                 "the lists of the long rows lie back to back");
-  const bool narrow_tiled = g->bin_edges[CLS_STREAM] + g->bin_edges[CLS_STREAM_LAST] <= g_stream_min_edges;
+  const bool narrow_tiled = g->bin_edges[CLS_STREAM] + g->bin_edges[CLS_STREAM_LAST] <= (uint64_t)option(g, OPT_STREAM_MIN_EDGES);
   const uint32_t stream_rows = narrow_tiled ? 0 : rows_of(CLS_STREAM) + rows_of(CLS_STREAM_LAST);
   const int t_first = narrow_tiled ? CLS_STREAM : CLS_STREAM_WIDE;
   uint32_t tiled_rows = 0;
@@ -1720,10 +1725,10 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
 
 int build_all_tables(sky_graph* g, double* seconds) {
   SKY_TRY(ensure_table_storage(g));
-  SKY_TRY(prepare_build_scratch(g->V));
+  SKY_TRY(prepare_build_scratch(g, g->V));
   EventTimer tm(g);
   SKY_TRY(tm.mark("start", 0));
-  if (g_build_profile) {
+  if (option(g, OPT_BUILD_PROFILE)) {
     SKY_TRY(build_rows(g, nullptr, g->V, &tm));
   } else {  // one bracket around the whole build: no event between the kernels
     SKY_TRY(build_rows(g, nullptr, g->V, nullptr));

@@ -627,14 +627,28 @@ struct TiledScratch {
   uint32_t* nfh = nullptr;
   uint4* ranges = nullptr;
   uint32_t row_cap = 0, tile_cap = 0;
-  bool lds_enabled = false;
+  size_t b_cap = 0;  // entries of BL and BH
 };
-TiledScratch g_tiled;
-uint32_t g_tiled_max_tiles = TILED_MAX_TILES;
+TiledScratch& tiled_of(sky_graph* g) {
+  if (!g->tiled_scratch) g->tiled_scratch = new TiledScratch();
+  return *static_cast<TiledScratch*>(g->tiled_scratch);
+}
 }  // namespace
 
-uint32_t tiled_max_tiles() { return g_tiled_max_tiles; }
-void set_tiled_max_tiles(uint32_t n) { g_tiled_max_tiles = std::min<uint32_t>(std::max<uint32_t>(n, 1), TILED_MAX_TILES); }
+void free_tiled_scratch(sky_graph* g) {
+  if (!g->tiled_scratch) return;
+  TiledScratch* sc = static_cast<TiledScratch*>(g->tiled_scratch);
+  void* ptrs[] = {sc->rows, sc->totals, sc->geom, sc->tsum, sc->ttot, sc->BL, sc->BH, sc->nfh, sc->ranges};
+  for (void* p : ptrs)
+    if (p) (void)hipFree(p);
+  delete sc;
+  g->tiled_scratch = nullptr;
+}
+
+uint32_t tiled_max_tiles(const sky_graph* g) {
+  const long long n = option(g, OPT_TILED_MAX_TILES);
+  return (uint32_t)std::min<long long>(std::max<long long>(n, 1), TILED_MAX_TILES);
+}
 
 // Builds the rows of `rows_list` (device, n entries) that have at most the configured number of
 // tiles; *skipped receives how many rows were left for the streaming kernel.  `edges` is the number of
@@ -645,7 +659,8 @@ void set_tiled_max_tiles(uint32_t n) { g_tiled_max_tiles = std::min<uint32_t>(st
 static int build_rows_tiled_any(sky_graph* g, const RowRef* rows_list, uint32_t n, const uint32_t* dev, int cls, int ncls,
                                 uint32_t* skipped, EventTimer* tm, uint64_t edges) {
   hipStream_t st = g->stream;
-  TiledScratch& sc = g_tiled;
+  TiledScratch& sc = tiled_of(g);
+  const uint32_t max_tiles = tiled_max_tiles(g);
   *skipped = 0;
   if (n == 0) return SKY_OK;
   if (sc.row_cap < n) {
@@ -658,8 +673,8 @@ static int build_rows_tiled_any(sky_graph* g, const RowRef* rows_list, uint32_t 
   if (!sc.totals) SKY_HIP(hipMalloc((void**)&sc.totals, sizeof(TiledCounters)));
   SKY_HIP(hipMemsetAsync(sc.totals, 0, sizeof(TiledCounters), st));
   hipLaunchKernelGGL(tiled_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, st, rows_list, n, dev, cls, ncls, g->xadj,
-                     g_tiled_max_tiles, sc.rows, sc.totals);
-  const bool bounded = edges != 0 && g_tiled_max_tiles == TILED_MAX_TILES && edges / TILE + 2ull * n < (1ull << 31);
+                     max_tiles, sc.rows, sc.totals);
+  const bool bounded = edges != 0 && max_tiles == TILED_MAX_TILES && edges / TILE + 2ull * n < (1ull << 31);
   uint32_t ntiles, nslots;
   if (bounded) {
     ntiles = (uint32_t)(edges / TILE + 2ull * n);
@@ -688,16 +703,15 @@ static int build_rows_tiled_any(sky_graph* g, const RowRef* rows_list, uint32_t 
     sc.tile_cap = (uint32_t)cap;
   }
   // prefix arrays hold ntiles + one extra entry per row
-  static size_t b_cap = 0;
   const size_t b_need = (size_t)ntiles + nslots;
-  if (b_cap < b_need) {
+  if (sc.b_cap < b_need) {
     if (sc.BL) SKY_HIP(hipFree(sc.BL));
     if (sc.BH) SKY_HIP(hipFree(sc.BH));
     sc.BL = sc.BH = nullptr;
-    b_cap = 0;
+    sc.b_cap = 0;
     SKY_HIP(hipMalloc((void**)&sc.BL, (b_need + b_need / 4 + 1024) * 8));
     SKY_HIP(hipMalloc((void**)&sc.BH, (b_need + b_need / 4 + 1024) * 8));
-    b_cap = b_need + b_need / 4 + 1024;
+    sc.b_cap = b_need + b_need / 4 + 1024;
   }
   if (bounded) SKY_HIP(hipMemsetAsync(sc.geom, 0, (size_t)ntiles * sizeof(TileGeom), st));  // span 0: no such tile
   hipLaunchKernelGGL(tiled_map_kernel, dim3(n), dim3(256), 0, st, sc.rows, n, sc.geom);
@@ -721,7 +735,7 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
 
 int build_rows_tiled_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int cls, int ncls, uint32_t n_upper,
                          uint64_t edges_upper) {
-  if (g_tiled_max_tiles != TILED_MAX_TILES || edges_upper == 0 || edges_upper / TILE + 2ull * n_upper >= (1ull << 31))
+  if (tiled_max_tiles(g) != TILED_MAX_TILES || edges_upper == 0 || edges_upper / TILE + 2ull * n_upper >= (1ull << 31))
     return fail(SKY_ERR_STATE, "build_rows_tiled_dev: the number of tiles has no usable bound");
   uint32_t skipped = 0;
   return build_rows_tiled_any(g, vlist, n_upper, dev, cls, ncls, &skipped, nullptr, edges_upper);

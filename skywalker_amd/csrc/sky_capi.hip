@@ -30,6 +30,24 @@ static int ensure_device() {
 
 using namespace sky;
 
+namespace sky {
+// process-wide values of the tuning knobs, in the order of SkyOpt (sky_set_option changes them)
+long long g_option_value[OPT_COUNT] = {
+    1ll << 22,                             // tiled_max_tiles: no limit
+    1,                                     // row_merge
+    4000000,                               // stream_min_edges
+    512ll * (sky::STREAM_MAX_DEG / 2),     // stream_wide_min_edges: 512 workgroups run at a time
+    -1,                                    // walk_read_once: by the size of the tables
+    0,                                     // sample_distinct
+    -1,                                    // small_in_place: builds of at least 2^25 rows
+    1,                                     // build_streams
+    0,                                     // build_profile
+    0,                                     // walk_compact_every
+    -1,                                    // online_full_build: by estimate
+    1,                                     // online_device_sized
+};
+}  // namespace sky
+
 extern "C" {
 
 const char* sky_last_error(void) { return g_last_error.c_str(); }
@@ -201,6 +219,8 @@ int sky_graph_free(sky_graph* g) {
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   pool_release(g);
+  free_build_scratch(g);
+  free_tiled_scratch(g);
   if (g->live_report) (void)hipHostFree(g->live_report);
   delete g;
   return SKY_OK;
@@ -448,63 +468,68 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
   return philox_selftest(ctr_host, key_host, n, out_host);
 }
 
+// name, smallest and largest accepted value of every knob, in the order of SkyOpt
+struct OptionSpec {
+  const char* name;
+  long long lo, hi;
+};
+static const OptionSpec g_option_spec[OPT_COUNT] = {
+    {"tiled_max_tiles", 1, 1ll << 22},
+    {"row_merge", 0, 1},
+    {"stream_min_edges", 0, 1ll << 40},
+    {"stream_wide_min_edges", 0, 1ll << 40},
+    {"walk_read_once", -1, 1},
+    {"sample_distinct", 0, 1},
+    {"small_in_place", -1, 1},
+    {"build_streams", 0, 1},
+    {"build_profile", 0, 1},
+    {"walk_compact_every", 0, 1ll << 31},
+    {"online_full_build", -1, 1},
+    {"online_device_sized", 0, 1},
+};
+static int parse_option(const char* who, const char* name, long value, int* index, long long* stored) {
+  if (!name) return fail(SKY_ERR_ARG, std::string(who) + ": null name");
+  for (int i = 0; i < OPT_COUNT; ++i) {
+    if (strcmp(name, g_option_spec[i].name)) continue;
+    const OptionSpec& sp = g_option_spec[i];
+    long long v = value;
+    if (sp.lo == 0 && sp.hi == 1) v = value != 0;  // switches take any non-zero value as "on"
+    if (i == OPT_TILED_MAX_TILES && v > sp.hi) v = sp.hi;
+    if (v < sp.lo || v > sp.hi)
+      return fail(SKY_ERR_ARG, std::string(who) + ": " + name + " takes " + std::to_string(sp.lo) + " .. " +
+                                   std::to_string(sp.hi));
+    *index = i;
+    *stored = v;
+    return SKY_OK;
+  }
+  return fail(SKY_ERR_ARG, std::string(who) + ": unknown option " + name);
+}
+
 int sky_set_option(const char* name, long value) {
-  if (!name) return fail(SKY_ERR_ARG, "sky_set_option: null name");
-  if (!strcmp(name, "tiled_max_tiles")) {
-    if (value < 1) return fail(SKY_ERR_ARG, "sky_set_option: tiled_max_tiles must be >= 1");
-    set_tiled_max_tiles((uint32_t)value);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "row_merge")) {
-    set_row_merge(value != 0);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "stream_min_edges")) {
-    if (value < 0) return fail(SKY_ERR_ARG, "sky_set_option: stream_min_edges must be >= 0");
-    set_stream_min_edges((uint64_t)value);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "walk_read_once")) {
-    if (value < -1 || value > 1) return fail(SKY_ERR_ARG, "sky_set_option: walk_read_once is -1, 0 or 1");
-    set_walk_read_once((int)value);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "sample_distinct")) {
-    set_sample_distinct(value != 0);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "small_in_place")) {
-    if (value < -1 || value > 1) return fail(SKY_ERR_ARG, "sky_set_option: small_in_place is -1, 0 or 1");
-    set_small_in_place((int)value);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "build_streams")) {
-    set_build_streams(value != 0);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "stream_wide_min_edges")) {
-    if (value < 0) return fail(SKY_ERR_ARG, "sky_set_option: stream_wide_min_edges must be >= 0");
-    set_stream_wide_min_edges((uint64_t)value);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "build_profile")) {
-    set_build_profile(value != 0);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "walk_compact_every")) {
-    if (value < 0) return fail(SKY_ERR_ARG, "sky_set_option: walk_compact_every must be >= 0");
-    set_walk_compact_every((uint32_t)value);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "online_device_sized")) {
-    set_online_device_sized(value != 0);
-    return SKY_OK;
-  }
-  if (!strcmp(name, "online_full_build")) {
-    set_online_full_build((int)value);
-    return SKY_OK;
-  }
-  return fail(SKY_ERR_ARG, std::string("sky_set_option: unknown option ") + name);
+  int i = 0;
+  long long v = 0;
+  SKY_TRY(parse_option("sky_set_option", name, value, &i, &v));
+  g_option_value[i] = v;
+  return SKY_OK;
+}
+int sky_graph_set_option(sky_graph* g, const char* name, long value) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_graph_set_option: null graph");
+  int i = 0;
+  long long v = 0;
+  SKY_TRY(parse_option("sky_graph_set_option", name, value, &i, &v));
+  g->opt_value[i] = v;
+  g->opt_own[i] = true;
+  return SKY_OK;
+}
+int sky_graph_unset_option(sky_graph* g, const char* name) {
+  if (!g) return fail(SKY_ERR_ARG, "sky_graph_unset_option: null graph");
+  if (!name) return fail(SKY_ERR_ARG, "sky_graph_unset_option: null name");
+  for (int i = 0; i < OPT_COUNT; ++i)
+    if (!strcmp(name, g_option_spec[i].name)) {
+      g->opt_own[i] = false;
+      return SKY_OK;
+    }
+  return fail(SKY_ERR_ARG, std::string("sky_graph_unset_option: unknown option ") + name);
 }
 
 int sky_last_build_profile(const sky_graph* g, const char** names, float* ms, uint64_t* edges, int max_entries) {

@@ -4,8 +4,32 @@
 
 #include "sky_common.h"
 
+// The tuning knobs of sky_set_option / sky_graph_set_option.  A graph reads a knob through option(g, ...): its own
+// value when sky_graph_set_option has given it one, the process-wide value otherwise.
+enum SkyOpt : int {
+  OPT_TILED_MAX_TILES = 0,
+  OPT_ROW_MERGE,
+  OPT_STREAM_MIN_EDGES,
+  OPT_STREAM_WIDE_MIN_EDGES,
+  OPT_WALK_READ_ONCE,
+  OPT_SAMPLE_DISTINCT,
+  OPT_SMALL_IN_PLACE,
+  OPT_BUILD_STREAMS,
+  OPT_BUILD_PROFILE,
+  OPT_WALK_COMPACT_EVERY,
+  OPT_ONLINE_FULL_BUILD,
+  OPT_ONLINE_DEVICE_SIZED,
+  OPT_COUNT
+};
+
 struct sky_graph {
   uint32_t V = 0, E = 0, max_degree = 0;
+  long long opt_value[OPT_COUNT] = {0};
+  bool opt_own[OPT_COUNT] = {false};  // the graph has a value of its own for the knob
+  // scratch memory of the table builds on this graph (allocated on first use, reused by every later build, freed
+  // with the graph): row lists and counters of the binning pass, and the arrays of the tile-parallel path
+  void* build_scratch = nullptr;
+  void* tiled_scratch = nullptr;
   int device = 0;  // the device that was current when the graph was created: its arrays live there
   // CSR, device resident.  Arrays are allocated with 16 spare bytes so that kernels may
   // read whole aligned float4/uint4 quads that straddle the end.
@@ -112,7 +136,7 @@ struct EventTimer {
 int pool_get(sky_graph* g, int slot, size_t bytes, void** out);
 void pool_release(sky_graph* g);
 int ensure_table_storage(sky_graph* g);
-int prepare_build_scratch(uint32_t max_rows);
+int prepare_build_scratch(sky_graph* g, uint32_t max_rows);
 int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm);
 int build_all_tables(sky_graph* g, double* seconds);
 // rows of more than 4093 entries: tile-parallel path, and how many tiles per row it accepts
@@ -121,7 +145,6 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
                      uint64_t edges);
 int build_rows_tiled_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int cls, int ncls, uint32_t n_upper,
                          uint64_t edges_upper);
-void set_tiled_max_tiles(uint32_t n);
 constexpr int MERGE_MAX_NW = 10;  // rows of at most 512 * 10 - 3 = 5117 entries pair by merge in LDS
 constexpr uint32_t STREAM_MAX_DEG = 524287;  // longest row of the streaming classes (one workgroup takes 1.5 ms for it)
 int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n);
@@ -132,20 +155,13 @@ int build_rows_stream_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev
 bool build_rows_dev_possible(const sky_graph* g);
 int ensure_class_census(sky_graph* g);
 int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uint32_t n_upper);
-void set_row_merge(bool on);
-void set_stream_min_edges(uint64_t n);
-void set_stream_wide_min_edges(uint64_t n);
-void set_build_streams(bool on);
-void set_small_in_place(int mode);
-void set_sample_distinct(bool on);
-void set_online_device_sized(bool on);
-extern bool g_online_device_sized;
-void set_walk_read_once(int mode);
-void set_build_profile(bool on);
-void set_online_full_build(int mode);
-void set_walk_compact_every(uint32_t steps);
 int build_walk_index(sky_graph* g, double* seconds);
-uint32_t tiled_max_tiles();
+uint32_t tiled_max_tiles(const sky_graph* g);
+// process-wide values of the knobs (sky_capi.hip) and the accessor every use goes through
+extern long long g_option_value[OPT_COUNT];
+inline long long option(const sky_graph* g, SkyOpt o) { return g && g->opt_own[o] ? g->opt_value[o] : g_option_value[o]; }
+void free_build_scratch(sky_graph* g);
+void free_tiled_scratch(sky_graph* g);
 int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,
                  uint32_t* paths, uint32_t* lengths, uint64_t* sampled, double* seconds);
 int walk_offline_noalloc(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, float stop_prob, uint64_t seed,

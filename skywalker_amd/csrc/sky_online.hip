@@ -94,15 +94,15 @@ int walk_online_node2vec(sky_graph* g, float p, float q, const uint32_t* seeds, 
                          float stop_prob, uint64_t seed, uint32_t* paths, uint32_t* lengths, uint64_t* sampled,
                          double* seconds);
 
-// -1: decide by the estimate below; 0: always build lazily, step by step; 1: always build every row first.
-static int g_online_full_build = -1;
-void set_online_full_build(int mode) { g_online_full_build = mode < 0 ? -1 : (mode ? 1 : 0); }
+// Option online_full_build: -1: decide by the estimate below; 0: always build lazily, step by step; 1: always build
+// every row first.
 
 // Estimated milliseconds of the two ways to serve a static-bias online walk.  A lazy round costs a
 // host round trip and a handful of small launches (about 1/8 ms measured), and the rounds together
 // build at most min(N * len, V) rows; the full build runs at about 1.3e8 edges per millisecond.
 static bool online_prefers_full_build(const sky_graph* g, uint32_t N, uint32_t len) {
-  if (g_online_full_build >= 0) return g_online_full_build == 1;
+  const long long mode = option(g, OPT_ONLINE_FULL_BUILD);
+  if (mode >= 0) return mode != 0;
   const double all_ms = (double)g->E / 1.3e8;
   const double visited = std::min(1.0, (double)N * len / std::max(1u, g->V));
   return 0.4 + all_ms < 0.125 * len + visited * all_ms;
@@ -133,7 +133,7 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
   // there (build_rows_dev), and whether any walker still walks comes back through pinned host words that the host
   // reads as they arrive, some steps behind what it has enqueued; the steps enqueued past the last walker's end find
   // nothing to do.
-  const bool dev_sized = build_rows_dev_possible(g) && g_online_device_sized;
+  const bool dev_sized = build_rows_dev_possible(g) && option(g, OPT_ONLINE_DEVICE_SIZED) != 0;
   auto body = [&]() -> int {
     SKY_TRY(ensure_table_storage(g));
     if (dev_sized) {
@@ -147,7 +147,7 @@ int walk_online(sky_graph* g, int bias_kind, float p, float q, const uint32_t* s
       }
       for (uint32_t s = 0; s < len; ++s) g->live_report[s] = 0xFFFFFFFFu;  // "not reported yet"
     }
-    SKY_TRY(prepare_build_scratch(std::min(N, g->V)));
+    SKY_TRY(prepare_build_scratch(g, std::min(N, g->V)));
     SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
     d_cnt = reinterpret_cast<uint32_t*>(d_sampled + 1);
     SKY_TRY(pool_get(g, sky_graph::POOL_BITMAP, (size_t)words * 4, (void**)&bitmap));

@@ -217,10 +217,6 @@ __global__ __launch_bounds__(256) void sample_init_kernel(const uint32_t* __rest
   if (i < N) data[(uint64_t)i * lps] = seeds[i];
 }
 
-static bool g_sample_distinct = false;
-void set_sample_distinct(bool on) { g_sample_distinct = on; }
-bool g_online_device_sized = true;  // option "online_device_sized": 0 makes the online modes wait for every frontier size
-void set_online_device_sized(bool on) { g_online_device_sized = on; }
 
 // One call of the k-hop sampler, taken apart hop by hop: begin (outputs cleared, start vertices in place), then for
 // every hop frontier (online: the distinct parents whose rows are not built yet), build (online: their rows) and
@@ -268,7 +264,7 @@ struct SampleSession {
     seed = seed_;
     data = data_;
     sample_lengths = sl_;
-    distinct = g_sample_distinct;
+    distinct = option(g, OPT_SAMPLE_DISTINCT) != 0;
     fanout.assign(fanout_, fanout_ + hops);
     if (distinct) {
       if (hops > 256) return fail(SKY_ERR_LIMIT, "sample: distinct children need at most 256 hops");
@@ -278,7 +274,7 @@ struct SampleSession {
     if (g->has_tables) online = false;  // every row is already there: nothing to build on the way
     // Without the option the host reads the size of every frontier and sizes the launches of its build exactly;
     // with it (the default) nothing inside the call waits for the device.
-    dev_sized = online && build_rows_dev_possible(g) && g_online_device_sized;
+    dev_sized = online && build_rows_dev_possible(g) && option(g, OPT_ONLINE_DEVICE_SIZED) != 0;
     width.assign(hops, 0);
     off.assign(hops, 0);
     loff.assign(hops, 0);
@@ -302,7 +298,7 @@ struct SampleSession {
     if (online) {
       SKY_TRY(ensure_table_storage(g));
       if (dev_sized) SKY_TRY(ensure_class_census(g));  // once per graph
-      SKY_TRY(prepare_build_scratch(g->V));
+      SKY_TRY(prepare_build_scratch(g, g->V));
       SKY_TRY(pool_get(g, sky_graph::POOL_BITMAP, (size_t)words * 4, (void**)&bitmap));
       SKY_TRY(pool_get(g, sky_graph::POOL_LIST, (size_t)g->V * 4, (void**)&list));
     }

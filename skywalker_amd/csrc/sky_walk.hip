@@ -143,13 +143,12 @@ __global__ __launch_bounds__(WALK_BLOCK) void walk_offline_kernel(
   }
 }
 
-static uint32_t g_walk_compact_every = 0;  // 0: one launch, every walker keeps its lane for the whole walk
-void set_walk_compact_every(uint32_t steps) { g_walk_compact_every = steps; }
-static int g_walk_read_once = -1;  // -1: by the size of the tables, 0 / 1: never / always load entries as read-once data
-void set_walk_read_once(int mode) { g_walk_read_once = mode; }
+// Options walk_compact_every (0: one launch, every walker keeps its lane for the whole walk) and walk_read_once
+// (-1: by the size of the tables, 0 / 1: never / always load entries as read-once data).
 // Tables of more than 2 GiB (the last-level cache holds 256 MiB) are gathered from as read-once data.
 static bool walk_reads_once(const sky_graph* g) {
-  return g_walk_read_once < 0 ? (uint64_t)g->E * sizeof(AliasEntry) > (2ull << 30) : g_walk_read_once != 0;
+  const long long mode = option(g, OPT_WALK_READ_ONCE);
+  return mode < 0 ? (uint64_t)g->E * sizeof(AliasEntry) > (2ull << 30) : mode != 0;
 }
 
 template <bool INDEXED>
@@ -173,7 +172,7 @@ int walk_offline(sky_graph* g, const uint32_t* seeds, uint32_t N, uint32_t len, 
   hipStream_t st = g->stream;
   unsigned long long* d_sampled = nullptr;
   SKY_TRY(pool_get(g, sky_graph::POOL_COUNTERS, 64, (void**)&d_sampled));
-  const uint32_t every = g_walk_compact_every;
+  const uint32_t every = (uint32_t)option(g, OPT_WALK_COMPACT_EVERY);
   const bool segmented = every > 0 && every < len && N > 0;
   const uint32_t nseg = segmented ? (len + every - 1) / every : 1;
   uint32_t *lists = nullptr, *counts = nullptr;

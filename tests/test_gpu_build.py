@@ -26,15 +26,11 @@ def build_and_compare(orc, xadj, adjncy, w, label):
     # vertices in order
     for stream_min_edges, small_in_place in [(r, 0) for r in routes] + [(routes[0], 1)]:
         g = capi.Graph.upload(xadj, adjncy, w)
-        capi.set_option("stream_min_edges", stream_min_edges)
-        capi.set_option("stream_wide_min_edges", stream_min_edges)  # 0: also the rows above 65533 entries are streamed
-        capi.set_option("small_in_place", small_in_place)
-        try:
-            g.build_tables()
-        finally:
-            capi.set_option("stream_min_edges", 4000000)
-            capi.set_option("stream_wide_min_edges", 512 * 262143)
-            capi.set_option("small_in_place", -1)
+        # knobs of this graph alone: nothing to restore, whatever happens below
+        g.set_option("stream_min_edges", stream_min_edges)
+        g.set_option("stream_wide_min_edges", stream_min_edges)  # 0: also the rows above 65533 entries are streamed
+        g.set_option("small_in_place", small_in_place)
+        g.build_tables()
         prob, alias, valid = g.tables()
         g.free()
         st = orc.alias_check(xadj, w, prob, alias, valid)
@@ -329,3 +325,30 @@ def test_random_mixtures_of_every_class(orc, seed):
         w[pick] = special[rng.integers(0, len(special), pick.sum())]
     with np.errstate(all="ignore"):
         build_and_compare(orc, xadj, adjncy, w, "mixture %d/%s" % (seed, dist))
+
+
+def test_two_graphs_hold_different_settings(orc):
+    # a knob set on one graph (sky_graph_set_option) leaves the other graph and the process-wide value alone
+    from skywalker_amd import capi
+    rng = np.random.default_rng(51)
+    xadj, adjncy, w = graph_from_degrees(list(rng.integers(1, 200, 500)) + [300, 2000], rng, "lognormal")
+    a = capi.Graph.upload(xadj, adjncy, w)
+    b = capi.Graph.upload(xadj, adjncy, w)
+    a.set_option("build_profile", 1)
+    a.build_tables()
+    b.build_tables()
+    assert len(a.build_profile()) > 3 and [p[0] for p in b.build_profile()] == ["build"]
+    c = capi.Graph.upload(xadj, adjncy, w)
+    c.build_tables()
+    assert [p[0] for p in c.build_profile()] == ["build"]  # the process-wide value did not move
+    a.set_option("build_profile", None)
+    a.build_tables()
+    assert [p[0] for p in a.build_profile()] == ["build"]
+    with pytest.raises(capi.SkyError):
+        a.set_option("no_such_knob", 1)
+    with pytest.raises(capi.SkyError):
+        a.set_option("small_in_place", 7)
+    want = a.tables()[0]
+    for g in (a, b, c):
+        assert np.array_equal(g.tables()[0], want)
+        g.free()
