@@ -61,6 +61,9 @@ def class_degrees(per_class, seed):
 # read the weights count 4; xadj / valid are per vertex and small
 BYTES_PER_EDGE = {"tiled_sum": 4, "tiled_totals": 4}
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "c5_kernel_traffic.txt")
+# measured HBM bytes of one whole batch of the online configurations (sum over the batch's kernels)
+BATCH_TRAFFIC_FILE = {"c3": os.path.join(ROOT, "profiles", "c3_batch_traffic.txt"),
+                      "c4": os.path.join(ROOT, "profiles", "c4_batch_traffic.txt")}
 METRIC = "sampled edges/sec (SEPS) + alias-table build edges/sec on 1 MI355X; % HBM peak"
 ARITHMETIC = "f64 classification and exact three-limb sums, u64 fixed-point ledger, f32 tables, u32 indices"
 KERNEL_OF = {  # build_profile entry -> kernel symbol
@@ -116,6 +119,24 @@ def load_traffic():
                 table[k] = float(v)
         return table, head
     except (OSError, ValueError):
+        return None, None
+
+
+def load_batch_traffic(config):
+    """profiles/<config>_batch_traffic.txt: `bytes_per_batch <n>` plus header lines `# key: value`.
+    Returns (bytes, header dict) or (None, None)."""
+    try:
+        head, val = {}, None
+        for line in open(BATCH_TRAFFIC_FILE[config]):
+            line = line.strip()
+            if line.startswith("#"):
+                if ":" in line:
+                    k, v = line[1:].split(":", 1)
+                    head[k.strip()] = v.strip()
+            elif line.startswith("bytes_per_batch"):
+                val = float(line.split()[1])
+        return val, head
+    except (OSError, ValueError, KeyError, IndexError):
         return None, None
 
 
@@ -204,14 +225,15 @@ def online_bench(args, cfg, capi, g, seeds, name, cus, t_gen, torch):
             per_slot += int((8 + 4 * d[d > 0] + 8 * np.minimum(d[d > 0], k)).sum())
             rows.append(np.unique(front))
         distinct = np.unique(np.concatenate(rows)) if rows else np.zeros(0, np.int64)
-        alg_bytes = per_slot
         # what one batch must move at least when every distinct frontier row is built once (as this library does):
-        # 12 bytes per entry of those rows + 8 per row, + 8 per sampled edge
+        # 12 bytes per entry of those rows + 8 per row, + 8 per sampled edge.  The per-slot formula of a sampler that
+        # rebuilds a row for every frontier slot that holds it counts the same row many times over: kept as detail.
         distinct_bytes = int(12 * deg[distinct].sum() + 8 * len(distinct)) + 8 * int(sampled)
-        detail = {"formula": "sum over frontier vertices of 8 + 4 d + 8 min(k, d)",
+        alg_bytes = distinct_bytes
+        detail = {"formula": "12 per entry and 8 per row of the distinct frontier rows (each built once) + 8 per sampled edge",
                   "distinct_rows_built": int(len(distinct)), "distinct_row_edges": int(deg[distinct].sum()),
-                  "bytes_with_each_distinct_row_built_once": distinct_bytes,
-                  "frac_with_each_distinct_row_built_once": distinct_bytes / ksec / HBM_PEAK}
+                  "per_slot_formula": "sum over frontier slots of 8 + 4 d + 8 min(k, d)",
+                  "per_slot_bytes": per_slot, "per_slot_frac": per_slot / ksec / HBM_PEAK}
         kernel = "one batch: frontier_collect_kernel, the build kernels of the frontier rows, sample_hop_kernel (per hop)"
     else:
         steps = sampled
@@ -232,8 +254,11 @@ def online_bench(args, cfg, capi, g, seeds, name, cus, t_gen, torch):
             detail = {"formula": "12 E + 5 V (first-order tables) + 24 per step; the rejection trials' reads "
                                  "(12 + 4 log2 d_prev each) are not counted: a lower bound"}
             kernel = "one batch: the offline build kernels, walk_n2v_reject_group_kernel"
+    traffic, thead = (None, None) if args.n2v_table else load_batch_traffic(args.config)
     roofline = {"bound": "hbm", "kernel": kernel, "achieved": alg_bytes / ksec / 1e9, "peak": HBM_PEAK / 1e9,
-                "unit": "GB/s", "frac": alg_bytes / ksec / HBM_PEAK, "traffic": None,
+                "unit": "GB/s", "frac": alg_bytes / ksec / HBM_PEAK, "traffic": traffic,
+                "traffic_source": ("%s (commit %s)" % (os.path.relpath(BATCH_TRAFFIC_FILE[args.config], ROOT),
+                                                       thead.get("commit", "?"))) if traffic else None,
                 "launch_ms": ksec * 1e3, "algorithmic_bytes_per_launch": alg_bytes, "detail": detail}
 
     cpu = None

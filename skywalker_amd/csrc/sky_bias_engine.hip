@@ -101,11 +101,16 @@ __global__ __launch_bounds__(256) void bias_init_kernel(const uint32_t* __restri
   states[i] = st;
 }
 
+// One workgroup per walker that is still walking: `live` lists them (null: walkers 0 .. gridDim.x - 1), *n_live says
+// how many they are (the grid covers an upper bound that the host knows).
 __global__ __launch_bounds__(sky::N2V_T) void bias_step_kernel(View g, uint32_t len, uint32_t s, float stop_prob,
-                                                               uint64_t seed, uint32_t* __restrict__ paths,
+                                                               uint64_t seed, const uint32_t* __restrict__ live,
+                                                               const uint32_t* __restrict__ n_live,
+                                                               uint32_t* __restrict__ paths,
                                                                uint32_t* __restrict__ lengths,
                                                                sky_walker_state* __restrict__ states) {
-  const uint32_t i = blockIdx.x;
+  if (live && blockIdx.x >= *n_live) return;
+  const uint32_t i = live ? live[blockIdx.x] : blockIdx.x;
   const int tid = threadIdx.x;
   if (lengths[i] != len) return;  // stopped at an earlier step
   const sky::u32x4 r = sky::philox(seed, i, s, 0, sky::DOM_WALK);
@@ -133,6 +138,39 @@ __global__ __launch_bounds__(sky::N2V_T) void bias_step_kernel(View g, uint32_t 
       sky_update_walker_state(&st, v);
       states[i] = st;
     }
+  }
+}
+
+// The walkers of `in` (null: 0 .. n_first - 1) that still walk after the step, appended to `out`: one counter
+// update per workgroup of 1024 lanes (every append goes through one word, which serves its atomics one by one).
+__global__ __launch_bounds__(1024) void bias_compact_kernel(const uint32_t* __restrict__ in,
+                                                            const uint32_t* __restrict__ n_in, uint32_t n_first,
+                                                            const uint32_t* __restrict__ lengths, uint32_t len,
+                                                            uint32_t* __restrict__ out, uint32_t* __restrict__ n_out) {
+  __shared__ uint32_t s_n[16];
+  __shared__ uint32_t s_base;
+  const uint32_t n = in ? *n_in : n_first;
+  const uint32_t idx = blockIdx.x * 1024u + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t i = 0;
+  bool alive = false;
+  if (idx < n) {
+    i = in ? in[idx] : idx;
+    alive = lengths[i] == len;
+  }
+  const unsigned long long m = __ballot(alive);
+  if (lane == 0) s_n[wave] = (uint32_t)__popcll(m);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t t = 0;
+    for (int w = 0; w < 16; ++w) t += s_n[w];
+    s_base = t ? atomicAdd(n_out, t) : 0u;
+  }
+  __syncthreads();
+  if (alive) {
+    uint32_t base = s_base;
+    for (int w = 0; w < wave; ++w) base += s_n[w];
+    out[base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = i;
   }
 }
 
@@ -232,11 +270,17 @@ int sky_bias_walk_online(sky_graph* g, float p, float q, const uint32_t* seeds, 
   BIAS_TRY(view_of(g, &v));
   sky_walker_state* states = nullptr;
   unsigned long long* d_sampled = nullptr;
+  uint32_t *lists = nullptr, *counts = nullptr, *report = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
   auto body = [&]() -> int {
     BIAS_TRY(sky_device_malloc((size_t)N * sizeof(sky_walker_state) + 16, (void**)&states));
     BIAS_TRY(sky_device_malloc(8, (void**)&d_sampled));
     BIAS_HIP(hipMemsetAsync(d_sampled, 0, 8, nullptr));
+    BIAS_TRY(sky_device_malloc((size_t)2 * N * 4 + 16, (void**)&lists));
+    BIAS_TRY(sky_device_malloc(((size_t)len + 2) * 4, (void**)&counts));
+    BIAS_HIP(hipMemsetAsync(counts, 0, ((size_t)len + 2) * 4, nullptr));
+    BIAS_HIP(hipHostMalloc((void**)&report, ((size_t)len + 1) * 4, hipHostMallocDefault));
+    for (uint32_t k = 0; k <= len; ++k) report[k] = 0xFFFFFFFFu;  // "not reported yet"
     BIAS_HIP(hipEventCreate(&e0));
     BIAS_HIP(hipEventCreate(&e1));
     BIAS_HIP(hipEventRecord(e0, nullptr));
@@ -244,9 +288,24 @@ int sky_bias_walk_online(sky_graph* g, float p, float q, const uint32_t* seeds, 
       const uint32_t blocks = (N + 255) / 256;
       hipLaunchKernelGGL(bias_init_kernel, dim3(blocks), dim3(256), 0, nullptr, seeds, N, len, v.V, p, q, paths,
                          lengths, states);
-      for (uint32_t s = 0; s < len; ++s)
-        hipLaunchKernelGGL(bias_step_kernel, dim3(N), dim3(sky::N2V_T), 0, nullptr, v, len, s, stop_prob, philox_seed,
-                           paths, lengths, states);
+      // A step launches workgroups for the walkers that still walk, not for all N: after every step the survivors
+      // are appended to a list the next step reads (the reference's walker queue, include/sampler_result.cuh:646-669).
+      // The list's length stays on the device; the host sizes the next launches from the lengths that have come back
+      // so far through pinned memory (they can only shrink), reads them without waiting, and stops once one is 0.
+      uint32_t upper = N;
+      for (uint32_t s = 0; s < len && upper; ++s) {
+        const uint32_t* in = s ? lists + (size_t)((s - 1) & 1) * N : nullptr;
+        uint32_t* out = lists + (size_t)(s & 1) * N;
+        hipLaunchKernelGGL(bias_step_kernel, dim3(upper), dim3(sky::N2V_T), 0, nullptr, v, len, s, stop_prob, philox_seed,
+                           in, s ? counts + s : nullptr, paths, lengths, states);
+        hipLaunchKernelGGL(bias_compact_kernel, dim3((upper + 1023) / 1024), dim3(1024), 0, nullptr, in,
+                           s ? counts + s : nullptr, N, lengths, len, out, counts + s + 1);
+        BIAS_HIP(hipMemcpyAsync(&report[s], counts + s + 1, 4, hipMemcpyDeviceToHost, nullptr));
+        for (uint32_t k = 0; k <= s; ++k) {
+          const uint32_t seen = *(volatile uint32_t*)&report[k];
+          if (seen != 0xFFFFFFFFu && seen < upper) upper = seen;
+        }
+      }
       hipLaunchKernelGGL(bias_sum_kernel, dim3(blocks < 1024 ? blocks : 1024), dim3(256), 0, nullptr, lengths, N,
                          d_sampled);
     }
@@ -266,6 +325,9 @@ int sky_bias_walk_online(sky_graph* g, float p, float q, const uint32_t* seeds, 
   if (e1) (void)hipEventDestroy(e1);
   if (states) (void)sky_device_free(states);
   if (d_sampled) (void)sky_device_free(d_sampled);
+  if (lists) (void)sky_device_free(lists);
+  if (counts) (void)sky_device_free(counts);
+  if (report) (void)hipHostFree(report);
   return rc;
 }
 
