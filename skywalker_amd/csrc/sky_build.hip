@@ -1453,14 +1453,23 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
-  SKY_TRY(grp(CLS_G2, build_group_kernel<2, 4>, 2, "g2"));
-  SKY_TRY(grp(CLS_G4, build_group_kernel<4, 4>, 4, "g4"));
-  SKY_TRY(grp(CLS_G8, build_group_kernel<8, 4>, 8, "g8"));
-  SKY_TRY(grp(CLS_G16, build_group_kernel<16, 4>, 16, "g16"));
-  SKY_TRY(grp(CLS_G32, build_group_kernel<32, 4>, 32, "g32"));
-  SKY_TRY(grp(CLS_G32S, build_group_kernel<32, 5>, 32, "g32s"));
-  SKY_TRY(grp(CLS_G32X, build_group_kernel<32, 6>, 32, "g32x"));
-
+  const bool row_merge = option(g, OPT_ROW_MERGE) != 0;
+  // Rows of 5118..STREAM_MAX_DEG entries: one workgroup streams a row.  A small streaming class is not worth its
+  // own launch (too few workgroups to fill the GPU): its rows then go to the tile-parallel path together with the
+  // HUGE class.  The rows above 65533 entries keep one workgroup busy for up to 1.5 ms; they join the launch (and
+  // start first) only when it holds enough other rows to run that long anyway, else they are built tile by tile.
+  // The lists lie back to back: STREAM, STREAM_LAST, STREAM_WIDE, HUGE.
+  const uint32_t narrow_rows = counts[CLS_STREAM] + counts[CLS_STREAM_LAST];
+  const uint64_t narrow_edges = host.edges[CLS_STREAM] + host.edges[CLS_STREAM_LAST];
+  const uint64_t all_stream_edges = narrow_edges + host.edges[CLS_STREAM_WIDE];
+  const bool stream_to_tiled = !row_merge || all_stream_edges <= (uint64_t)option(g, OPT_STREAM_MIN_EDGES);
+  const bool wide_streamed = !stream_to_tiled && all_stream_edges >= (uint64_t)option(g, OPT_STREAM_WIDE_MIN_EDGES);
+  const uint32_t wide_rows = wide_streamed ? counts[CLS_STREAM_WIDE] : 0;
+  if (!stream_to_tiled && narrow_rows + wide_rows) {
+    StreamSwap sw(g, fan.next());
+    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], wide_rows, vlist + starts[CLS_STREAM], narrow_rows));
+    if (tm) SKY_TRY(tm->mark("stream", narrow_edges + (wide_streamed ? host.edges[CLS_STREAM_WIDE] : 0)));
+  }
   auto lds = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
     const uint32_t cnt = counts[cls];
     if (cnt) {
@@ -1480,7 +1489,6 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
   static const char* const mw_name[9] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9", "mw10"};
-  const bool row_merge = option(g, OPT_ROW_MERGE) != 0;
   if (row_merge) {
     SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 4>, 64, 4, "lds_w1"));
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 8>, 64, 8, "lds_w2"));
@@ -1520,22 +1528,14 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     }
   }
 
-  // Rows of 5118..STREAM_MAX_DEG entries: one workgroup streams a row.  A small streaming class is not worth its
-  // own launch (too few workgroups to fill the GPU): its rows then go to the tile-parallel path together with the
-  // HUGE class.  The rows above 65533 entries keep one workgroup busy for up to 1.5 ms; they join the launch (and
-  // start first) only when it holds enough other rows to run that long anyway, else they are built tile by tile.
-  // The lists lie back to back: STREAM, STREAM_LAST, STREAM_WIDE, HUGE.
-  const uint32_t narrow_rows = counts[CLS_STREAM] + counts[CLS_STREAM_LAST];
-  const uint64_t narrow_edges = host.edges[CLS_STREAM] + host.edges[CLS_STREAM_LAST];
-  const uint64_t all_stream_edges = narrow_edges + host.edges[CLS_STREAM_WIDE];
-  const bool stream_to_tiled = !row_merge || all_stream_edges <= (uint64_t)option(g, OPT_STREAM_MIN_EDGES);
-  const bool wide_streamed = !stream_to_tiled && all_stream_edges >= (uint64_t)option(g, OPT_STREAM_WIDE_MIN_EDGES);
-  const uint32_t wide_rows = wide_streamed ? counts[CLS_STREAM_WIDE] : 0;
-  if (!stream_to_tiled && narrow_rows + wide_rows) {
-    StreamSwap sw(g, fan.next());
-    SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], wide_rows, vlist + starts[CLS_STREAM], narrow_rows));
-    if (tm) SKY_TRY(tm->mark("stream", narrow_edges + (wide_streamed ? host.edges[CLS_STREAM_WIDE] : 0)));
-  }
+  SKY_TRY(grp(CLS_G2, build_group_kernel<2, 4>, 2, "g2"));
+  SKY_TRY(grp(CLS_G4, build_group_kernel<4, 4>, 4, "g4"));
+  SKY_TRY(grp(CLS_G8, build_group_kernel<8, 4>, 8, "g8"));
+  SKY_TRY(grp(CLS_G16, build_group_kernel<16, 4>, 16, "g16"));
+  SKY_TRY(grp(CLS_G32, build_group_kernel<32, 4>, 32, "g32"));
+  SKY_TRY(grp(CLS_G32S, build_group_kernel<32, 5>, 32, "g32s"));
+  SKY_TRY(grp(CLS_G32X, build_group_kernel<32, 6>, 32, "g32x"));
+
   const uint32_t tiled_rows = counts[CLS_HUGE] + (wide_streamed ? 0 : counts[CLS_STREAM_WIDE]) + (stream_to_tiled ? narrow_rows : 0);
   const uint64_t tiled_edges =
       host.edges[CLS_HUGE] + (wide_streamed ? 0 : host.edges[CLS_STREAM_WIDE]) + (stream_to_tiled ? narrow_edges : 0);
