@@ -30,6 +30,25 @@ static int ensure_device() {
 
 using namespace sky;
 
+namespace {
+// The table as two arrays and back, on the device: a host loop over a table of a billion entries takes seconds.
+__global__ __launch_bounds__(256) void split_table_kernel(const sky::AliasEntry* __restrict__ table, size_t lo, size_t n,
+                                                          float* __restrict__ prob, uint32_t* __restrict__ alias) {
+  const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+  if (i >= n) return;
+  const sky::AliasEntry e = table[lo + i];
+  prob[i] = e.prob;
+  alias[i] = e.alias;
+}
+__global__ __launch_bounds__(256) void join_table_kernel(const float* __restrict__ prob, const uint32_t* __restrict__ alias,
+                                                         size_t lo, size_t n, sky::AliasEntry* __restrict__ table) {
+  const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+  if (i >= n) return;
+  table[lo + i] = sky::AliasEntry{prob[i], alias[i]};
+}
+constexpr size_t TABLE_PIECE = 64u << 20;  // entries moved per round: 512 MB of staging on the device
+}  // namespace
+
 namespace sky {
 // process-wide values of the tuning knobs, in the order of SkyOpt (sky_set_option changes them)
 long long g_option_value[OPT_COUNT] = {
@@ -277,12 +296,25 @@ int sky_alias_download(const sky_graph* g, float* prob, uint32_t* alias, int8_t*
   if (!g) return fail(SKY_ERR_ARG, "sky_alias_download: null graph");
   if (!g->has_tables) return fail(SKY_ERR_STATE, "sky_alias_download: tables have not been built");
   if ((prob || alias) && g->E) {
-    std::vector<AliasEntry> host(g->E);
-    SKY_HIP(hipMemcpy(host.data(), g->table, (size_t)g->E * sizeof(AliasEntry), hipMemcpyDeviceToHost));
-    for (size_t i = 0; i < g->E; ++i) {
-      if (prob) prob[i] = host[i].prob;
-      if (alias) alias[i] = host[i].alias;
+    const size_t piece = std::min<size_t>(g->E, TABLE_PIECE);
+    float* d_prob = nullptr;
+    uint32_t* d_alias = nullptr;
+    SKY_HIP(hipMalloc((void**)&d_prob, piece * 4));
+    if (hipMalloc((void**)&d_alias, piece * 4) != hipSuccess) {
+      (void)hipFree(d_prob);
+      return fail(SKY_ERR_HIP, "sky_alias_download: no device memory for the staging arrays");
     }
+    int rc = SKY_OK;
+    for (size_t lo = 0; lo < g->E && rc == SKY_OK; lo += piece) {
+      const size_t n = std::min(piece, (size_t)g->E - lo);
+      hipLaunchKernelGGL(split_table_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, g->stream, g->table, lo, n,
+                         d_prob, d_alias);
+      if (prob && hipMemcpy(prob + lo, d_prob, n * 4, hipMemcpyDeviceToHost) != hipSuccess) rc = SKY_ERR_HIP;
+      if (alias && hipMemcpy(alias + lo, d_alias, n * 4, hipMemcpyDeviceToHost) != hipSuccess) rc = SKY_ERR_HIP;
+    }
+    (void)hipFree(d_prob);
+    (void)hipFree(d_alias);
+    if (rc != SKY_OK) return fail(rc, "sky_alias_download: copy to host failed");
   }
   if (valid && g->V) SKY_HIP(hipMemcpy(valid, g->valid, (size_t)g->V, hipMemcpyDeviceToHost));
   return SKY_OK;
@@ -322,9 +354,28 @@ int sky_alias_upload(sky_graph* g, const float* prob, const uint32_t* alias, con
   if (!g->table) SKY_TRY(alloc_padded(&g->table, (size_t)g->E));
   if (!g->valid) SKY_TRY(alloc_padded(&g->valid, (size_t)g->V));
   if (g->E) {
-    std::vector<AliasEntry> host(g->E);
-    for (size_t i = 0; i < g->E; ++i) host[i] = AliasEntry{prob[i], alias[i]};
-    SKY_HIP(hipMemcpy(g->table, host.data(), (size_t)g->E * sizeof(AliasEntry), hipMemcpyHostToDevice));
+    const size_t piece = std::min<size_t>(g->E, TABLE_PIECE);
+    float* d_prob = nullptr;
+    uint32_t* d_alias = nullptr;
+    SKY_HIP(hipMalloc((void**)&d_prob, piece * 4));
+    if (hipMalloc((void**)&d_alias, piece * 4) != hipSuccess) {
+      (void)hipFree(d_prob);
+      return fail(SKY_ERR_HIP, "sky_alias_upload: no device memory for the staging arrays");
+    }
+    int rc = SKY_OK;
+    for (size_t lo = 0; lo < g->E && rc == SKY_OK; lo += piece) {
+      const size_t n = std::min(piece, (size_t)g->E - lo);
+      if (hipMemcpy(d_prob, prob + lo, n * 4, hipMemcpyHostToDevice) != hipSuccess ||
+          hipMemcpy(d_alias, alias + lo, n * 4, hipMemcpyHostToDevice) != hipSuccess)
+        rc = SKY_ERR_HIP;
+      else
+        hipLaunchKernelGGL(join_table_kernel, dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, g->stream, d_prob, d_alias, lo,
+                           n, g->table);
+    }
+    if (rc == SKY_OK && hipStreamSynchronize(g->stream) != hipSuccess) rc = SKY_ERR_HIP;
+    (void)hipFree(d_prob);
+    (void)hipFree(d_alias);
+    if (rc != SKY_OK) return fail(rc, "sky_alias_upload: copy to the device failed");
   }
   if (g->V) SKY_HIP(hipMemcpy(g->valid, valid, (size_t)g->V, hipMemcpyHostToDevice));
   g->has_tables = true;
