@@ -39,7 +39,7 @@ CONFIGS = {
 # degree ranges of the build's classes (skywalker_amd/csrc/sky_build.hip, degree_class)
 CLASS_RANGES = ([(1, 2), (3, 8), (9, 16), (17, 32), (33, 64), (65, 128), (129, 160), (161, 192), (193, 253), (254, 509)] +
                 [(512 * (nw - 1) - 2, 512 * nw - 3) for nw in range(2, 11)] +
-                [(5118, 24576), (24577, 65533), (65534, 524287), (524288, 1200000)])
+                [(5118, 8189), (8190, 24576), (24577, 65533), (65534, 524287), (524288, 1200000)])
 
 
 def class_degrees(per_class, seed):
@@ -71,7 +71,7 @@ KERNEL_OF = {  # build_profile entry -> kernel symbol
     "lds_w2": "build_merge_kernel<64,8>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
-    "streamed": "huge_prefix_kernel+build_huge_kernel", "stream": "build_stream_kernel",
+    "streamed": "huge_prefix_kernel+build_huge_kernel", "stream": "build_stream_kernel", "hold": "build_hold_kernel",
 }
 KERNEL_OF.update({"g%d%s" % (g, x): "build_group_kernel<%d,%d>" % (g, 6 if x else 4)
                   for g in (2, 4, 8, 16, 32) for x in ("", "x")})

@@ -224,13 +224,14 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
  *      built tile by tile (1024 entries per tile) up to this many tiles (default: no limit); longer rows
  *      fall to a kernel in which one workgroup walks the whole row.  Tests lower it to exercise that kernel.
  *      "row_merge" (default 1): rows of 62..5117 entries pair lights and heavies by a merge of their prefix
- *      sums; 0 selects the kernel that does one binary search per entry.  Both give the same table.
- *      "stream_min_edges" (default 4000000): rows of 5118..524287 entries have a kernel of their own (one workgroup
+ *      sums, rows of 5118..8189 entries are held by one workgroup; 0 selects the kernel that does one binary search per
+ *      entry (the tile-parallel path from 4094 entries on).  Both give the same table.
+ *      "stream_min_edges" (default 4000000): rows of 8190..524287 entries have a kernel of their own (one workgroup
  *      streams a row); when a build holds no more than this many entries in such rows, too few to fill the GPU
  *      with one workgroup each, they go to the tile-parallel path instead.  Tests set 0.
  *      "stream_wide_min_edges" (default 134217216): the rows of more than 65533 entries among them keep a workgroup
  *      busy for up to 1.5 ms; they join that kernel only when the build holds at least this many entries in rows
- *      of 5118..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
+ *      of 8190..524287 entries (the launch then runs that long anyway), else they are built tile by tile.  Tests set 0.
  *      "walk_read_once" (default -1): 1 makes the walks load a step's table entry and neighbour id as read-once
  *      data, which keeps the row offsets of the well-connected vertices in L2 on a graph whose tables are far larger
  *      than the caches; 0 loads them as ordinary data (better when the tables fit the caches); -1 decides by the size of

@@ -47,10 +47,11 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 253) return CLS_LDS_W1;
   if (d <= 509) return CLS_LDS_W2;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
-  // Longer rows stream through one workgroup: the arrays of a row of more than 5117 entries leave room for one
-  // workgroup per CU only (14 bytes of LDS per slot), and wavefronts that all wait at the same barriers ran such
-  // rows at 1.6 TB/s where the streaming kernel reaches 2.5.
+  // The arrays of a longer row (14 bytes of LDS per slot) would leave room for one workgroup per CU only: such a row
+  // keeps its heavies alone in LDS, and its entries in registers as long as 512 threads can hold them (1024 threads
+  // for rows of up to 16381 entries, one workgroup per CU, ran at 1.7 TB/s where the streaming kernel reaches 1.95).
   if (nw <= MERGE_MAX_NW) return CLS_MW2 + (int)nw - 2;
+  if (d <= HOLD_MAX_DEG) return CLS_HOLD;
   if (d > STREAM_MAX_DEG) return CLS_HUGE;
   if (d > 65533u) return CLS_STREAM_WIDE;
   return d > 24576u ? CLS_STREAM : CLS_STREAM_LAST;
@@ -1454,7 +1455,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
   };
   const bool row_merge = option(g, OPT_ROW_MERGE) != 0;
-  // Rows of 5118..STREAM_MAX_DEG entries: one workgroup streams a row.  A small streaming class is not worth its
+  // Rows of 8190..STREAM_MAX_DEG entries: one workgroup streams a row.  A small streaming class is not worth its
   // own launch (too few workgroups to fill the GPU): its rows then go to the tile-parallel path together with the
   // HUGE class.  The rows above 65533 entries keep one workgroup busy for up to 1.5 ms; they join the launch (and
   // start first) only when it holds enough other rows to run that long anyway, else they are built tile by tile.
@@ -1469,6 +1470,14 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     StreamSwap sw(g, fan.next());
     SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], wide_rows, vlist + starts[CLS_STREAM], narrow_rows));
     if (tm) SKY_TRY(tm->mark("stream", narrow_edges + (wide_streamed ? host.edges[CLS_STREAM_WIDE] : 0)));
+  }
+  // Rows of 5118..8189 entries: one workgroup holds the row (without row_merge they are built tile by tile).
+  if (row_merge && counts[CLS_HOLD]) {
+    {
+      StreamSwap sw(g, fan.next());
+      SKY_TRY(build_rows_hold(g, vlist + starts[CLS_HOLD], counts[CLS_HOLD], nullptr, 0));
+    }
+    if (tm) SKY_TRY(tm->mark("hold", host.edges[CLS_HOLD]));
   }
   auto lds = [&](int cls, auto kernel, int rowt, int t, const char* name) -> int {
     const uint32_t cnt = counts[cls];
@@ -1536,11 +1545,16 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   SKY_TRY(grp(CLS_G32S, build_group_kernel<32, 5>, 32, "g32s"));
   SKY_TRY(grp(CLS_G32X, build_group_kernel<32, 6>, 32, "g32x"));
 
-  const uint32_t tiled_rows = counts[CLS_HUGE] + (wide_streamed ? 0 : counts[CLS_STREAM_WIDE]) + (stream_to_tiled ? narrow_rows : 0);
-  const uint64_t tiled_edges =
-      host.edges[CLS_HUGE] + (wide_streamed ? 0 : host.edges[CLS_STREAM_WIDE]) + (stream_to_tiled ? narrow_edges : 0);
+  // the lists HOLD, STREAM, STREAM_LAST, STREAM_WIDE, HUGE lie back to back (the class numbers between are unused)
+  const uint32_t held_rows = row_merge ? 0 : counts[CLS_HOLD];
+  const uint32_t tiled_rows =
+      counts[CLS_HUGE] + (wide_streamed ? 0 : counts[CLS_STREAM_WIDE]) + (stream_to_tiled ? narrow_rows : 0) + held_rows;
+  const uint64_t tiled_edges = host.edges[CLS_HUGE] + (wide_streamed ? 0 : host.edges[CLS_STREAM_WIDE]) +
+                               (stream_to_tiled ? narrow_edges : 0) +
+                               (row_merge ? 0 : host.edges[CLS_HOLD]);
   const RowRef* tiled_list =
-      vlist + (stream_to_tiled ? starts[CLS_STREAM] : (wide_streamed ? starts[CLS_HUGE] : starts[CLS_STREAM_WIDE]));
+      vlist + (held_rows ? starts[CLS_HOLD]
+                         : stream_to_tiled ? starts[CLS_STREAM] : (wide_streamed ? starts[CLS_HUGE] : starts[CLS_STREAM_WIDE]));
   if (tiled_rows) {
     const uint32_t cnt = tiled_rows;
     uint32_t skipped = 0;
@@ -1648,7 +1662,7 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   // the class kernels are independent of one another: they go out in turn over the graph's stream and its side streams
   StreamFan fan(g, st);
   if (option(g, OPT_BUILD_STREAMS) && n_upper >= 4096) SKY_TRY(fan.start());
-  // Rows of 5118 entries and more first, because theirs is the longest chain of launches.  The classes STREAM,
+  // Rows of 8190 entries and more first, because theirs is the longest chain of launches.  The classes STREAM,
   // STREAM_LAST, STREAM_WIDE, HUGE lie back to back.  What the graph holds of them decides, as in a build of all
   // rows, which go to the streaming kernel (one workgroup per row) and which are built tile by tile by the whole
   // GPU: the two longest classes always are (a frontier holds a few such rows at most, and one workgroup would need
@@ -1715,10 +1729,19 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   SKY_Q(CLS_MW2 + 7, mrg(CLS_MW2 + 7, (build_merge_kernel<768, 6, 4, 1>), 768, 6));
   SKY_Q(CLS_MW2 + 8, mrg(CLS_MW2 + 8, (build_merge_kernel<512, 10, 4, 1>), 512, 10));
 #undef SKY_MW
+  auto hold = [&](int cls) -> int {
+    const uint32_t rows = rows_of(cls);
+    if (!rows) return SKY_OK;
+    StreamSwap sw(g, fan.next());
+    return build_rows_hold(g, vlist, rows, dev, cls);
+  };
+  int hold_rc = SKY_OK;
+  SKY_Q(CLS_HOLD, { const int rc = hold(CLS_HOLD); if (rc != SKY_OK) hold_rc = rc; });
 #undef SKY_Q
   std::stable_sort(queue.begin(), queue.end(), [](const auto& a, const auto& b) { return a.first > b.first; });
   for (auto& q : queue) q.second();
   SKY_TRY(fan.join());
+  if (hold_rc != SKY_OK) return hold_rc;
   SKY_HIP(hipGetLastError());
   return SKY_OK;
 }

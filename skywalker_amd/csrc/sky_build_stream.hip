@@ -1,5 +1,6 @@
-// Alias tables of rows of 5118..524287 entries: one workgroup streams the row and keeps a window of
-// the row's heavies in LDS.
+// Alias tables of rows of 8190..524287 entries: one workgroup streams the row and keeps a window of
+// the row's heavies in LDS.  (Rows of 5118..8189 entries: build_hold_kernel at the end of this file, which keeps
+// the row itself in registers.)
 //
 // The table is the same pure function of the weights as everywhere else (see sky_build.hip).
 // Only the heavies of a row need random access: a light's alias is the first heavy whose surplus
@@ -560,7 +561,303 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
   }  // rows of this workgroup
 }
 
-// Builds the n_first rows of `first_list` and the n rows of `rows_list` (5118..STREAM_MAX_DEG entries each) in one
+// ---------------------------------------------------------------- rows held in registers
+// Rows of 5118..8189 entries: one workgroup of 512 threads holds the whole row, 16 consecutive slots per thread, so
+// the weights are read once and every entry is classified once.  As in the streaming kernel only the heavies go to
+// LDS, {surplus prefix, slot, residual} of each in slot order, 14 bytes; a thread knows the rank and the surplus
+// prefix of its own heavies from one scan over the workgroup, so the list needs no second pass.  Then one list
+// search per thread, its lights walk the list from there and leave the residual of every heavy they finish in the
+// list; after a barrier every thread completes its own heavies from the list and writes its 16 entries as whole
+// quads: each entry is written once.  A row with more heavies than the list holds repeats list, walk and completion
+// for the next ranks; everything it needs is still in registers.  (2.1 TB/s on such rows against 1.9 for the
+// streaming kernel.  The same with 1024 threads for rows of up to 16381 entries leaves one workgroup per CU, all
+// of whose wavefronts wait at the same barriers: 1.7 TB/s.)
+constexpr int HOLD_PER = 16;
+constexpr int HOLD_T = 512;
+constexpr uint32_t HOLD_CAP = 5632;  // heavies per list: two workgroups fill a CU's LDS
+constexpr size_t HOLD_LDS_BYTES = (size_t)(HOLD_CAP + 2) * 14;
+static_assert(HOLD_T * HOLD_PER >= HOLD_MAX_DEG + 3, "the row fits from any 16-byte phase");
+
+template <bool DEV>
+__global__ __launch_bounds__(HOLD_T, 4) void build_hold_kernel(const RowRef* __restrict__ vlist, uint32_t count,
+                                                       const uint32_t* __restrict__ dev, int cls,
+                                                       const float* __restrict__ wgt, AliasEntry* __restrict__ table,
+                                                       int8_t* __restrict__ valid) {
+  constexpr int PER = HOLD_PER, T = HOLD_T, NW = T / 64;
+  constexpr uint32_t CAPH = HOLD_CAP;
+  extern __shared__ uint64_t smem[];
+  uint64_t* s_sh = smem;                                              // [CAPH + 2] surplus prefix of the list's h-th heavy, then two sentinels
+  float* s_prob = reinterpret_cast<float*>(smem + CAPH + 2);          // [CAPH + 2] its residual probability
+  uint16_t* s_slot = reinterpret_cast<uint16_t*>(s_prob + CAPH + 2);  // [CAPH + 2] its slot; after them the slot lights beyond the list take
+  __shared__ WSum3 s_wsum[NW];
+  __shared__ double s_fsum[NW];
+  __shared__ uint32_t s_mn[NW];
+  __shared__ uint64_t s_ex[3 * NW];
+
+  uint32_t start = 0;
+  if (DEV) {  // the class's rows start after those of the classes before it; the grid is an upper bound
+    for (int c = 0; c < cls; ++c) start += dev[c];
+    count = dev[cls];
+  }
+  if (blockIdx.x >= count) return;
+  const RowRef rr = vlist[start + blockIdx.x];
+  const uint32_t d = rr.d;
+  const uint32_t base = rr.off & ~3u, lead = rr.off - base, span = lead + d;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t pos0 = (uint32_t)PER * (uint32_t)tid;
+  const bool wave_on = (uint32_t)(PER * 64 * wave) < span;
+
+  float cw[PER];
+  uint32_t live = 0;  // bit j: slot pos0 + j belongs to the row
+  double rsum = 0.0;
+  uint32_t mn = 0xFFFFFFFFu;
+  if (wave_on) {
+#pragma unroll
+    for (int q = 0; q < PER / 4; ++q) {
+      const uint32_t pos = pos0 + 4u * q;
+      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (pos < span) x = *reinterpret_cast<const float4*>(wgt + base + pos);
+      const float xs[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const bool in = pos + k - lead < d;  // one unsigned compare: slots before the row wrap around
+        if (in) live |= 1u << (q * 4 + k);
+        cw[q * 4 + k] = masked_weight(xs[k], in);
+        rsum += (double)cw[q * 4 + k];
+        mn = min(mn, __float_as_uint(cw[q * 4 + k]) - 1u);
+      }
+    }
+    rsum = group_sum_f64<64>(rsum);
+    mn = wave_min_u32(mn);
+  } else {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) cw[j] = 0.0f;
+  }
+  if (lane == 0) {
+    s_fsum[wave] = rsum;
+    s_mn[wave] = mn;
+  }
+  __syncthreads();
+  rsum = s_fsum[0];
+  mn = s_mn[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) {
+    rsum += s_fsum[i];
+    mn = min(mn, s_mn[i]);
+  }
+  if (!plain_sum_is_exact(rsum, uniform_u32(mn))) {  // uniform over the workgroup: the three-limb sum instead
+    WSum3 sum{0.0, 0.0, 0.0};
+    if (wave_on) {
+#pragma unroll
+      for (int j = 0; j < PER; ++j) wsum3_add(sum, (double)cw[j]);
+      sum = group_sum_wsum3<64>(sum);
+    }
+    if (lane == 0) s_wsum[wave] = sum;
+    __syncthreads();
+    sum = s_wsum[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) {
+      sum.top += s_wsum[i].top;
+      sum.mid += s_wsum[i].mid;
+      sum.low += s_wsum[i].low;
+    }
+    rsum = sum.top + sum.mid + sum.low != 0.0 ? wsum3_to_double(sum) : 0.0;
+  }
+  if (rsum == 0.0) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if ((live >> j) & 1) table[base + pos0 + j] = AliasEntry{0.0f, SKY_INVALID};
+    if (tid == 0) valid[rr.v] = 0;
+    return;
+  }
+  const Ledger L = make_ledger_small(d, rsum);
+  const double neg_fs = -L.fs;
+
+  // classify once: op = float(p); amt = deficit of a light, surplus of a heavy, 0 outside the row
+  float op[PER];
+  uint64_t amt[PER];
+  uint32_t heavy = 0;
+  uint64_t run_d = 0, run_u = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const bool in = (live >> j) & 1;
+    const double pj = (double)cw[j] * L.scale;
+    const double t = fma(pj, L.fs, neg_fs);  // = (pj - 1) * 2^F rounded once: the product with 2^F is exact
+    const bool hj = in && t >= 0.5;
+    const double a = fmax(fabs(t), hj ? 1.0 : 0.0);  // |t| < 0.5 for a light with t > 0: rounds to the deficit 0
+    uint64_t x;
+    if (a < 4503599627370496.0)
+      x = (uint64_t)__double_as_longlong(a + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
+    else
+      x = (uint64_t)a;  // a surplus of 2^52 units and more is an integer already
+    amt[j] = in ? x : 0;
+    op[j] = (float)pj;
+    if (hj) heavy |= 1u << j;
+    run_d += hj ? 0 : amt[j];
+    run_u += hj ? amt[j] : 0;
+  }
+  // exclusive prefixes over the workgroup of deficits, surpluses and heavy counts, and their totals
+  uint64_t ex_d, ex_u, tot_d;
+  uint32_t ex_c, nh;
+  {
+    const uint32_t c = (uint32_t)__popc(heavy);
+    const uint64_t id = group_scan_u64<64>(run_d), iu = group_scan_u64<64>(run_u);
+    const uint32_t ic = group_scan_u32<64>(c);
+    if (lane == 63) {
+      s_ex[3 * wave] = id;
+      s_ex[3 * wave + 1] = iu;
+      s_ex[3 * wave + 2] = ic;
+    }
+    __syncthreads();
+    // the wavefronts' sums, one per lane of the first row of 16 lanes, scanned there
+    uint64_t wd = 0, wu = 0;
+    uint32_t wc = 0;
+    if (lane < NW) {
+      wd = s_ex[3 * lane];
+      wu = s_ex[3 * lane + 1];
+      wc = (uint32_t)s_ex[3 * lane + 2];
+    }
+    wd = group_scan_u64<16>(wd);
+    wu = group_scan_u64<16>(wu);
+    wc = group_scan_u32<16>(wc);
+    const int prev = max(wave - 1, 0);
+    uint64_t bd = shfl_u64(wd, prev), bu = shfl_u64(wu, prev);
+    uint32_t bc = (uint32_t)__shfl((int)wc, prev, 64);
+    if (wave == 0) {
+      bd = bu = 0;
+      bc = 0;
+    }
+    tot_d = shfl_u64(wd, NW - 1);
+    nh = (uint32_t)__shfl((int)wc, NW - 1, 64);
+    ex_d = bd + id - run_d;
+    ex_u = bu + iu - run_u;
+    ex_c = bc + ic - c;
+  }
+  nh = uniform_u32(nh);
+  tot_d = uniform_u64(tot_d);
+
+  uint32_t oa[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) oa[j] = pos0 + (uint32_t)j - lead;  // a light of a row without heavies, and a heavy nobody finishes, point at themselves
+  uint64_t sh_lo = 0;  // surplus prefix of the heavies before the list
+  for (uint32_t hb = 0; hb < nh; hb += CAPH) {
+    const uint32_t nw = min(CAPH, nh - hb);
+    const bool more = hb + nw < nh;
+    const bool whole_row = hb == 0 && !more;  // the usual case: one list holds every heavy of the row
+    if (hb) __syncthreads();                  // the previous list is read until its heavies are complete
+    // ---- list: this thread's heavies of ranks [hb, hb + nw], the last one only when more follow (its slot is what
+    // the list's last heavy points at); without more, the slot after the list repeats the last heavy's
+    if (heavy) {
+      uint32_t r = ex_c - hb;
+      uint64_t su = ex_u;
+#pragma unroll
+      for (int j = 0; j < PER; ++j)
+        if ((heavy >> j) & 1) {
+          su += amt[j];
+          if (r <= nw) {  // ranks before the list wrap around
+            if (r < nw) s_sh[r] = su;
+            s_slot[r] = (uint16_t)(pos0 + j);
+            if (!more && r + 1 == nw) s_slot[nw] = (uint16_t)(pos0 + j);
+          }
+          ++r;
+        }
+    }
+    if (tid == 0) {
+      s_sh[nw] = ~0ull;
+      s_sh[nw + 1] = ~0ull;
+      s_slot[nw + 1] = 0;
+    }
+    __syncthreads();
+    const uint64_t sh_hi = uniform_u64(s_sh[nw - 1]);  // surplus prefix of the list's last heavy
+    // ---- walk: one search, then every light of this thread takes the list entry it stands at as its alias and
+    // finishes the heavies whose surplus prefix its deficit reaches
+    if (wave_on) {
+      uint64_t sl = ex_d;
+      const uint64_t k1[1] = {sl};
+      uint32_t o1[1];
+      count_le<1>(s_sh, nw, k1, o1);
+      uint32_t b = o1[0];
+      uint64_t hv = s_sh[b], hvn = s_sh[b + 1];  // ~0 once the list is exhausted
+      uint32_t hal = (uint32_t)s_slot[b] - lead, haln = (uint32_t)s_slot[b + 1] - lead;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        const bool lt = ((live & ~heavy) >> j) & 1;  // a light of the row
+        // its alias is the first heavy whose surplus prefix exceeds sl: in this list iff sh_lo <= sl < sh_hi, or
+        // beyond every heavy of the row
+        if (lt && (whole_row || (sl >= sh_lo && (sl < sh_hi || !more)))) oa[j] = hal;
+        sl += ((heavy >> j) & 1) ? 0 : amt[j];
+        if (hv <= sl) {
+          do {
+            s_prob[b] = residual_below(sl - hv);
+            ++b;
+            hv = hvn;
+            hal = haln;
+            hvn = s_sh[b + 1];
+            haln = (uint32_t)s_slot[b + 1] - lead;
+          } while (hv <= sl);
+        }
+      }
+    }
+    __syncthreads();
+    // ---- this thread's heavies of the list: {residual, next heavy} when a light reached it and it is not the row's
+    // last heavy, {1, itself} otherwise
+    if (heavy) {
+      uint32_t r = ex_c - hb;
+      uint64_t su = ex_u;
+#pragma unroll
+      for (int j = 0; j < PER; ++j)
+        if ((heavy >> j) & 1) {
+          su += amt[j];
+          if (r < nw) {
+            const bool fin = (r + 1 < nw || more) && su <= tot_d;
+            op[j] = fin ? s_prob[r] : 1.0f;
+            if (fin) oa[j] = (uint32_t)s_slot[r + 1] - lead;
+          }
+          ++r;
+        }
+    }
+    sh_lo = sh_hi;
+  }
+
+  if (pos0 < span) {
+#pragma unroll
+    for (int q = 0; q < PER / 4; ++q) {
+      const uint32_t pos = pos0 + 4u * q;
+      if (pos >= lead && pos + 4 <= span) {
+        const float p4[4] = {op[4 * q], op[4 * q + 1], op[4 * q + 2], op[4 * q + 3]};
+        const uint32_t a4[4] = {oa[4 * q], oa[4 * q + 1], oa[4 * q + 2], oa[4 * q + 3]};
+        store_entries4(table + base + pos, p4, a4);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if ((live >> (4 * q + k)) & 1) table[base + pos + k] = AliasEntry{op[4 * q + k], oa[4 * q + k]};
+      }
+    }
+  }
+}
+
+static bool g_hold_lds_enabled = false;
+// The n rows of `rows` (5118..HOLD_MAX_DEG entries each), or with `dev` the rows of class `cls` of a list whose class
+// sizes only the device knows (n is then an upper bound of their number).
+int build_rows_hold(sky_graph* g, const RowRef* rows, uint32_t n, const uint32_t* dev, int cls) {
+  if (n == 0) return SKY_OK;
+  if (!g_hold_lds_enabled) {
+    SKY_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(build_hold_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)HOLD_LDS_BYTES));
+    SKY_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(build_hold_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)HOLD_LDS_BYTES));
+    g_hold_lds_enabled = true;
+  }
+  if (dev)
+    hipLaunchKernelGGL(build_hold_kernel<true>, dim3(n), dim3(HOLD_T), HOLD_LDS_BYTES, g->stream, rows, n, dev, cls,
+                       g->adjwgt, g->table, g->valid);
+  else
+    hipLaunchKernelGGL(build_hold_kernel<false>, dim3(n), dim3(HOLD_T), HOLD_LDS_BYTES, g->stream, rows, n, dev, cls,
+                       g->adjwgt, g->table, g->valid);
+  return SKY_OK;
+}
+
+// Builds the n_first rows of `first_list` and the n rows of `rows_list` (8190..STREAM_MAX_DEG entries each) in one
 // launch that starts with the former.
 int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n) {
   if (n + n_first == 0) return SKY_OK;

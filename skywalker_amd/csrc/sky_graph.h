@@ -99,9 +99,10 @@ enum BuildClass : int {
   CLS_LDS_W1 = 8,   // deg <= 253       one wavefront per row, 4 slots per lane
   CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
   CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..10 (class CLS_MW2 + nw - 2, up to 18): one workgroup per row whose
-                    //                  threads cover 512 * nw slots (the numbers 19..24 are not used)
+                    //                  threads cover 512 * nw slots (the numbers 20..24 are not used)
+  CLS_HOLD = 19,         // deg 5118..8189     one workgroup holds the row in registers, its heavies in LDS
   CLS_STREAM = 25,       // deg 24577..65533   one workgroup streams the row, a window of its heavies stays in LDS.
-  CLS_STREAM_LAST = 26,  // deg 5118..24576    Three classes built by one launch that takes the longest rows first
+  CLS_STREAM_LAST = 26,  // deg 8190..24576    Three classes built by one launch that takes the longest rows first
   CLS_STREAM_WIDE = 27,  // deg 65534..524287  and so
                     //                  does not end on its longest rows
   CLS_HUGE = 28,    // above            built tile by tile by the whole GPU
@@ -146,9 +147,11 @@ int build_rows_tiled(sky_graph* g, const RowRef* rows_list, uint32_t n, uint32_t
 int build_rows_tiled_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int cls, int ncls, uint32_t n_upper,
                          uint64_t edges_upper);
 constexpr int MERGE_MAX_NW = 10;  // rows of at most 512 * 10 - 3 = 5117 entries pair by merge in LDS
+constexpr uint32_t HOLD_MAX_DEG = 8189;  // 512 threads x 16 slots hold such a row from any 16-byte phase
 constexpr uint32_t STREAM_MAX_DEG = 524287;  // longest row of the streaming classes (one workgroup takes 1.5 ms for it)
 int build_rows_stream(sky_graph* g, const RowRef* first_list, uint32_t n_first, const RowRef* rows_list, uint32_t n);
 int build_rows_stream_dev(sky_graph* g, const RowRef* vlist, const uint32_t* dev, int ncls, uint32_t grid);
+int build_rows_hold(sky_graph* g, const RowRef* rows, uint32_t n, const uint32_t* dev, int cls);
 // Builds the rows listed in src[0 .. *n_dev) (n_dev: a device word the host never reads; n_upper: what it cannot
 // exceed) without waiting for the device at any point.  Needs the graph's class census and a longest row the
 // streaming kernel takes (build_rows_dev_possible).

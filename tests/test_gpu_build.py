@@ -11,7 +11,7 @@ TOL = 1e-6
 # degrees that straddle every dispatch class boundary of the build
 EDGE_DEGREES = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 16, 17, 22, 23, 24, 25, 28, 29, 30, 32, 33, 46, 47, 48,
                 49, 60, 61, 62, 63, 64, 65, 66, 67, 68, 94, 95, 96, 97, 124, 125, 126, 127, 190, 191, 192, 193, 253, 254, 255, 256, 257, 1021,
-                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 5116, 5117, 5118, 5119, 5120, 5121, 8189, 8190, 8191, 8192, 8193, 20000, 70001, 128, 129, 130, 144, 145, 159, 160, 161, 162, 34, 35, 36, 45]
+                1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 5116, 5117, 5118, 5119, 5120, 5121, 8189, 8190, 8191, 8192, 8193, 16380, 16381, 16382, 16383, 20000, 70001, 128, 129, 130, 144, 145, 159, 160, 161, 162, 34, 35, 36, 45]
 
 
 def build_and_compare(orc, xadj, adjncy, w, label):
@@ -208,11 +208,13 @@ def test_search_variant_of_the_row_kernels_gives_the_same_table(orc):
 
 @pytest.mark.parametrize("dist", ["lognormal2", "uniform", "nearequal", "sparse", "fewlights", "fewheavies"])
 def test_rows_streamed_by_one_workgroup(orc, dist):
-    # rows of 5118..524287 entries: a window of 5080 heavies kept in LDS ("fewlights" and "uniform" have rows with
-    # many windows, "nearequal" rows without a heavy); 524288 is the first degree of the tile-parallel class
+    # rows of 5118..8189 entries are held by one workgroup, its heavies listed in LDS (5632 at a time), rows of
+    # 8190..524287 entries stream through one with a window of 5080 heavies ("fewlights" has rows with several lists
+    # or windows, "uniform" too among the streamed ones, "nearequal" rows without a heavy); 524288 is the first degree
+    # of the tile-parallel class
     from helpers import weights
     rng = np.random.default_rng(31)
-    degs = [5118, 5119, 6000, 8190, 8191, 7, 8193, 12288, 2, 12289, 16385, 1, 30000, 65533, 65534, 0, 9001, 150001, 524287, 524288]
+    degs = [5118, 5119, 6000, 8189, 8190, 8191, 7, 8193, 12288, 2, 12289, 16381, 16382, 16385, 1, 30000, 65533, 65534, 0, 9001, 150001, 524287, 524288]
     xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=4096)
     if dist == "fewlights":
         w = np.where(rng.random(len(w)) < 0.01, 0.01, 1.01).astype(np.float32)
@@ -306,7 +308,7 @@ def test_random_mixtures_of_every_class(orc, seed):
     from helpers import weights
     rng = np.random.default_rng(1000 + seed)
     ends = [0, 1, 2, 3, 5, 6, 8, 9, 13, 14, 16, 17, 29, 30, 32, 33, 61, 62, 64, 65, 125, 126, 128, 129, 191, 192, 193, 253, 254,
-            509, 5117, 5118, 8190, 24576, 24577, 65533, 65534]
+            509, 5117, 5118, 8189, 8190, 16381, 16382, 24576, 24577, 65533, 65534]
     for nw in range(2, 11):
         ends += [512 * (nw - 1) - 2, 512 * nw - 3]
     degs = ends + list(rng.integers(0, 70, 3000)) + list(rng.integers(60, 600, 600)) + \
