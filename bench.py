@@ -311,6 +311,8 @@ def main():
                     help="config c4: build the second-order table of every (walker, step) instead of rejection sampling")
     ap.add_argument("--calibrate", action="store_true",
                     help="first run one plain 1 GiB copy kernel (copy_u32_kernel): known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="tuning knob of the library (sky_set_option), e.g. online_coarse_rows=65536; may be repeated")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the multi-GPU path of the reference is out of scope); "
@@ -322,6 +324,9 @@ def main():
     import numpy as np
 
     cfg = CONFIGS[args.config]
+    for opt in args.option:
+        name, value = opt.split("=", 1)
+        capi.set_option(name, int(value))
     if args.calibrate:
         words = 1 << 28
         a = capi.DeviceArray(words, np.uint32, fill=1)
