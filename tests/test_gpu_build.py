@@ -229,7 +229,7 @@ def test_special_weight_values_in_every_kind_of_row(orc):
     # NaN, infinities, negatives, -0, denormals, values at and beyond the 2^32 clamp, and values whose
     # contribution to the exact sum is only a few units of 2^-64: same bits as the oracle in every class
     rng = np.random.default_rng(41)
-    degs = [1, 2, 3, 5, 9, 20, 40, 100, 150, 200, 400, 700, 1500, 3000, 5000, 9000, 20000, 70000]
+    degs = [1, 2, 3, 5, 9, 20, 40, 100, 150, 200, 400, 700, 1500, 3000, 5000, 6000, 8189, 9000, 20000, 70000]
     xadj, adjncy, w = graph_from_degrees(degs, rng, "lognormal", V=4096)
     special = np.array([np.nan, np.inf, -np.inf, -1.0, -0.0, 0.0, 1e-45, 1e-40, 2.0 ** -64, 2.0 ** -63, 3e-19,
                         2.0 ** 32, 2.0 ** 32 * 1.5, 3e38, 2.0 ** -20, 1.0, 123456.789], np.float32)
