@@ -12,10 +12,9 @@
 //   emit     classify every entry, running deficit prefix; a light whose alias lies in the window
 //            gets its entry, and every light leaves the residual of the window's heavies that fall
 //            into its deficit interval (usually none, sometimes one) in the window; entries go out
-//            four at a time as two 16-byte stores; a heavy among them whose residual has arrived by
-//            the end of its chunk (nine in ten) leaves complete, the others carry a placeholder
-//   sweep    every other heavy of the window gets its final entry from the window: {residual, next
-//            heavy} when a light reached it and it is not the row's last heavy, {1, itself} otherwise
+//            four at a time as two 16-byte stores, heavy slots among them carry a placeholder
+//   sweep    every heavy of the window gets its final entry from the window: {residual, next heavy}
+//            when a light reached it and it is not the row's last heavy, {1, itself} otherwise
 // Rows with more heavies than one window holds repeat collect, emit and sweep: all move through
 // the row in slot order and only come back to the chunk in which the previous window ended, because
 // the alias ranks of the lights and the slots of the heavies both grow along the row.  An emit pass
@@ -434,7 +433,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       // deficit of a light of the row, 0 for any other slot
       float op[ST_PER];
       uint64_t dl[ST_PER];
-      uint32_t hmask = 0;  // bit j: slot j holds a heavy of the row
+      uint32_t nheavy = 0;
       uint64_t run = 0;
       auto classify_chunk = [&](auto edge) {
         constexpr bool EDGE = decltype(edge)::value;
@@ -451,7 +450,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
           const bool hj = lv && __float_as_uint(cw[j]) >= thr_bits;
           op[j] = hj ? -1.0f : (float)pj;
           dl[j] = (lv && !hj) ? d : 0;
-          hmask |= hj ? 1u << j : 0u;
+          nheavy += hj ? 1u : 0u;
           run += dl[j];
         }
       };
@@ -467,7 +466,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       }
       uint64_t ex_d, tot_d;
       uint32_t ex_c, tot_c;
-      stream_excl(run, (uint32_t)__popc(hmask), s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
+      stream_excl(run, nheavy, s_a[c & 1], s_c[c & 1], ex_d, ex_c, tot_d, tot_c);
       const uint32_t pos0 = c * ST_CH + (uint32_t)ST_PER * tid;
       uint32_t oa[ST_PER];
       uint32_t wr = 0;  // entries this window writes: its lights, and heavies as placeholders unless an earlier window owns them
@@ -516,27 +515,6 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
         }
         if (whole_row) wr = live;
       }
-      // Most heavies are finished by a light a few slots further on.  After a barrier the residuals that this chunk's
-      // lights have left are in the window, and a thread completes those of its own heavies whose surplus prefix lies
-      // within the deficits seen so far: their entry then leaves once, inside its quad, instead of as a placeholder
-      // now and a lone 8-byte store from the sweep later, into a line that has left L2 by then (12.2 -> 8.4 bytes
-      // written per entry, and 2 bytes fewer fetched).  The residual's sign tells the sweep (a residual is positive).
-      __syncthreads();
-      if (hmask) {
-        const uint64_t seen = carry_d + uniform_u64(tot_d);
-        uint32_t idx = carry_c + ex_c - hb;  // place in the window of this thread's first heavy (wraps for one of an earlier window)
-#pragma unroll
-        for (int j = 0; j < ST_PER; ++j)
-          if ((hmask >> j) & 1) {
-            if (idx < nw && (idx + 1 < nw || more) && s_sh[idx] <= seen) {
-              const float p = s_prob[idx];
-              op[j] = p;
-              oa[j] = s_slot[idx + 1] - r.lead;
-              s_prob[idx] = -p;
-            }
-            ++idx;
-          }
-      }
       // The weights of the next chunk, requested at the top of this iteration, are waited for here, before this
       // chunk's stores are issued: loads and stores complete in one in-order count, so a wait for the load placed
       // after the stores (at its first use in the next iteration) would wait for the stores as well.
@@ -568,9 +546,7 @@ __global__ __launch_bounds__(ST_T, 4) void build_stream_kernel(const RowRef* __r
       const uint32_t slot = s_slot[h];
       const uint32_t nxt = h + 1 < nw ? (uint32_t)s_slot[h + 1] : next_slot;
       const bool fin = nxt != NONE32 && s_sh[h] <= carry_d;
-      const float p = s_prob[h];
-      if (fin && p < 0.0f) continue;  // completed by its own thread in the emit pass
-      table[r.base + slot] = fin ? AliasEntry{p, nxt - r.lead} : AliasEntry{1.0f, slot - r.lead};
+      table[r.base + slot] = fin ? AliasEntry{s_prob[h], nxt - r.lead} : AliasEntry{1.0f, slot - r.lead};
     }
     if (!more) break;
     hb += nw;
