@@ -37,8 +37,8 @@ CONFIGS = {
                     length=80, ppr=False),
 }
 # degree ranges of the build's classes (skywalker_amd/csrc/sky_build.hip, degree_class)
-CLASS_RANGES = ([(1, 2), (3, 8), (9, 16), (17, 32), (33, 64), (65, 128), (129, 160), (161, 192), (193, 253), (254, 509)] +
-                [(512 * (nw - 1) - 2, 512 * nw - 3) for nw in range(2, 11)] +
+CLASS_RANGES = ([(1, 2), (3, 8), (9, 16), (17, 32), (33, 64), (65, 128), (129, 160), (161, 192), (193, 253), (254, 381), (382, 509), (510, 765), (766, 1021)] +
+                [(512 * (nw - 1) - 2, 512 * nw - 3) for nw in range(3, 11)] +
                 [(5118, 8189), (8190, 24576), (24577, 65533), (65534, 524287), (524288, 1200000)])
 
 
@@ -68,7 +68,7 @@ METRIC = "sampled edges/sec (SEPS) + alias-table build edges/sec on 1 MI355X; % 
 ARITHMETIC = "f64 classification and exact three-limb sums, u64 fixed-point ledger, f32 tables, u32 indices"
 KERNEL_OF = {  # build_profile entry -> kernel symbol
     "bin": "bin_count_kernel+bin_scatter_kernel", "small": "small_rows_kernel", "lds_w1": "build_merge_kernel<64,4>",
-    "lds_w2": "build_merge_kernel<64,8>",
+    "lds_w2": "build_merge_kernel<64,8>", "lds_w6": "build_merge_kernel<64,6>", "mw2_6": "build_merge_kernel<128,6>",
     "tiled_rows": "tiled_rows_kernel+tiled_map_kernel", "tiled_sum": "tiled_sum_kernel+tiled_ledger_kernel",
     "tiled_totals": "tiled_totals_kernel", "tiled_emit": "tiled_scan_kernel+tiled_emit_kernel",
     "streamed": "huge_prefix_kernel+build_huge_kernel", "stream": "build_stream_kernel", "hold": "build_hold_kernel",

@@ -45,7 +45,12 @@ __host__ __device__ __forceinline__ int degree_class(uint32_t d) {
   if (d <= 160) return CLS_G32S;
   if (d <= 192) return CLS_G32X;
   if (d <= 253) return CLS_LDS_W1;
+  // These kernels are bound by instruction issue: a row pays for the slots of its class, not for its entries.  The
+  // two classes whose rows differ most in length (by a factor of two) are halved: 6 instead of 8 slots per thread
+  // for their shorter rows.
+  if (d <= 381) return CLS_LDS_W6;
   if (d <= 509) return CLS_LDS_W2;
+  if (d <= 765) return CLS_MW2_6;
   const uint32_t nw = (d + 3 + 511) / 512;  // wavefronts of 512 slots that hold the row from any 16-byte phase
   // The arrays of a longer row (14 bytes of LDS per slot) would leave room for one workgroup per CU only: such a row
   // keeps its heavies alone in LDS, and its entries in registers as long as 512 threads can hold them (1024 threads
@@ -1500,7 +1505,9 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   static const char* const mw_name[9] = {"mw2", "mw3", "mw4", "mw5", "mw6", "mw7", "mw8", "mw9", "mw10"};
   if (row_merge) {
     SKY_TRY(mrg(CLS_LDS_W1, build_merge_kernel<64, 4>, 64, 4, "lds_w1"));
+    SKY_TRY(mrg(CLS_LDS_W6, build_merge_kernel<64, 6>, 64, 6, "lds_w6"));
     SKY_TRY(mrg(CLS_LDS_W2, build_merge_kernel<64, 8>, 64, 8, "lds_w2"));
+    SKY_TRY(mrg(CLS_MW2_6, build_merge_kernel<128, 6>, 128, 6, "mw2_6"));
 #define SKY_MW(NW) SKY_TRY(mrg(CLS_MW2 + NW - 2, build_merge_kernel<64 * NW, 8>, 64 * NW, 8, mw_name[NW - 2]))
     // Class nw holds rows that fit 512 nw slots.  Where a shape with an even number of slots per thread and a
     // multiple of 4 wavefronts covers that span exactly, it is used instead of nw wavefronts of 8 slots: every
@@ -1519,7 +1526,9 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
 #undef SKY_MW
   } else {
     SKY_TRY(lds(CLS_LDS_W1, build_lds_kernel<64, 1>, 64, 1, "lds_w1"));
+    SKY_TRY(lds(CLS_LDS_W6, build_lds_kernel<64, 2>, 64, 2, "lds_w6"));
     SKY_TRY(lds(CLS_LDS_W2, build_lds_kernel<64, 2>, 64, 2, "lds_w2"));
+    SKY_TRY(lds(CLS_MW2_6, build_lds_kernel<128, 2>, 128, 2, "mw2_6"));
     for (int nw = 2; nw <= MERGE_MAX_NW; ++nw) {
       const int cls = CLS_MW2 + nw - 2;
       if (nw <= 2) SKY_TRY(lds(cls, build_lds_kernel<128, 2>, 128, 2, mw_name[nw - 2]));
@@ -1717,7 +1726,9 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   SKY_Q(CLS_G32S, grp(CLS_G32S, (build_group_kernel<32, 5, true>), 32));
   SKY_Q(CLS_G32X, grp(CLS_G32X, (build_group_kernel<32, 6, true>), 32));
   SKY_Q(CLS_LDS_W1, mrg(CLS_LDS_W1, (build_merge_kernel<64, 4, 4, 2>), 64, 4));
+  SKY_Q(CLS_LDS_W6, mrg(CLS_LDS_W6, (build_merge_kernel<64, 6, 4, 2>), 64, 6));
   SKY_Q(CLS_LDS_W2, mrg(CLS_LDS_W2, (build_merge_kernel<64, 8, 4, 2>), 64, 8));
+  SKY_Q(CLS_MW2_6, mrg(CLS_MW2_6, (build_merge_kernel<128, 6, 4, 1>), 128, 6));
 #define SKY_MW(NW) SKY_Q(CLS_MW2 + NW - 2, mrg(CLS_MW2 + NW - 2, (build_merge_kernel<64 * NW, 8, 4, 1>), 64 * NW, 8))
   SKY_MW(2);
   SKY_Q(CLS_MW2 + 1, mrg(CLS_MW2 + 1, (build_merge_kernel<256, 6, 4, 1>), 256, 6));

@@ -97,10 +97,12 @@ enum BuildClass : int {
   CLS_G32 = 6,      // deg <= 128       32 lanes
   CLS_G32X = 7,     // deg 161..192     32 lanes, 6 slots per lane
   CLS_LDS_W1 = 8,   // deg <= 253       one wavefront per row, 4 slots per lane
-  CLS_LDS_W2 = 9,   // deg <= 509       one wavefront per row, 8 slots per lane
-  CLS_MW2 = 10,     // deg <= 512 * nw - 3, nw = 2..10 (class CLS_MW2 + nw - 2, up to 18): one workgroup per row whose
-                    //                  threads cover 512 * nw slots (the numbers 20..24 are not used)
-  CLS_HOLD = 19,         // deg 5118..8189     one workgroup holds the row in registers, its heavies in LDS
+  CLS_LDS_W2 = 9,   // deg 382..509     one wavefront per row, 8 slots per lane
+  CLS_MW2 = 10,     // deg 766.. for nw = 2, then <= 512 * nw - 3, nw = 2..10 (class CLS_MW2 + nw - 2, up to 18): one workgroup per row whose
+                    //                  threads cover 512 * nw slots (the numbers 22..24 are not used)
+  CLS_LDS_W6 = 19,  // deg 254..381     one wavefront per row, 6 slots per lane (the lower half of what CLS_LDS_W2 would hold)
+  CLS_MW2_6 = 20,   // deg 510..765     two wavefronts per row, 6 slots per lane (the lower half of what CLS_MW2 would hold)
+  CLS_HOLD = 21,         // deg 5118..8189     one workgroup holds the row in registers, its heavies in LDS
   CLS_STREAM = 25,       // deg 24577..65533   one workgroup streams the row, a window of its heavies stays in LDS.
   CLS_STREAM_LAST = 26,  // deg 8190..24576    Three classes built by one launch that takes the longest rows first
   CLS_STREAM_WIDE = 27,  // deg 65534..524287  and so

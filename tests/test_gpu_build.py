@@ -10,7 +10,7 @@ TOL = 1e-6
 
 # degrees that straddle every dispatch class boundary of the build
 EDGE_DEGREES = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 16, 17, 22, 23, 24, 25, 28, 29, 30, 32, 33, 46, 47, 48,
-                49, 60, 61, 62, 63, 64, 65, 66, 67, 68, 94, 95, 96, 97, 124, 125, 126, 127, 190, 191, 192, 193, 253, 254, 255, 256, 257, 1021,
+                49, 60, 61, 62, 63, 64, 65, 66, 67, 68, 94, 95, 96, 97, 124, 125, 126, 127, 190, 191, 192, 193, 253, 254, 255, 256, 257, 380, 381, 382, 383, 509, 510, 511, 764, 765, 766, 767, 1021,
                 1022, 1023, 1024, 1025, 4093, 4094, 4095, 4096, 4097, 5116, 5117, 5118, 5119, 5120, 5121, 8189, 8190, 8191, 8192, 8193, 16380, 16381, 16382, 16383, 20000, 70001, 128, 129, 130, 144, 145, 159, 160, 161, 162, 34, 35, 36, 45]
 
 
@@ -308,7 +308,7 @@ def test_random_mixtures_of_every_class(orc, seed):
     from helpers import weights
     rng = np.random.default_rng(1000 + seed)
     ends = [0, 1, 2, 3, 5, 6, 8, 9, 13, 14, 16, 17, 29, 30, 32, 33, 61, 62, 64, 65, 125, 126, 128, 129, 191, 192, 193, 253, 254,
-            509, 5117, 5118, 8189, 8190, 16381, 16382, 24576, 24577, 65533, 65534]
+            381, 382, 509, 510, 765, 766, 5117, 5118, 8189, 8190, 16381, 16382, 24576, 24577, 65533, 65534]
     for nw in range(2, 11):
         ends += [512 * (nw - 1) - 2, 512 * nw - 3]
     degs = ends + list(rng.integers(0, 70, 3000)) + list(rng.integers(60, 600, 600)) + \
