@@ -223,7 +223,7 @@ int sky_philox_selftest(const uint32_t* ctr_host, const uint32_t* key_host, uint
 /* ---- tuning knobs (no counterpart in the reference).  "tiled_max_tiles": rows too long for one workgroup are
  *      built tile by tile (1024 entries per tile) up to this many tiles (default: no limit); longer rows
  *      fall to a kernel in which one workgroup walks the whole row.  Tests lower it to exercise that kernel.
- *      "row_merge" (default 1): rows of 62..5117 entries pair lights and heavies by a merge of their prefix
+ *      "row_merge" (default 1): rows of 193..5117 entries pair lights and heavies by a merge of their prefix
  *      sums, rows of 5118..8189 entries are held by one workgroup; 0 selects the kernel that does one binary search per
  *      entry (the tile-parallel path from 4094 entries on).  Both give the same table.
  *      "stream_min_edges" (default 4000000): rows of 8190..524287 entries have a kernel of their own (one workgroup
