@@ -63,7 +63,9 @@ const char* sky_last_error(void);
 const char* sky_version(void);
 
 /* ---- device memory helpers (replace the cudaMalloc/cudaMemcpy calls scattered through
- *      include/sampler_result.cuh:490-566 and include/gpu_graph.cuh:68-117) ---- */
+ *      include/sampler_result.cuh:490-566 and include/gpu_graph.cuh:68-117).  sky_device_malloc allocates 16 bytes
+ *      more than asked for: the build kernels read weights as whole 16-byte vectors, and an array from here can be
+ *      handed to them where it lies ---- */
 int sky_device_malloc(size_t bytes, void** out);
 int sky_device_free(void* p);
 int sky_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
@@ -202,8 +204,9 @@ int sky_sample_online(sky_graph* g, const uint32_t* seeds_device, uint32_t N, co
  *                  ids in *list_device, their number in the device word *count_device (the host is not told it),
  *                  at most *upper of them
  *        hop       builds those rows from weights_device (E floats in CSR slot order, of which only the slots of
- *                  the listed rows are read; one allocation with 16 readable bytes after them; NULL: the graph's own
- *                  weights), then draws the children of `hop`
+ *                  the listed rows are read; an array whose allocation does not hold 16 more bytes, which
+ *                  sky_device_malloc always adds, is copied first, as in sky_alias_build_from_weights; NULL: the
+ *                  graph's own weights), then draws the children of `hop`
  *        end       sampled edges and kernel-region seconds; frees the session
  *      Calls come in that order, frontier and hop once per hop, on one host thread.  Results are those of
  *      sky_sample_online on a graph whose weights are the ones supplied. ---- */

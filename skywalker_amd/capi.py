@@ -271,6 +271,31 @@ class Graph:
         """OnlineGBSampleNew."""
         return self._sample(lib().sky_sample_online, seeds, fanout, seed, out)
 
+    def sample_session(self, seeds, fanout, seed, weights_of_hop=None):
+        """sky_sample_session_*: online k-hop sampling one hop at a time.  weights_of_hop(hop, frontier_upper) returns
+        the DeviceArray of E weights (16 spare bytes, as DeviceArray gives them) from which that hop's frontier rows are
+        built, or None for the graph's own."""
+        seeds_d = seeds if isinstance(seeds, DeviceArray) else DeviceArray.from_host(np.asarray(seeds, np.uint32))
+        N = seeds_d.count
+        fan = np.asarray(fanout, np.uint32)
+        lps, slen = sample_layout(fan)
+        data = DeviceArray(N * lps, np.uint32, fill=FILL)
+        sl = DeviceArray(N * slen, np.uint32, fill=0)
+        sess = C.c_void_p()
+        _ck(lib().sky_sample_session_begin(self.h, seeds_d.ptr, C.c_uint32(N), _p(fan), C.c_uint32(len(fan)),
+                                           C.c_uint64(seed), data.ptr, sl.ptr, C.byref(sess)))
+        try:
+            for hop in range(len(fan) - 1):
+                lst, cnt, upper = C.c_void_p(), C.c_void_p(), C.c_uint32(0)
+                _ck(lib().sky_sample_session_frontier(sess, C.c_uint32(hop), C.byref(lst), C.byref(cnt), C.byref(upper)))
+                w = weights_of_hop(hop, upper.value) if weights_of_hop else None
+                _ck(lib().sky_sample_session_hop(sess, C.c_uint32(hop), w.ptr if w is not None else None))
+        finally:
+            sampled, sec = C.c_uint64(0), C.c_double(0)
+            rc = lib().sky_sample_session_end(sess, C.byref(sampled), C.byref(sec))
+        _ck(rc)
+        return data, sl, sampled.value, sec.value
+
     def set_option(self, name, value):
         """A tuning knob for this graph alone (None: back to the process-wide value)."""
         if value is None:

@@ -75,7 +75,7 @@ const char* sky_version(void) { return "skywalker_hip 0.1 (gfx950)"; }
 int sky_device_malloc(size_t bytes, void** out) {
   if (!out) return fail(SKY_ERR_ARG, "sky_device_malloc: null output");
   SKY_TRY(ensure_device());
-  SKY_HIP(hipMalloc(out, bytes ? bytes : 16));
+  SKY_HIP(hipMalloc(out, bytes + 16));  // 16 spare bytes, as every array of the library has: kernels read whole vectors
   return SKY_OK;
 }
 int sky_device_free(void* p) {
@@ -264,6 +264,23 @@ static bool padded_allocation(const void* p, size_t bytes) {
   return before <= asize && asize - before >= bytes + 16;
 }
 
+// A caller's array of E weights as the build kernels can read it: the array itself when its allocation is known to
+// hold 16 more bytes, else a copy in a padded array that stays with the graph.
+static int readable_weights(sky_graph* g, const float* weights_device, const float** use) {
+  *use = weights_device;
+  if (!g->E || !weights_device || padded_allocation(weights_device, (size_t)g->E * 4)) return SKY_OK;
+  if (g->wgt_copy_cap < g->E) {
+    if (g->wgt_copy) SKY_HIP(hipFree(g->wgt_copy));
+    g->wgt_copy = nullptr;
+    g->wgt_copy_cap = 0;
+    SKY_TRY(alloc_padded(&g->wgt_copy, (size_t)g->E));
+    g->wgt_copy_cap = g->E;
+  }
+  SKY_HIP(hipMemcpyAsync(g->wgt_copy, weights_device, (size_t)g->E * 4, hipMemcpyDeviceToDevice, g->stream));
+  *use = g->wgt_copy;
+  return SKY_OK;
+}
+
 int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, double* seconds) {
   if (!g) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null graph");
   if (g->E && !weights_device) return fail(SKY_ERR_ARG, "sky_alias_build_from_weights: null weights");
@@ -271,20 +288,7 @@ int sky_alias_build_from_weights(sky_graph* g, const float* weights_device, doub
   // caller's array is used where it lies only when its allocation is known to hold those bytes; otherwise the
   // weights are copied into a padded array that stays with the graph.
   const float* use = weights_device;
-  if (g->E) {
-    const bool padded = padded_allocation(weights_device, (size_t)g->E * 4);
-    if (!padded) {
-      if (g->wgt_copy_cap < g->E) {
-        if (g->wgt_copy) SKY_HIP(hipFree(g->wgt_copy));
-        g->wgt_copy = nullptr;
-        g->wgt_copy_cap = 0;
-        SKY_TRY(alloc_padded(&g->wgt_copy, (size_t)g->E));
-        g->wgt_copy_cap = g->E;
-      }
-      SKY_HIP(hipMemcpyAsync(g->wgt_copy, weights_device, (size_t)g->E * 4, hipMemcpyDeviceToDevice, g->stream));
-      use = g->wgt_copy;
-    }
-  }
+  SKY_TRY(readable_weights(g, weights_device, &use));
   float* const own = g->adjwgt;
   g->adjwgt = const_cast<float*>(use);  // the build only reads it
   const int rc = build_all_tables(g, seconds);
@@ -488,9 +492,9 @@ int sky_sample_session_frontier(sky_sample_session* s, uint32_t hop, const uint3
 }
 int sky_sample_session_hop(sky_sample_session* s, uint32_t hop, const float* weights_device) {
   if (!s) return fail(SKY_ERR_ARG, "sky_sample_session_hop: null session");
-  if (weights_device && s->g->E && !padded_allocation(weights_device, (size_t)s->g->E * 4))
-    return fail(SKY_ERR_ARG, "sky_sample_session_hop: the weight array needs E * 4 + 16 readable bytes in one allocation");
-  return sample_session_hop(s->s, hop, weights_device);
+  const float* use = weights_device;
+  SKY_TRY(readable_weights(s->g, weights_device, &use));
+  return sample_session_hop(s->s, hop, use);
 }
 int sky_sample_session_end(sky_sample_session* s, uint64_t* sampled, double* seconds) {
   if (!s) return fail(SKY_ERR_ARG, "sky_sample_session_end: null session");

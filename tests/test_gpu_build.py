@@ -119,12 +119,14 @@ def test_rebuild_is_idempotent(orc):
         assert np.array_equal(x, y)
 
 
-@pytest.mark.parametrize("spare_floats", [0, 4])
-def test_build_from_a_callers_weight_array(orc, spare_floats):
-    # sky_alias_build_from_weights with weights other than the graph's own, in a device array of exactly E floats
-    # (E a multiple of 1024, ending in a short row whose 16-byte loads reach past the last weight: the library
-    # copies such an array into a padded one) and in an array with 16 spare bytes (read where it lies)
+@pytest.mark.parametrize("exact", [True, False])
+def test_build_from_a_callers_weight_array(orc, exact):
+    # sky_alias_build_from_weights with weights other than the graph's own: in device memory that ends with the
+    # last of its E floats (E a multiple of 1024, ending in a short row whose 16-byte loads reach past the last
+    # weight: the library copies such an array into a padded one), and in an array from sky_device_malloc, which
+    # adds 16 bytes to every allocation (read where it lies)
     from skywalker_amd import capi
+    import ctypes
     rng = np.random.default_rng(41)
     degs = list(rng.integers(1, 200, 300)) + [3000, 9000, 70, 33, 17]
     fill = (-sum(degs) - 5) % 1024
@@ -134,10 +136,14 @@ def test_build_from_a_callers_weight_array(orc, spare_floats):
     assert E % 1024 == 0 and xadj[-1] == E and xadj[len(degs)] - xadj[len(degs) - 1] == 5
     other = rng.lognormal(0, 2, E).astype(np.float32)
     g = capi.Graph.upload(xadj, adjncy, w)
-    dev = capi.DeviceArray(E + spare_floats, np.float32)
-    capi._ck(capi.lib().sky_memcpy_h2d(dev.ptr, capi._p(other), E * 4))
+    # the allocation holds 4 * (E + 8) + 16 bytes: 32 bytes in, exactly E floats are left
+    dev = capi.DeviceArray(E + 8 if exact else E, np.float32)
+
+    class View:
+        ptr = ctypes.c_void_p(dev.ptr.value + 32) if exact else dev.ptr
+    capi._ck(capi.lib().sky_memcpy_h2d(View.ptr, capi._p(other), E * 4))
     for rep in range(2):  # the second call finds the padded copy in place
-        g.build_tables_from_weights(dev)
+        g.build_tables_from_weights(View)
         prob, alias, valid = g.tables()
         oprob, oalias, ovalid = orc.alias_build(xadj, other)
         assert np.array_equal(prob, oprob) and np.array_equal(alias, oalias) and np.array_equal(valid, ovalid)

@@ -175,3 +175,39 @@ def test_online_sampling_builds_rows_of_every_class_without_waiting(orc):
         assert np.array_equal(d_on.to_host((n, lps)), odata) and np.array_equal(sl_on.to_host((n, slen)), osl)
         assert s_on == osampled
     g.free()
+
+
+def test_sampling_hop_by_hop_with_the_callers_weights(orc):
+    # sky_sample_session_*: the frontier of every hop is handed out, the rows are built from the weights the caller
+    # gives for that hop.  With the graph's own weights the result is sky_sample_online's; with other weights it is
+    # the oracle's online sample on a graph that carries those
+    from skywalker_amd import capi
+    xadj, adjncy = orc.rmat_csr(12, 8, 23)
+    w = orc.gen_weights(orc.W_LOGNORMAL, 23, len(adjncy), 0.0, 1.0)
+    w2 = orc.gen_weights(orc.W_UNIFORM, 29, len(adjncy), 1.0, 100.0)
+    seeds = orc.gen_seeds(6, 1 << 12, 900)
+    fanout = [1, 6, 4]
+    lps, slen = capi.sample_layout(fanout)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    d0, s0, n0, _ = g.sample_online(seeds, fanout, 31)
+    want = (d0.to_host((900, lps)), s0.to_host((900, slen)), n0)
+    d1, s1, n1, _ = g.sample_session(seeds, fanout, 31)
+    assert np.array_equal(d1.to_host((900, lps)), want[0]) and np.array_equal(s1.to_host((900, slen)), want[1]) and n1 == n0
+    import ctypes
+    E = len(w2)
+    w2_d = capi.DeviceArray.from_host(w2)
+    # the same weights in memory that ends with the last of them (the allocation holds 4 * (E + 8) + 16 bytes): the
+    # library copies such an array before its kernels read whole vectors from it
+    room = capi.DeviceArray(E + 8, np.float32)
+
+    class Exact:
+        ptr = ctypes.c_void_p(room.ptr.value + 32)
+    capi._ck(capi.lib().sky_memcpy_h2d(Exact.ptr, capi._p(w2), E * 4))
+    odata, osl, osampled = orc.sample_online(xadj, adjncy, w2, seeds, fanout, 31)
+    for arr in (w2_d, Exact):
+        uppers = []
+        d2, s2, n2, _ = g.sample_session(seeds, fanout, 31, lambda hop, upper: (uppers.append(upper), arr)[1])
+        got = (d2.to_host((900, lps)), s2.to_host((900, slen)))
+        assert uppers[0] == 900 and 0 < uppers[1] <= 900 * 6
+        assert np.array_equal(got[1], osl) and np.array_equal(got[0], odata) and n2 == osampled
+    g.free()
