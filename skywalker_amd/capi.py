@@ -271,6 +271,12 @@ class Graph:
         """OnlineGBSampleNew."""
         return self._sample(lib().sky_sample_online, seeds, fanout, seed, out)
 
+    def device_ptrs(self):
+        """Device addresses of xadj, adjncy, adjwgt, table, valid (integers; 0 for an array that does not exist)."""
+        ptrs = [C.c_void_p() for _ in range(5)]
+        _ck(lib().sky_graph_device_ptrs(self.h, *[C.byref(p) for p in ptrs]))
+        return tuple(p.value or 0 for p in ptrs)
+
     def sample_session(self, seeds, fanout, seed, weights_of_hop=None):
         """sky_sample_session_*: online k-hop sampling one hop at a time.  weights_of_hop(hop, frontier_upper) returns
         the DeviceArray of E weights (16 spare bytes, as DeviceArray gives them) from which that hop's frontier rows are

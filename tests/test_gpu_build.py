@@ -360,3 +360,28 @@ def test_two_graphs_hold_different_settings(orc):
     for g in (a, b, c):
         assert np.array_equal(g.tables()[0], want)
         g.free()
+
+
+def test_device_addresses_of_the_resident_arrays(orc):
+    # sky_graph_device_ptrs: what lies at the addresses is what sky_graph_download and sky_alias_download give
+    from skywalker_amd import capi
+    import ctypes
+    xadj, adjncy = orc.rmat_csr(10, 8, 5)
+    w = orc.gen_weights(orc.W_UNIFORM, 5, len(adjncy), 1.0, 100.0)
+    g = capi.Graph.upload(xadj, adjncy, w)
+    g.build_tables()
+    prob, alias, valid = g.tables()
+    px, pa, pw, pt, pv = g.device_ptrs()
+    assert px and pa and pw and pt and pv
+
+    def read(addr, count, dtype):
+        out = np.empty(count, dtype)
+        capi._ck(capi.lib().sky_memcpy_d2h(capi._p(out), ctypes.c_void_p(addr), ctypes.c_size_t(out.nbytes)))
+        return out
+    assert np.array_equal(read(px, len(xadj), np.uint32), xadj)
+    assert np.array_equal(read(pa, len(adjncy), np.uint32), adjncy)
+    assert np.array_equal(read(pw, len(w), np.float32), w)
+    entries = read(pt, 2 * len(w), np.uint32).reshape(-1, 2)  # {float prob; uint32 alias} per slot
+    assert np.array_equal(entries[:, 0].view(np.float32), prob) and np.array_equal(entries[:, 1], alias)
+    assert np.array_equal(read(pv, len(xadj) - 1, np.int8), valid)
+    g.free()
