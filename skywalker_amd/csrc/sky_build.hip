@@ -1287,6 +1287,19 @@ struct StreamFan {
     used[k] = true;
     return g->side[k];
   }
+  // The stream that carries the least work so far (`work`: the launch's entries, weighted by the caller where a
+  // kernel is slow): a kernel queued behind a long one waits for it while other streams run dry.
+  uint64_t load[sky_graph::SIDE_STREAMS + 1] = {0, 0, 0, 0};
+  hipStream_t next(uint64_t work) {
+    if (!on) return main;
+    int k = 0;
+    for (int i = 1; i <= sky_graph::SIDE_STREAMS; ++i)
+      if (load[i] < load[k]) k = i;
+    load[k] += work + 1;
+    if (k == sky_graph::SIDE_STREAMS) return main;
+    used[k] = true;
+    return g->side[k];
+  }
   int join() {
     if (!joinable) return SKY_OK;
     on = joinable = false;
@@ -1454,7 +1467,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const uint32_t per_block = 256 / G;
-      hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, fan.next(), vlist + starts[cls],
+      hipLaunchKernelGGL(kernel, dim3((cnt + per_block - 1) / per_block), dim3(256), 0, fan.next(host.edges[cls]), vlist + starts[cls],
                          cnt, (const uint32_t*)nullptr, 0, g->adjwgt, g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
@@ -1472,14 +1485,15 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
   const bool wide_streamed = !stream_to_tiled && all_stream_edges >= (uint64_t)option(g, OPT_STREAM_WIDE_MIN_EDGES);
   const uint32_t wide_rows = wide_streamed ? counts[CLS_STREAM_WIDE] : 0;
   if (!stream_to_tiled && narrow_rows + wide_rows) {
-    StreamSwap sw(g, fan.next());
+    // the streaming kernel takes three times as long for an entry as the others when it shares the GPU with them
+    StreamSwap sw(g, fan.next(3 * (narrow_edges + (wide_streamed ? host.edges[CLS_STREAM_WIDE] : 0))));
     SKY_TRY(build_rows_stream(g, vlist + starts[CLS_STREAM_WIDE], wide_rows, vlist + starts[CLS_STREAM], narrow_rows));
     if (tm) SKY_TRY(tm->mark("stream", narrow_edges + (wide_streamed ? host.edges[CLS_STREAM_WIDE] : 0)));
   }
   // Rows of 5118..8189 entries: one workgroup holds the row (without row_merge they are built tile by tile).
   if (row_merge && counts[CLS_HOLD]) {
     {
-      StreamSwap sw(g, fan.next());
+      StreamSwap sw(g, fan.next(2 * host.edges[CLS_HOLD]));
       SKY_TRY(build_rows_hold(g, vlist + starts[CLS_HOLD], counts[CLS_HOLD], nullptr, 0));
     }
     if (tm) SKY_TRY(tm->mark("hold", host.edges[CLS_HOLD]));
@@ -1488,7 +1502,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const size_t bytes = (size_t)rowt * 4 * t * 16;
-      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(), vlist + starts[cls], g->xadj, g->adjwgt,
+      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(host.edges[cls]), vlist + starts[cls], g->xadj, g->adjwgt,
                          g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
@@ -1497,7 +1511,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t cnt = counts[cls];
     if (cnt) {
       const size_t bytes = ((size_t)rowt * per + 2) * 14;
-      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(), vlist + starts[cls], cnt,
+      hipLaunchKernelGGL(kernel, dim3(cnt), dim3(rowt), bytes, fan.next(host.edges[cls]), vlist + starts[cls], cnt,
                          (const uint32_t*)nullptr, 0, g->adjwgt, g->table, g->valid);
     }
     return (tm && cnt) ? tm->mark(name, host.edges[cls]) : SKY_OK;  // no bracket for an empty class
@@ -1568,7 +1582,7 @@ int build_rows(sky_graph* g, const uint32_t* src, uint32_t n, EventTimer* tm) {
     const uint32_t cnt = tiled_rows;
     uint32_t skipped = 0;
     {
-      StreamSwap sw(g, fan.next());
+      StreamSwap sw(g, fan.next(2 * tiled_edges));
       SKY_TRY(build_rows_tiled(g, tiled_list, cnt, &skipped, tm, tiled_edges));
     }
     SKY_TRY(fan.join());
