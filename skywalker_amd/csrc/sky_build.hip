@@ -1702,22 +1702,24 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
     tiled_rows += rows_of(c);
     tiled_edges += g->bin_edges[c];
   }
+  // A stream is chosen by the work it already carries; the work of a class is what the graph holds of it (a
+  // frontier mirrors the graph), weighted for the kernels of the long rows, which are slow beside the others.
   if (tiled_rows) {
-    StreamSwap sw(g, fan.next());
+    StreamSwap sw(g, fan.next(2 * tiled_edges));
     SKY_TRY(build_rows_tiled_dev(g, vlist, dev, t_first, CLS_HUGE - t_first + 1, tiled_rows, tiled_edges));
   }
   // the streaming kernel fills the LDS of every CU it reaches: the tile-parallel path, whose first kernels are small,
   // is enqueued before it
   if (stream_rows) {
-    StreamSwap sw(g, fan.next());
+    StreamSwap sw(g, fan.next(3 * (g->bin_edges[CLS_STREAM] + g->bin_edges[CLS_STREAM_LAST])));
     SKY_TRY(build_rows_stream_dev(g, vlist, dev, 2, std::min(DEV_GRID_STREAM, stream_rows)));
   }
   auto grp = [&](int cls, auto kernel, int G) {
     const uint32_t rows = rows_of(cls);
     if (!rows) return;
     const uint32_t per = 256 / G;
-    hipLaunchKernelGGL(kernel, dim3(std::min(dev_grid_cap(256), (rows + per - 1) / per)), dim3(256), 0, fan.next(), vlist,
-                       0u, dev, cls, g->adjwgt, g->table, g->valid);
+    hipLaunchKernelGGL(kernel, dim3(std::min(dev_grid_cap(256), (rows + per - 1) / per)), dim3(256), 0,
+                       fan.next(g->bin_edges[cls]), vlist, 0u, dev, cls, g->adjwgt, g->table, g->valid);
   };
   auto mrg = [&](int cls, auto kernel, int rowt, int per) {
     const uint32_t rows = rows_of(cls);
@@ -1725,8 +1727,8 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
     const size_t bytes = ((size_t)rowt * per + 2) * 14;
     // one wavefront per row: a striding grid; larger workgroups: one per row the class can hold (the code of a
     // loop over rows costs these kernels registers they do not have)
-    hipLaunchKernelGGL(kernel, dim3(rowt <= 64 ? std::min(dev_grid_cap(rowt), rows) : rows), dim3(rowt), bytes, fan.next(),
-                       vlist, 0u, dev, cls, g->adjwgt, g->table, g->valid);
+    hipLaunchKernelGGL(kernel, dim3(rowt <= 64 ? std::min(dev_grid_cap(rowt), rows) : rows), dim3(rowt), bytes,
+                       fan.next(g->bin_edges[cls]), vlist, 0u, dev, cls, g->adjwgt, g->table, g->valid);
   };
   // The class kernels go out in the order of the classes' sizes in the graph, the largest first: a frontier mirrors
   // the graph, and the streams should not end on a long kernel that started last.
@@ -1757,7 +1759,7 @@ int build_rows_dev(sky_graph* g, const uint32_t* src, const uint32_t* n_dev, uin
   auto hold = [&](int cls) -> int {
     const uint32_t rows = rows_of(cls);
     if (!rows) return SKY_OK;
-    StreamSwap sw(g, fan.next());
+    StreamSwap sw(g, fan.next(2 * g->bin_edges[cls]));
     return build_rows_hold(g, vlist, rows, dev, cls);
   };
   int hold_rc = SKY_OK;
