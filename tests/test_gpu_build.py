@@ -19,9 +19,9 @@ def build_and_compare(orc, xadj, adjncy, w, label):
     print("case", label, "V", len(xadj) - 1, "E", len(w), flush=True)
     oprob, oalias, ovalid = orc.alias_build(xadj, w)
     deg = np.diff(xadj)
-    # rows of 5118..524287 entries: once through their own kernel, once (the default for so few of them)
+    # rows of 8190..524287 entries: once through their own kernel, once (the default for so few of them)
     # through the tile-parallel path
-    routes = (0, 4000000) if ((deg >= 5118) & (deg <= 524287)).any() else (4000000,)
+    routes = (0, 4000000) if ((deg >= 8190) & (deg <= 524287)).any() else (4000000,)
     # rows of at most 32 entries: by degree class (the default below 2^25 rows), and by the kernel that walks the
     # vertices in order
     for stream_min_edges, small_in_place in [(r, 0) for r in routes] + [(routes[0], 1)]:
